@@ -1,0 +1,253 @@
+"""Pins the oracle's operators (compress, decompress, attention, paged decode,
+TurboQuantProd) by brute force on tiny inputs, library routines and
+invariants, so that a dropped term, wrong sign or transposed operand fails."""
+from __future__ import annotations
+
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import tq_oracle as O
+from tests.conftest import outlier_rows
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def book():
+    c, b = O.lloyd_max_gaussian(128, 4)
+    return c, b, O.haar_orthogonal(128, 42)
+
+
+# ---- compress ---------------------------------------------------------------
+
+def test_compress_tie_rule_and_division():
+    """(3,4) has norm 5; the unit vector is (0.6f, 0.8f).  With boundaries
+    placed exactly on those values the index counts boundaries strictly below
+    the coordinate (torch.bucketize, right=False)."""
+    x = torch.tensor([[[3.0, 4.0]]])
+    a, b = torch.tensor(3.0) / 5.0, torch.tensor(4.0) / 5.0
+    bnd = torch.stack([a, b])
+    packed, norms = O.compress(x, torch.eye(2), bnd)
+    assert norms.item() == 5.0
+    assert packed.tolist() == [[[(0 << 4) | 1]]]
+    # a rotation that swaps the coordinates must swap the nibbles: y = x_hat @ R.T
+    swap = torch.tensor([[0.0, 1.0], [1.0, 0.0]])
+    packed, _ = O.compress(x, swap, bnd)
+    assert packed.tolist() == [[[(1 << 4) | 0]]]
+    # a non-symmetric rotation tells R.T from R: R = [[0,1],[-1,0]], y = (x1, -x0)
+    rot = torch.tensor([[0.0, 1.0], [-1.0, 0.0]])
+    packed, _ = O.compress(x, rot, torch.tensor([-0.7, 0.7]))
+    assert packed.tolist() == [[[(2 << 4) | 1]]]       # y = (0.8, -0.6)
+
+
+def test_compress_scalar_brute_force(book):
+    c, b, r = book
+    x = outlier_rows(3, 2, 128, seed=5)
+    packed, norms = O.compress(x, r, b)
+    idx = O.nibble_unpack(packed)
+    r64, b64 = r.double().tolist(), b.double().tolist()
+    for n in range(3):
+        for h in range(2):
+            row = x[n, h].double().tolist()
+            nrm = math.sqrt(sum(v * v for v in row))
+            assert abs(nrm - norms[n, h, 0].item()) < 1e-5 * nrm
+            for j in range(128):
+                y = sum(row[k] / (nrm + 1e-10) * r64[j][k] for k in range(128))
+                want = sum(1 for t in b64 if t < y)
+                if min(abs(y - t) for t in b64) > 1e-6:
+                    assert idx[n, h, j].item() == want, (n, h, j)
+
+
+def test_compress_adversarial_inputs_stay_in_range(book):
+    # the cases of the reference's tests/test_adversarial.py
+    c, b, r = book
+    for x in (torch.zeros(2, 2, 128), torch.full((2, 2, 128), 1e6),
+              torch.full((2, 2, 128), 1e-30)):
+        packed, norms = O.compress(x, r, b)
+        assert torch.isfinite(norms).all()
+        assert torch.isfinite(O.decompress(packed, norms, c)).all()
+    x = torch.randn(2, 2, 128)
+    x[0, 0, 3] = 1e8
+    packed, norms = O.compress(x, r, b)
+    assert torch.isfinite(norms).all()
+
+
+def test_compress_matches_committed_case(book):
+    c, b, r = book
+    z = np.load(os.path.join(GOLDEN, "compress_case_6x2x128.npz"))
+    packed, norms = O.compress(torch.from_numpy(z["x"]), r, b)
+    mism = (O.nibble_unpack(packed) != O.nibble_unpack(torch.from_numpy(z["packed"]))).float().mean()
+    assert mism <= 1e-3       # 1536 entries: at most one boundary flip across BLAS builds
+    assert np.allclose(norms.numpy(), z["norms"], rtol=1e-6)
+
+
+def test_config0_round_trip_distortion(book):
+    """BASELINE configuration 0: one layer, 8 KV heads, d=128, 4096 tokens,
+    outlier channels; relative MSE of the 4-bit round trip is the Lloyd-Max
+    distortion (about 0.0095) and the record is 68 bytes per token per head."""
+    c, b, r = book
+    x = outlier_rows(4096, 8, 128, seed=1000)
+    packed, norms = O.compress(x, r, b)
+    rec = (O.decompress(packed, norms, c).reshape(-1, 128) @ r).reshape(x.shape)
+    rel = ((x - rec) ** 2).sum() / (x ** 2).sum()
+    assert abs(rel.item() - 0.0095) < 0.001
+    assert packed.shape[-1] + norms.shape[-1] * 4 == 68
+    cos = F.cosine_similarity(x.reshape(-1, 128), rec.reshape(-1, 128), dim=-1)
+    assert cos.min() > 0.93        # tests/test_quantizer_mse.py:37-41
+
+
+# ---- decompress -------------------------------------------------------------
+
+def test_decompress_brute_force(book):
+    c, _, _ = book
+    packed = torch.randint(0, 256, (3, 2, 64), dtype=torch.uint8)
+    norms = torch.rand(3, 2, 1) * 7
+    out = O.decompress(packed, norms, c)
+    assert out.shape == (3, 2, 128) and out.dtype == torch.float32
+    for n in range(3):
+        for h in range(2):
+            for j in range(64):
+                byte = packed[n, h, j].item()
+                assert out[n, h, 2 * j].item() == (c[byte >> 4] * norms[n, h, 0]).item()
+                assert out[n, h, 2 * j + 1].item() == (c[byte & 15] * norms[n, h, 0]).item()
+
+
+# ---- attention --------------------------------------------------------------
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_against_sdpa(causal):
+    q = torch.randn(2, 8, 12, 64)
+    k = torch.randn(2, 2, 12, 64)
+    v = torch.randn(2, 2, 12, 64)
+    got = O.attention(q, k, v, is_causal=causal)
+    want = F.scaled_dot_product_attention(
+        q, k.repeat_interleave(4, 1), v.repeat_interleave(4, 1), is_causal=causal)
+    assert torch.allclose(got, want, atol=1e-5)
+
+
+def test_attention_causal_is_top_left_and_dropped_for_one_query():
+    q = torch.randn(1, 1, 3, 16)
+    k = torch.randn(1, 1, 5, 16)
+    v = torch.randn(1, 1, 5, 16)
+    got = O.attention(q, k, v, is_causal=True)
+    for i in range(3):   # query i sees keys 0..i
+        want = O.attention(q[:, :, i:i + 1], k[:, :, :i + 1], v[:, :, :i + 1])
+        assert torch.allclose(got[:, :, i:i + 1], want, atol=1e-6)
+    one = O.attention(q[:, :, :1], k, v, is_causal=True)
+    assert torch.allclose(one, O.attention(q[:, :, :1], k, v, is_causal=False))
+
+
+def test_fused_attention_equals_attention_on_reconstruction(book):
+    """Rotated-space attention on decompressed K/V, rotated back, equals plain
+    attention on the reconstructed K/V in the original space
+    (tests/test_attention_kernel.py:95-148 of the reference)."""
+    c, b, r = book
+    B, HQ, HKV, N = 1, 4, 2, 40
+    q = torch.randn(B, HQ, N, 128)
+    k = torch.randn(B * HKV * N, 1, 128)
+    v = torch.randn(B * HKV * N, 1, 128)
+    kp, kn = O.compress(k, r, b)
+    vp, vn = O.compress(v, r, b)
+    shp = (B, HKV, N)
+    got = O.fused_tq_attention(q, kp.reshape(*shp, 64), kn.reshape(*shp, 1), vp.reshape(*shp, 64),
+                               vn.reshape(*shp, 1), c, c, r, is_causal=True)
+    k_rec = (O.decompress(kp, kn, c).reshape(-1, 128) @ r).reshape(B, HKV, N, 128)
+    v_rec = (O.decompress(vp, vn, c).reshape(-1, 128) @ r).reshape(B, HKV, N, 128)
+    want = O.attention(q, k_rec, v_rec, is_causal=True)
+    assert torch.allclose(got, want, atol=2e-5)
+
+
+# ---- paged decode -----------------------------------------------------------
+
+def _paged_case(book, lens, hq=8, hkv=2, bs=16, seed=3, dtype=torch.bfloat16):
+    c, b, r = book
+    g = torch.Generator().manual_seed(seed)
+    S = len(lens)
+    max_blocks = max(1, (max(lens) + bs - 1) // bs)
+    nb = S * max_blocks + 3
+    cache = torch.randint(0, 256, (nb, bs, hkv * 136), dtype=torch.uint8, generator=g)
+    perm = torch.randperm(nb, generator=g)[: S * max_blocks].reshape(S, max_blocks).int()
+    for s, L in enumerate(lens):
+        if L == 0:
+            continue
+        k = torch.randn(L, hkv, 128, generator=g)
+        v = torch.randn(L, hkv, 128, generator=g)
+        kp, kn = O.compress(k, r, b)
+        vp, vn = O.compress(v, r, b)
+        t = torch.arange(L)
+        slots = perm[s].long()[t // bs] * bs + t % bs
+        O.store_rows(cache, slots, kp, kn, vp, vn)
+    q = torch.randn(S, hq, 128, generator=g).to(dtype)
+    return q, cache, perm, torch.tensor(lens, dtype=torch.int32)
+
+
+def test_page_layout_offsets():
+    # src/flashquant/vllm/impl.py:132-138 with 8 heads, d=128
+    assert O.page_layout(8, 128) == (512, 544, 1056, 1088)
+
+
+def test_paged_loop_equals_gather_and_sdpa(book):
+    c, b, r = book
+    q, cache, bt, lens = _paged_case(book, [37, 0, 16, 5])
+    a = O.paged_decode_loop(q, cache, bt, lens, c, c, 2, 128, 16)
+    g = O.paged_decode_gather(q, cache, bt, lens, c, c, 2, 128, 16)
+    assert torch.equal(a, g)
+    assert (a[1] == 0).all()                         # cpu_reference.py:286-287
+    k, v = O.gather_sequence(cache, bt[0], 37, c, c, 2, 128, 16)
+    want = F.scaled_dot_product_attention(
+        q[0].float().unsqueeze(1), k.repeat_interleave(4, 0), v.repeat_interleave(4, 0))
+    assert torch.allclose(a[0].float(), want.squeeze(1), atol=2e-2)
+
+
+def test_paged_block_table_permutation_invariance(book):
+    """Moving pages and updating the table must not change the result
+    (tests/test_paged_decode_kernel.py:210-259 of the reference)."""
+    c, b, r = book
+    q, cache, bt, lens = _paged_case(book, [45, 20])
+    base = O.split_k_paged_decode(q, cache, bt, lens, c, c, r, 2, 128, 16)
+    perm = torch.randperm(cache.shape[0])
+    moved = torch.empty_like(cache)
+    moved[perm] = cache
+    bt2 = perm[bt.long()].int()
+    again = O.split_k_paged_decode(q, moved, bt2, lens, c, c, r, 2, 128, 16)
+    assert torch.equal(base, again)
+    loop = O.split_k_paged_decode(q, cache, bt, lens, c, c, r, 2, 128, 16, faithful_loop=True)
+    assert torch.equal(base, loop)
+
+
+# ---- TurboQuantProd ---------------------------------------------------------
+
+def test_prod_signs_and_shapes():
+    c3, b3 = O.lloyd_max_gaussian(128, 3)
+    r, s = O.haar_orthogonal(128, 42), O.qjl_matrix(128, 42)
+    x = torch.randn(5, 128)
+    idx, norms, signs, gamma = O.prod_quantize(x, r, b3, c3, s)
+    assert idx.max() <= 7 and idx.min() >= 0
+    assert set(signs.unique().tolist()) <= {-1.0, 1.0}
+    resid = x - O.mse_dequantize(idx, norms, r, c3)
+    assert torch.allclose(gamma, resid.norm(dim=-1, keepdim=True))
+    assert torch.equal(signs, torch.where(resid @ s.T >= 0, 1.0, -1.0))
+    z = O.prod_quantize(torch.zeros(1, 128), r, b3, c3, s)
+    assert (z[2] == 1.0).all()      # a zero projection maps to +1
+
+
+def test_prod_estimator_unbiased():
+    """Averaged over many keys the QJL-corrected estimate matches the true
+    inner product far better than the MSE-only term
+    (tests/test_quantizer_prod.py:32-99 of the reference: relative bias < 0.05)."""
+    c3, b3 = O.lloyd_max_gaussian(128, 3)
+    r, s = O.haar_orthogonal(128, 42), O.qjl_matrix(128, 42)
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(1, 128, generator=g)
+    k = q * 0.5 + torch.randn(10000, 128, generator=g)
+    idx, norms, signs, gamma = O.prod_quantize(k, r, b3, c3, s)
+    est = O.prod_inner_product(q.expand(10000, 128), idx, norms, signs, gamma, r, c3, s).squeeze(-1)
+    true = (k * q).sum(-1)
+    assert abs((est - true).mean().item()) / true.abs().mean().item() < 0.05
+    mse_only = (q * O.mse_dequantize(idx, norms, r, c3)).sum(-1)
+    assert abs((est - true).mean()) < abs((mse_only - true).mean()) + 0.05
