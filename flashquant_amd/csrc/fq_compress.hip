@@ -1,0 +1,325 @@
+// TQ4 compress for gfx950.
+//
+// Per row x (D elements, fp16 or bf16):  n = ||x||_2,  y = (x / (n + 1e-10)) R^T,
+// idx_j = #{boundaries < y_j},  byte_j = idx_2j << 4 | idx_2j+1,  norm = n
+// (compress_reference, src/flashquant/kernels/cpu_reference.py:39-61).
+//
+// The rotation is a rows x D x D contraction on the 32x32x16 fp16 MFMA, with
+// float32 accumulation.  A plain 16-bit rotation would move about 1 index in
+// 200 across a bucket boundary, so the matrix is split R = R_hi + 2^-12 R_lo
+// (two fp16 terms, 22 significant bits) and the row is rotated un-normalised:
+// the raw fp16/bf16 row, scaled by a power of two so that its largest element
+// lies in [1, 2), is exact in fp16 up to elements 2^-24 below the largest, and
+// the division by (n + 1e-10) is applied to the float32 accumulators.
+//
+// Layout.  One workgroup owns the whole matrix in registers: wave w keeps the
+// MFMA A operands (R_hi, R_lo rows of its 32 output coordinates, all k) for the
+// kernel's lifetime.  Tiles of 64 rows stream through LDS as the B operand
+// (row-major fp16, padded rows so that the 128-bit operand reads are
+// conflict-free), double buffered against the global loads of the next tile.
+// A lane of the accumulator holds one row and 16 consecutive output
+// coordinates (the MFMA row index is permuted on the R side to make them
+// consecutive), so a lane bucketizes and nibble-packs 8 output bytes without
+// any cross-lane traffic.  Bucketize is one LDS lookup in a 256-cell table
+// built from the boundaries (base count + the single boundary that can fall in
+// the cell) plus one compare; if two boundaries share a cell the kernel falls
+// back to the 15-compare scan.
+
+#include "fq_common.hpp"
+
+namespace fq {
+
+template <int D>
+struct CompressCfg {
+    static constexpr int NK = D / 16;                  // MFMA k-steps
+    static constexpr int CB = D / 32;                  // 32-coordinate output blocks
+    static constexpr int WAVES = CB < 4 ? 4 : CB;
+    static constexpr int THREADS = WAVES * kWave;
+    static constexpr int TT = D == 256 ? 32 : 64;      // rows per tile
+    static constexpr int TB = TT / 32;                 // 32-row blocks per tile
+    static constexpr int TB_STEP = WAVES / CB;         // row blocks handled in parallel
+    static constexpr int CPR = D / 8;                  // 16-byte chunks per row
+    static constexpr int ROWS_PER_PASS = THREADS / CPR;
+    static constexpr int PASSES = TT / ROWS_PER_PASS;
+    static constexpr int XS_STRIDE = D * 2 + 16;       // bytes per staged row
+    static constexpr int OUT_STRIDE = D / 2 + 8;       // bytes per packed row in LDS
+    static constexpr int CELLS = 256;
+};
+
+constexpr float kLoScale = 1.0f / 4096.0f;
+
+struct BucketTable {
+    uint2v cell[256];   // x = threshold bits, y = base count
+    float bnd[16];
+    float inv_w;
+    float offset;
+    int slow;
+};
+
+// Builds the cell table from the 15 boundaries (block-wide, ends with a barrier).
+__device__ __forceinline__ void build_bucket_table(BucketTable& t, const float* __restrict__ boundaries,
+                                                   int tid, int nthreads) {
+    if (tid < 15) t.bnd[tid] = boundaries[tid];
+    if (tid == 15) t.bnd[15] = __builtin_inff();
+    if (tid == 0) t.slow = 0;
+    __syncthreads();
+    const float b0 = t.bnd[0], b14 = t.bnd[14];
+    const float span = b14 - b0;
+    const float pad = span > 0.0f ? span * (1.0f / 256.0f) : 1.0f;
+    const float lo = b0 - pad;
+    const float w = (span + 2.0f * pad) * (1.0f / 256.0f);
+    const float margin = 0.01f * w;
+    for (int c = tid; c < 256; c += nthreads) {
+        const float lo_c = lo + w * float(c) - margin;
+        const float hi_c = lo + w * float(c + 1) + margin;
+        int base = 0, inside = 0;
+        float thr = __builtin_inff();
+        for (int b = 0; b < 15; ++b) {
+            const float v = t.bnd[b];
+            if (v < lo_c) {
+                ++base;
+            } else if (v <= hi_c) {
+                ++inside;
+                thr = v;
+            }
+        }
+        if (inside > 1 || !(span > 0.0f)) t.slow = 1;
+        t.cell[c] = uint2v{float_to_bits(thr), uint32_t(base)};
+    }
+    if (tid == 0) {
+        t.inv_w = 1.0f / w;
+        t.offset = -lo / w;
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ uint32_t bucket_fast(const BucketTable& t, float y, float inv_w, float offset) {
+    const float pos = __builtin_fmaf(y, inv_w, offset);
+    const int c = int(__builtin_amdgcn_fmed3f(pos, 0.0f, 255.0f));
+    const uint2v e = t.cell[c];
+    return e.y + (bits_to_float(e.x) < y ? 1u : 0u);
+}
+
+__device__ __forceinline__ uint32_t bucket_slow(const BucketTable& t, float y) {
+    uint32_t n = 0;
+#pragma unroll
+    for (int b = 0; b < 15; ++b) n += (t.bnd[b] < y) ? 1u : 0u;
+    return n;
+}
+
+// MFMA row r of a 32-row block <-> output coordinate (within the block) such
+// that accumulator register i of lane half h holds coordinate 16h + i.
+__device__ __forceinline__ int mfma_row_to_coord(int r) {
+    return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
+}
+
+template <int D, int DT>
+__global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
+    const uint4v* __restrict__ x, const float* __restrict__ rot_T_even,
+    const float* __restrict__ rot_T_odd, const float* __restrict__ boundaries,
+    uint8_t* __restrict__ packed, float* __restrict__ norms, int64_t M, int64_t num_tiles) {
+    using C = CompressCfg<D>;
+    __shared__ __attribute__((aligned(16))) uint8_t xs[2][C::TT * C::XS_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint8_t outs[C::TT * C::OUT_STRIDE];
+    __shared__ float inv_s[2][C::TT];
+    __shared__ BucketTable table;
+
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int lane = tid % kWave;
+    const int n32 = lane % 32;   // MFMA row (A side) / tile row (B, C side)
+    const int kg = lane / 32;    // k group (A, B side) / coordinate half (C side)
+    const int cb = wave % C::CB;
+    const int tb0 = wave / C::CB;
+
+    // ---- the rotation rows of this wave, split into two fp16 terms ----------
+    half8 a_hi[C::NK], a_lo[C::NK];
+    {
+        const int j = 32 * cb + mfma_row_to_coord(n32);
+        const float* src = (j & 1) ? rot_T_odd : rot_T_even;
+        const int col = j >> 1;
+#pragma unroll
+        for (int ks = 0; ks < C::NK; ++ks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int k = 16 * ks + 8 * kg + e;
+                const float r = src[k * (D / 2) + col];
+                const _Float16 hi = _Float16(r);
+                a_hi[ks][e] = hi;
+                a_lo[ks][e] = _Float16((r - float(hi)) * 4096.0f);
+            }
+        }
+    }
+    build_bucket_table(table, boundaries, tid, C::THREADS);
+    const float inv_w = table.inv_w, offset = table.offset;
+    const bool slow = table.slow != 0;
+
+    // ---- staging helpers -----------------------------------------------------
+    const int chunk = tid % C::CPR;
+    const int row_in_pass = tid / C::CPR;
+    uint4v pre[C::PASSES];
+
+    auto issue_loads = [&](int64_t tile) {
+#pragma unroll
+        for (int p = 0; p < C::PASSES; ++p) {
+            const int64_t row = tile * C::TT + p * C::ROWS_PER_PASS + row_in_pass;
+            pre[p] = row < M ? __builtin_nontemporal_load(x + row * C::CPR + chunk) : uint4v{0, 0, 0, 0};
+        }
+    };
+    auto stage = [&](int64_t tile, int buf) {
+#pragma unroll
+        for (int p = 0; p < C::PASSES; ++p) {
+            const int r = p * C::ROWS_PER_PASS + row_in_pass;
+            const int64_t row = tile * C::TT + r;
+            float e[8];
+            const uint32_t w[4] = {pre[p].x, pre[p].y, pre[p].z, pre[p].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                e[2 * i] = load_elem<DT>(uint16_t(w[i] & 0xffffu));
+                e[2 * i + 1] = load_elem<DT>(uint16_t(w[i] >> 16));
+            }
+            float ss = 0.0f, mx = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                ss = __builtin_fmaf(e[i], e[i], ss);
+                mx = __builtin_fmaxf(mx, __builtin_fabsf(e[i]));
+            }
+#pragma unroll
+            for (int m = 1; m < C::CPR; m <<= 1) {
+                ss += xor_shuffle(ss, m);
+                mx = __builtin_fmaxf(mx, xor_shuffle(mx, m));
+            }
+            const float nrm = __builtin_sqrtf(ss);
+            int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+            if (ex < -126 || ex > 126) ex = 0;   // zero / subnormal / non-finite rows: no scaling
+            const float down = bits_to_float(uint32_t(127 - ex) << 23);
+            const float up = bits_to_float(uint32_t(127 + ex) << 23);
+            uint4v h;
+            h.x = pack_h2(_Float16(e[0] * down), _Float16(e[1] * down));
+            h.y = pack_h2(_Float16(e[2] * down), _Float16(e[3] * down));
+            h.z = pack_h2(_Float16(e[4] * down), _Float16(e[5] * down));
+            h.w = pack_h2(_Float16(e[6] * down), _Float16(e[7] * down));
+            *reinterpret_cast<uint4v*>(&xs[buf][r * C::XS_STRIDE + chunk * 16]) = h;
+            if (chunk == 0) {
+                inv_s[buf][r] = up / (nrm + 1e-10f);
+                if (row < M) norms[row] = nrm;
+            }
+        }
+    };
+
+    int64_t tile = blockIdx.x;
+    if (tile < num_tiles) {
+        issue_loads(tile);
+        stage(tile, 0);
+    }
+    __syncthreads();
+
+    for (int it = 0; tile < num_tiles; tile += gridDim.x, ++it) {
+        const int cur = it & 1;
+        const int64_t next = tile + gridDim.x;
+        if (next < num_tiles) issue_loads(next);
+
+        // ---- rotate + bucketize + pack ---------------------------------------
+        for (int tb = tb0; tb < C::TB; tb += C::TB_STEP) {
+            float16v acc_hi = {}, acc_lo = {};
+            const uint8_t* brow = &xs[cur][(32 * tb + n32) * C::XS_STRIDE + kg * 16];
+#pragma unroll
+            for (int ks = 0; ks < C::NK; ++ks) {
+                const half8 b = *reinterpret_cast<const half8*>(brow + ks * 32);
+                acc_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[ks], b, acc_hi, 0, 0, 0);
+                acc_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_lo[ks], b, acc_lo, 0, 0, 0);
+            }
+            const float inv = inv_s[cur][32 * tb + n32];
+            uint32_t idx[16];
+            if (!slow) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    idx[i] = bucket_fast(table, __builtin_fmaf(acc_lo[i], kLoScale, acc_hi[i]) * inv, inv_w, offset);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    idx[i] = bucket_slow(table, __builtin_fmaf(acc_lo[i], kLoScale, acc_hi[i]) * inv);
+            }
+            uint2v o;
+            o.x = (idx[0] << 4 | idx[1]) | (idx[2] << 4 | idx[3]) << 8 | (idx[4] << 4 | idx[5]) << 16 |
+                  (idx[6] << 4 | idx[7]) << 24;
+            o.y = (idx[8] << 4 | idx[9]) | (idx[10] << 4 | idx[11]) << 8 | (idx[12] << 4 | idx[13]) << 16 |
+                  (idx[14] << 4 | idx[15]) << 24;
+            *reinterpret_cast<uint2v*>(&outs[(32 * tb + n32) * C::OUT_STRIDE + 16 * cb + 8 * kg]) = o;
+        }
+        __syncthreads();
+
+        // ---- packed rows of this tile: LDS -> global, 16 bytes per lane ------
+        constexpr int OC = D / 32;   // 16-byte chunks per packed row
+        for (int c = tid; c < C::TT * OC; c += C::THREADS) {
+            const int r = c / OC, q = c % OC;
+            const int64_t row = tile * C::TT + r;
+            if (row < M) {
+                const uint2v lo = *reinterpret_cast<const uint2v*>(&outs[r * C::OUT_STRIDE + q * 16]);
+                const uint2v hi = *reinterpret_cast<const uint2v*>(&outs[r * C::OUT_STRIDE + q * 16 + 8]);
+                uint4v v = {lo.x, lo.y, hi.x, hi.y};
+                __builtin_nontemporal_store(v, reinterpret_cast<uint4v*>(packed + row * (D / 2)) + q);
+            }
+        }
+        if (next < num_tiles) stage(next, cur ^ 1);
+        __syncthreads();
+    }
+}
+
+template <int D, int DT>
+int launch_compress(const void* x, const float* re, const float* ro, const float* bnd, uint8_t* packed,
+                    float* norms, int64_t M, int num_cus, hipStream_t s) {
+    using C = CompressCfg<D>;
+    const int64_t tiles = (M + C::TT - 1) / C::TT;
+    const int64_t cap = int64_t(num_cus) * 2;
+    const unsigned grid = unsigned(tiles < cap ? tiles : cap);
+    hipLaunchKernelGGL((tq4_compress_kernel<D, DT>), dim3(grid), dim3(C::THREADS), 0, s,
+                       reinterpret_cast<const uint4v*>(x), re, ro, bnd, packed, norms, M, tiles);
+    return fq_host::check_launch();
+}
+
+}  // namespace fq
+
+namespace fq_host {
+int device_cu_count() {
+    static thread_local int cached_dev = -1;
+    static thread_local int cached_cus = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev != cached_dev) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        cached_dev = dev;
+        cached_cus = cus;
+    }
+    return cached_cus;
+}
+}  // namespace fq_host
+
+extern "C" int fq_tq4_compress(const void* x, int x_dtype, const float* rot_T_even,
+                               const float* rot_T_odd, const float* boundaries, uint8_t* packed,
+                               float* norms, int64_t M, int D, void* stream) {
+    using namespace fq;
+    if (M < 0) return FQ_ERR_BAD_SHAPE;
+    if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
+    if (x_dtype != FQ_F16 && x_dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
+    if (M == 0) return FQ_OK;
+    if (!x || !rot_T_even || !rot_T_odd || !boundaries || !packed || !norms) return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(x, 16) || !fq_host::aligned(packed, 16) || !fq_host::aligned(norms, 4))
+        return FQ_ERR_MISALIGNED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int cus = fq_host::device_cu_count();
+#define FQ_COMPRESS_CASE(DD)                                                                              \
+    case DD:                                                                                              \
+        return x_dtype == FQ_F16                                                                          \
+                   ? launch_compress<DD, FQ_F16>(x, rot_T_even, rot_T_odd, boundaries, packed, norms, M, cus, s) \
+                   : launch_compress<DD, FQ_BF16>(x, rot_T_even, rot_T_odd, boundaries, packed, norms, M, cus, s);
+    switch (D) {
+        FQ_COMPRESS_CASE(64)
+        FQ_COMPRESS_CASE(128)
+        FQ_COMPRESS_CASE(256)
+        default: return FQ_ERR_UNSUPPORTED_DIM;
+    }
+#undef FQ_COMPRESS_CASE
+}

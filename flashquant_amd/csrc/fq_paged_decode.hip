@@ -1,0 +1,640 @@
+// Split-K paged decode from the packed TQ4 cache, gfx950.
+//
+// Operator: paged_decode_reference (src/flashquant/kernels/cpu_reference.py:230-368)
+// wrapped by the query pre-rotation and output post-rotation of
+// src/flashquant/kernels/paged_decode.py:112-128.  Token row of the cache:
+// [K idx H*D/2 | K norm H*4 | V idx H*D/2 | V norm H*4] (src/flashquant/vllm/impl.py:132-138).
+//
+// Three launches on the caller's stream:
+//   1. rotate_q_kernel       q_rot = (q @ R^T) rounded to the query dtype
+//   2. paged_decode_kernel   one workgroup per (split, sequence, group of <= 8 KV
+//                            heads), one wavefront per KV head; writes float32
+//                            partials (m, l, acc[D]) per (sequence, query head, split)
+//   3. reduce_rotate_kernel  log-sum-exp combine of the splits, rounded to the
+//                            query dtype, then (out_rot @ R) rounded again
+//
+// The decode kernel is bound by HBM traffic (136 bytes per token per KV head)
+// but only if the per-byte work is small: with 4 query heads per KV head,
+// float32 FMAs alone would cost more than the memory time, so both products
+// run on the 16x16x32 fp16 MFMA and the dequantisation is one LDS lookup per
+// packed byte: a 256-entry table maps a byte to the fp16 pair
+// (centroid[hi nibble], centroid[lo nibble]), replicated 32 times so that lane
+// l always reads bank l % 32 (no bank conflicts whatever the data).
+//
+// Tile = 64 tokens = 4 blocks of 16.
+//   scores   S^T_blk = K_blk (16 tokens x D) . Q^T (D x 16 columns).  Column n
+//            carries query head n % GP (GP = group size padded to 4, 8 or 16), so
+//            every block's result holds each head 16/GP times; lane (n, g) keeps
+//            the copy of block class n / GP.  After that selection a lane owns
+//            4 consecutive tokens of one head per kept block, all lanes busy.
+//            A lane's K operand is the 16 bytes it loaded (token n, quarter g of
+//            the row): the contraction index is permuted (k-step ks, group g,
+//            element e) <-> d = g*D/4 + 8*ks + e, and Q is loaded the same way.
+//   softmax  the V norm is folded into the exponent: w = 2^(s + log2|v| - M) lies
+//            in (0, 1] and is safe in fp16 whatever the scale of V; the
+//            denominator accumulates w / |v|.
+//   output   O (16 rows x D) += P (16 x 64 tokens) . V (64 tokens x D), where row
+//            n of P holds the weights of head n % GP for the tokens of block class
+//            n / GP only (zero elsewhere), so the lane that computed a weight is
+//            the lane that feeds it to the MFMA: no cross-lane movement.  The
+//            classes are summed once per split.  V's contraction index is the
+//            token, so a lane loads, for its 16 tokens of the tile, the bytes of
+//            D/16 consecutive coordinates (lane n <-> d = n*D/16 ...), and a
+//            2x2 nibble transpose of token pairs makes each byte hold the same
+//            coordinate of two consecutive tokens: again one lookup per byte.
+
+#include "fq_common.hpp"
+
+namespace fq {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kTinyNorm = 1e-30f;
+constexpr int kLutCopies = 32;
+constexpr int kLutWords = 256 * kLutCopies;   // per table
+
+struct DecodeParams {
+    const void* q_rot;          // (S, H_Q, D) query dtype, rotated space
+    const uint8_t* cache;       // (num_blocks, BS, H_KV*(D+8))
+    const int32_t* block_table; // (S, max_blocks)
+    const int32_t* seq_lens;    // (S,)
+    const float* centroids_k;
+    const float* centroids_v;
+    float* part_acc;            // (S, H_Q, NS, D)
+    float* part_m;              // (S, H_Q, NS)
+    float* part_l;              // (S, H_Q, NS)
+    int H_Q, H_KV, G;           // G = H_Q / H_KV
+    int max_blocks;
+    int num_blocks;
+    int num_splits;
+    int two_tables;             // centroids_v differs from centroids_k
+    float scale_log2e;          // sm_scale * log2(e)
+};
+
+__device__ __forceinline__ uint32_t byte_of(uint32_t w, int b) { return (w >> (8 * b)) & 0xffu; }
+
+template <int D, int BSL, int GP, int DT>
+__global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p) {
+    constexpr int BS = 1 << BSL;
+    constexpr int KS = D / 32;            // k-steps of the score product
+    constexpr int KW = D / 32;            // K dwords per lane per block
+    constexpr int DPL = D / 16;           // V coordinates per lane
+    constexpr int VW = DPL > 8 ? 2 : 1;   // V dwords per lane per token
+    constexpr int NB = 16 / GP;           // block classes
+    constexpr int NC = 4 / NB;            // kept blocks per lane per tile
+    constexpr int PAGES = 64 / BS;        // pages per tile
+    constexpr int ROW_HALF = D / 2;
+
+    extern __shared__ uint32_t lut[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;
+    const int n = lane & 15;
+    const int g = lane >> 4;
+    const int hd = n % GP;                // query head inside the group
+    const int bc_lane = n / GP;           // block class kept by this lane
+    const int split = blockIdx.x;
+    const int seq = blockIdx.y;
+    const int h = blockIdx.z * waves + wave;
+
+    // ---- byte -> (fp16, fp16) tables, one copy per LDS bank ----------------------
+    {
+        const int tables = p.two_tables ? 2 : 1;
+        for (int e = threadIdx.x; e < tables * kLutWords; e += blockDim.x) {
+            const float* c = e >= kLutWords ? p.centroids_v : p.centroids_k;
+            const int byte = (e % kLutWords) / kLutCopies;
+            lut[e] = pack_h2(_Float16(c[byte >> 4]), _Float16(c[byte & 15]));
+        }
+    }
+    __syncthreads();
+    if (h >= p.H_KV) return;
+    const uint32_t* lut_k = lut + (lane & 31);
+    const uint32_t* lut_v = lut_k + (p.two_tables ? kLutWords : 0);
+
+    int L = p.seq_lens[seq];
+    L = L < 0 ? 0 : L;
+    L = L > p.max_blocks * BS ? p.max_blocks * BS : L;
+    const int NS = p.num_splits;
+    const int chunk = (((L + NS - 1) / NS) + 63) & ~63;
+    const int begin = split * chunk;
+    const int end = L < begin + chunk ? L : begin + chunk;
+
+    const int hq_lane = h * p.G + n;      // for lanes n < G: the query head whose m, l they publish
+    if (begin >= end) {
+        if (g == 0 && n < p.G) {
+            const int64_t o = (int64_t(seq) * p.H_Q + hq_lane) * NS + split;
+            p.part_m[o] = -__builtin_inff();
+            p.part_l[o] = 0.0f;
+        }
+        return;
+    }
+
+    const int row_bytes = p.H_KV * (D + 8);
+    const int k_norm_off = p.H_KV * ROW_HALF + 4 * h;
+    const int v_idx_off = p.H_KV * (ROW_HALF + 4) + h * ROW_HALF;
+    const int v_norm_off = p.H_KV * (D + 4) + 4 * h;
+    const int32_t* bt = p.block_table + int64_t(seq) * p.max_blocks;
+    const int last_page_idx = (L - 1) >> BSL;
+
+    // ---- the query of this lane's head, as the B operand of the score product ----
+    half8 qh[KS];
+    float qscale;
+    {
+        float qf[KS][8];
+        float mx = 0.0f;
+        const bool live = hd < p.G;
+        const uint16_t* qsrc = reinterpret_cast<const uint16_t*>(p.q_rot) +
+                               (int64_t(seq) * p.H_Q + h * p.G + (live ? hd : 0)) * D + g * (D / 4);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint4v raw = *reinterpret_cast<const uint4v*>(qsrc + 8 * ks);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                qf[ks][2 * i] = live ? load_elem<DT>(uint16_t(w[i] & 0xffffu)) : 0.0f;
+                qf[ks][2 * i + 1] = live ? load_elem<DT>(uint16_t(w[i] >> 16)) : 0.0f;
+                mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(qf[ks][2 * i]), __builtin_fabsf(qf[ks][2 * i + 1])));
+            }
+        }
+        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 16));
+        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 32));
+        int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+        if (ex < -100 || ex > 100) ex = 0;
+        const float down = bits_to_float(uint32_t(127 - ex) << 23);
+        qscale = p.scale_log2e * bits_to_float(uint32_t(127 + ex) << 23);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qh[ks][e] = _Float16(qf[ks][e] * down);
+    }
+
+    // ---- per-tile register image ----------------------------------------------
+    struct Tile {
+        uint32_t k[4][KW];
+        uint32_t v[2][8][VW];
+        float kn[NC][4];
+        float vn[NC][4];
+    };
+
+    const uint8_t* cache = p.cache;
+    const int max_page = p.num_blocks - 1;
+
+    auto load_tile = [&](int t0, Tile& t) {
+        // the pages of this tile (wave-uniform)
+        int pg[PAGES];
+        const int p0 = t0 >> BSL;
+#pragma unroll
+        for (int i = 0; i < PAGES; ++i) {
+            int idx = p0 + i;
+            idx = idx > last_page_idx ? last_page_idx : idx;
+            int v = bt[idx];
+            v = v < 0 ? 0 : (v > max_page ? max_page : v);
+            pg[i] = v;
+        }
+        // byte offset of the row of tile-local token u (0..63); tokens at or past
+        // `end` read the last valid token of the split instead
+        auto row_off = [&](int blk, int r) -> int64_t {
+            int u = 16 * blk + r;
+            const int lim = end - 1 - t0;
+            int page;
+            if (u > lim) {
+                u = lim;
+                // u is now a run-time value: pick its page by comparison
+                page = pg[0];
+#pragma unroll
+                for (int i = 1; i < PAGES; ++i) page = (u >> BSL) >= i ? pg[i] : page;
+            } else if (BSL == 4) {
+                page = pg[blk];
+            } else if (BSL == 5) {
+                page = pg[blk >> 1];
+            } else {
+                page = (r & 8) ? pg[2 * blk + 1] : pg[2 * blk];
+            }
+            return (int64_t(page) * BS + ((t0 + u) & (BS - 1))) * row_bytes;
+        };
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            const uint8_t* src = cache + row_off(blk, n) + h * ROW_HALF + g * (D / 8);
+            if (KW == 4) {
+                const uint4v w = *reinterpret_cast<const uint4v*>(src);
+                t.k[blk][0] = w.x; t.k[blk][1] = w.y; t.k[blk][2] = w.z; t.k[blk][3] = w.w;
+            } else if (KW == 2) {
+                const uint2v w = *reinterpret_cast<const uint2v*>(src);
+                t.k[blk][0] = w.x; t.k[blk][1] = w.y;
+            } else {
+#pragma unroll
+                for (int q4 = 0; q4 < KW / 4; ++q4) {
+                    const uint4v w = *reinterpret_cast<const uint4v*>(src + 16 * q4);
+                    t.k[blk][4 * q4] = w.x; t.k[blk][4 * q4 + 1] = w.y;
+                    t.k[blk][4 * q4 + 2] = w.z; t.k[blk][4 * q4 + 3] = w.w;
+                }
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint8_t* src = cache + row_off(2 * ks + j / 4, 4 * g + j % 4) + v_idx_off + n * (DPL / 2);
+                if (DPL == 4) {
+                    t.v[ks][j][0] = *reinterpret_cast<const uint16_t*>(src);
+                } else if (DPL == 8) {
+                    t.v[ks][j][0] = *reinterpret_cast<const uint32_t*>(src);
+                } else {
+                    const uint2v w = *reinterpret_cast<const uint2v*>(src);
+                    t.v[ks][j][0] = w.x;
+                    t.v[ks][j][VW - 1] = w.y;
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // block c*NB + bc_lane is a run-time block: go through the generic path
+                const int blk = c * NB + bc_lane;
+                int u = 16 * blk + 4 * g + i;
+                const int lim = end - 1 - t0;
+                u = u > lim ? lim : u;
+                int page = pg[0];
+#pragma unroll
+                for (int q = 1; q < PAGES; ++q) page = (u >> BSL) >= q ? pg[q] : page;
+                const uint8_t* row = cache + (int64_t(page) * BS + ((t0 + u) & (BS - 1))) * row_bytes;
+                t.kn[c][i] = *reinterpret_cast<const float*>(row + k_norm_off);
+                t.vn[c][i] = *reinterpret_cast<const float*>(row + v_norm_off);
+            }
+        }
+    };
+
+    // ---- running state ----------------------------------------------------------
+    float4v O[DPL];
+#pragma unroll
+    for (int db = 0; db < DPL; ++db) O[db] = float4v{0.f, 0.f, 0.f, 0.f};
+    float M = -__builtin_inff();
+    float lsum = 0.0f;
+
+    Tile cur;
+    load_tile(begin, cur);
+
+    for (int t0 = begin; t0 < end; t0 += 64) {
+        Tile nxt;
+        const bool more = t0 + 64 < end;
+        if (more) load_tile(t0 + 64, nxt);
+
+        // ---- scores --------------------------------------------------------------
+        float4v sacc[4];
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            sacc[blk] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const uint32_t w = cur.k[blk][ks];
+                uint4v a;
+                a.x = lut_k[byte_of(w, 0) * kLutCopies];
+                a.y = lut_k[byte_of(w, 1) * kLutCopies];
+                a.z = lut_k[byte_of(w, 2) * kLutCopies];
+                a.w = lut_k[byte_of(w, 3) * kLutCopies];
+                sacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), qh[ks], sacc[blk], 0, 0, 0);
+            }
+        }
+        float a_[NC][4], rv[NC][4];
+        float tmax = -__builtin_inff();
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float s = sacc[c * NB][i];
+#pragma unroll
+                for (int bc = 1; bc < NB; ++bc) s = bc_lane == bc ? sacc[c * NB + bc][i] : s;
+                const float vn = __builtin_fmaxf(cur.vn[c][i], kTinyNorm);
+                rv[c][i] = __builtin_amdgcn_rcpf(vn);
+                float a = __builtin_fmaf(s * cur.kn[c][i], qscale, __builtin_amdgcn_logf(vn));
+                const int tok = t0 + 16 * (c * NB + bc_lane) + 4 * g + i;
+                a = tok < end ? a : -__builtin_inff();
+                a_[c][i] = a;
+                tmax = __builtin_fmaxf(tmax, a);
+            }
+        }
+#pragma unroll
+        for (int mask = GP; mask < 64; mask <<= 1) tmax = __builtin_fmaxf(tmax, xor_shuffle(tmax, mask));
+        const float Mnew = __builtin_fmaxf(M, tmax);
+        const float Ms = Mnew == -__builtin_inff() ? 0.0f : Mnew;
+        const float alpha = __builtin_amdgcn_exp2f(M - Ms);
+        M = Mnew;
+
+        _Float16 wh[NC][4];
+        float psum = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float w = __builtin_amdgcn_exp2f(a_[c][i] - Ms);
+                psum = __builtin_fmaf(w, rv[c][i], psum);
+                wh[c][i] = _Float16(w);
+            }
+        }
+        lsum = __builtin_fmaf(lsum, alpha, psum);
+
+        // ---- rescale the accumulators when a maximum moved --------------------------
+        if (__any(alpha != 1.0f)) {
+            float ar[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * g + i, kWave);
+#pragma unroll
+            for (int db = 0; db < DPL; ++db)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) O[db][i] *= ar[i];
+        }
+
+        // ---- weights as the A operand: row n feeds only its own block class -------------
+        half8 pa[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                constexpr _Float16 zero = _Float16(0.0f);
+                const int blk = 2 * ks + hf;
+                const int c = blk / NB, bc = blk % NB;
+                const bool mine = bc_lane == bc;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) pa[ks][4 * hf + i] = mine ? wh[c][i] : zero;
+            }
+        }
+
+        // ---- O += P . V ---------------------------------------------------------------
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            uint32_t X[4][VW], Y[4][VW];
+#pragma unroll
+            for (int jp = 0; jp < 4; ++jp) {
+#pragma unroll
+                for (int wv = 0; wv < VW; ++wv) {
+                    const uint32_t A = cur.v[ks][2 * jp][wv], B = cur.v[ks][2 * jp + 1][wv];
+                    X[jp][wv] = (A & 0xF0F0F0F0u) | ((B >> 4) & 0x0F0F0F0Fu);
+                    Y[jp][wv] = ((A << 4) & 0xF0F0F0F0u) | (B & 0x0F0F0F0Fu);
+                }
+            }
+#pragma unroll
+            for (int db = 0; db < DPL; ++db) {
+                const int bi = db / 2;
+                uint4v b;
+                uint32_t src[4];
+#pragma unroll
+                for (int jp = 0; jp < 4; ++jp) src[jp] = (db & 1) ? Y[jp][bi / 4] : X[jp][bi / 4];
+                b.x = lut_v[byte_of(src[0], bi % 4) * kLutCopies];
+                b.y = lut_v[byte_of(src[1], bi % 4) * kLutCopies];
+                b.z = lut_v[byte_of(src[2], bi % 4) * kLutCopies];
+                b.w = lut_v[byte_of(src[3], bi % 4) * kLutCopies];
+                O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[ks], __builtin_bit_cast(half8, b), O[db], 0, 0, 0);
+            }
+        }
+        if (more) cur = nxt;
+    }
+
+    // ---- publish the partial of this split --------------------------------------------
+#pragma unroll
+    for (int mask = GP; mask < 64; mask <<= 1) lsum += xor_shuffle(lsum, mask);
+#pragma unroll
+    for (int db = 0; db < DPL; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = O[db][i];
+#pragma unroll
+            for (int mask = 4 * GP; mask < 64; mask <<= 1) v += xor_shuffle(v, mask);
+            O[db][i] = v;
+        }
+    if (g == 0 && n < p.G) {
+        const int64_t o = (int64_t(seq) * p.H_Q + hq_lane) * NS + split;
+        p.part_m[o] = M;
+        p.part_l[o] = lsum;
+    }
+    if (g < GP / 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int head = 4 * g + i;
+            if (head < p.G) {
+                float* dst = p.part_acc + ((int64_t(seq) * p.H_Q + h * p.G + head) * NS + split) * D + n * DPL;
+#pragma unroll
+                for (int q4 = 0; q4 < DPL / 4; ++q4) {
+                    const float4v v = {O[4 * q4][i], O[4 * q4 + 1][i], O[4 * q4 + 2][i], O[4 * q4 + 3][i]};
+                    *reinterpret_cast<float4v*>(dst + 4 * q4) = v;
+                }
+            }
+        }
+    }
+}
+
+// q_rot[s, h, j] = sum_k q[s, h, k] * R[j, k], rounded to the query dtype
+// (src/flashquant/kernels/paged_decode.py:113).  One workgroup per (sequence, 8 heads).
+template <int D, int DT>
+__global__ __launch_bounds__(256) void rotate_q_kernel(const uint16_t* __restrict__ q, const float* __restrict__ R,
+                                                       uint16_t* __restrict__ q_rot, int H_Q) {
+    constexpr int HB = 8;
+    __shared__ float qs[HB][D];
+    const int seq = blockIdx.x, h0 = blockIdx.y * HB;
+    const int heads = H_Q - h0 < HB ? H_Q - h0 : HB;
+    for (int i = threadIdx.x; i < heads * D; i += 256)
+        qs[i / D][i % D] = load_elem<DT>(q[(int64_t(seq) * H_Q + h0) * D + i]);
+    __syncthreads();
+    for (int j = threadIdx.x; j < D; j += 256) {
+        float acc[HB];
+#pragma unroll
+        for (int hh = 0; hh < HB; ++hh) acc[hh] = 0.0f;
+        const float4v* row = reinterpret_cast<const float4v*>(R + int64_t(j) * D);
+        for (int k4 = 0; k4 < D / 4; ++k4) {
+            const float4v r = row[k4];
+#pragma unroll
+            for (int hh = 0; hh < HB; ++hh) {
+                acc[hh] = __builtin_fmaf(qs[hh][4 * k4], r.x, acc[hh]);
+                acc[hh] = __builtin_fmaf(qs[hh][4 * k4 + 1], r.y, acc[hh]);
+                acc[hh] = __builtin_fmaf(qs[hh][4 * k4 + 2], r.z, acc[hh]);
+                acc[hh] = __builtin_fmaf(qs[hh][4 * k4 + 3], r.w, acc[hh]);
+            }
+        }
+        for (int hh = 0; hh < heads; ++hh)
+            q_rot[(int64_t(seq) * H_Q + h0 + hh) * D + j] = store_elem<DT>(acc[hh]);
+    }
+}
+
+// Combine of the split partials: out_rot = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
+// (0 when every split is empty), rounded to the query dtype as the reference's
+// rotated-space result is (cpu_reference.py:366), then multiplied by R in float32
+// and rounded again (paged_decode.py:123).  One workgroup per (sequence, 8 heads).
+template <int D, int DT>
+__global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restrict__ part_acc,
+                                                            const float* __restrict__ part_m,
+                                                            const float* __restrict__ part_l,
+                                                            const float* __restrict__ R, uint16_t* __restrict__ out,
+                                                            int H_Q, int NS) {
+    constexpr int HB = 8;
+    __shared__ float os[HB][D];
+    const int seq = blockIdx.x, h0 = blockIdx.y * HB;
+    const int heads = H_Q - h0 < HB ? H_Q - h0 : HB;
+    for (int i = threadIdx.x; i < heads * D; i += 256) {
+        const int hh = i / D, d = i % D;
+        const int64_t base = (int64_t(seq) * H_Q + h0 + hh) * NS;
+        float mstar = -__builtin_inff();
+        for (int s = 0; s < NS; ++s) mstar = __builtin_fmaxf(mstar, part_m[base + s]);
+        float num = 0.0f, den = 0.0f;
+        for (int s = 0; s < NS; ++s) {
+            const float m = part_m[base + s];
+            if (m == -__builtin_inff()) continue;
+            const float w = __builtin_amdgcn_exp2f(m - mstar);
+            num = __builtin_fmaf(part_acc[(base + s) * D + d], w, num);
+            den = __builtin_fmaf(part_l[base + s], w, den);
+        }
+        const float v = den > 0.0f ? num / den : 0.0f;
+        os[hh][d] = load_elem<DT>(store_elem<DT>(v));
+    }
+    __syncthreads();
+    if (R == nullptr) {
+        for (int i = threadIdx.x; i < heads * D; i += 256)
+            out[(int64_t(seq) * H_Q + h0) * D + i] = store_elem<DT>(os[i / D][i % D]);
+        return;
+    }
+    for (int j = threadIdx.x; j < D; j += 256) {
+        float acc[HB];
+#pragma unroll
+        for (int hh = 0; hh < HB; ++hh) acc[hh] = 0.0f;
+        for (int d = 0; d < D; ++d) {
+            const float r = R[int64_t(d) * D + j];
+#pragma unroll
+            for (int hh = 0; hh < HB; ++hh) acc[hh] = __builtin_fmaf(os[hh][d], r, acc[hh]);
+        }
+        for (int hh = 0; hh < heads; ++hh)
+            out[(int64_t(seq) * H_Q + h0 + hh) * D + j] = store_elem<DT>(acc[hh]);
+    }
+}
+
+struct DecodeLaunch {
+    const void* q; const uint8_t* cache; const int32_t* bt; const int32_t* lens;
+    const float* ck; const float* cv; const float* R; void* out;
+    int S, H_Q, H_KV, D, BS, max_blocks; int64_t num_blocks; float sm_scale; int NS;
+    uint8_t* ws; hipStream_t stream;
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct WorkspaceLayout {
+    size_t acc, m, l, qrot, total;
+};
+inline WorkspaceLayout workspace_layout(int S, int H_Q, int D, int NS) {
+    WorkspaceLayout w;
+    const size_t rows = size_t(S) * H_Q;
+    w.acc = 0;
+    w.m = align_up(w.acc + rows * NS * D * sizeof(float), 256);
+    w.l = align_up(w.m + rows * NS * sizeof(float), 256);
+    w.qrot = align_up(w.l + rows * NS * sizeof(float), 256);
+    w.total = align_up(w.qrot + rows * D * 2, 256);
+    return w;
+}
+
+template <int D, int DT>
+int launch_decode(const DecodeLaunch& a) {
+    const WorkspaceLayout w = workspace_layout(a.S, a.H_Q, D, a.NS);
+    const int G = a.H_Q / a.H_KV;
+    const void* q_rot = a.q;
+    if (a.R) {
+        uint16_t* qr = reinterpret_cast<uint16_t*>(a.ws + w.qrot);
+        hipLaunchKernelGGL((rotate_q_kernel<D, DT>), dim3(a.S, (a.H_Q + 7) / 8), dim3(256), 0, a.stream,
+                           reinterpret_cast<const uint16_t*>(a.q), a.R, qr, a.H_Q);
+        q_rot = qr;
+    }
+    DecodeParams p;
+    p.q_rot = q_rot; p.cache = a.cache; p.block_table = a.bt; p.seq_lens = a.lens;
+    p.centroids_k = a.ck; p.centroids_v = a.cv;
+    p.part_acc = reinterpret_cast<float*>(a.ws + w.acc);
+    p.part_m = reinterpret_cast<float*>(a.ws + w.m);
+    p.part_l = reinterpret_cast<float*>(a.ws + w.l);
+    p.H_Q = a.H_Q; p.H_KV = a.H_KV; p.G = G; p.max_blocks = a.max_blocks;
+    p.num_blocks = int(a.num_blocks); p.num_splits = a.NS;
+    p.two_tables = a.ck != a.cv ? 1 : 0;
+    p.scale_log2e = a.sm_scale * kLog2e;
+
+    const int waves = a.H_KV < 8 ? a.H_KV : 8;
+    const dim3 grid(a.NS, a.S, (a.H_KV + waves - 1) / waves), block(64 * waves);
+    const size_t lds = size_t(p.two_tables ? 2 : 1) * kLutWords * sizeof(uint32_t);
+#define FQ_DECODE_GP(BSL, GPV) \
+    hipLaunchKernelGGL((paged_decode_kernel<D, BSL, GPV, DT>), grid, block, lds, a.stream, p)
+#define FQ_DECODE_BS(BSL)                       \
+    do {                                        \
+        if (G <= 4) FQ_DECODE_GP(BSL, 4);       \
+        else if (G <= 8) FQ_DECODE_GP(BSL, 8);  \
+        else FQ_DECODE_GP(BSL, 16);             \
+    } while (0)
+    switch (a.BS) {
+        case 8: FQ_DECODE_BS(3); break;
+        case 16: FQ_DECODE_BS(4); break;
+        default: FQ_DECODE_BS(5); break;
+    }
+#undef FQ_DECODE_BS
+#undef FQ_DECODE_GP
+    hipLaunchKernelGGL((reduce_rotate_kernel<D, DT>), dim3(a.S, (a.H_Q + 7) / 8), dim3(256), 0, a.stream,
+                       p.part_acc, p.part_m, p.part_l, a.R, reinterpret_cast<uint16_t*>(a.out), a.H_Q, a.NS);
+    return fq_host::check_launch();
+}
+
+}  // namespace fq
+
+namespace fq_host {
+int device_cu_count();
+}
+
+extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_size, int max_blocks_per_seq) {
+    if (num_seqs <= 0 || H_KV <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 1;
+    const int64_t max_ctx = int64_t(block_size) * max_blocks_per_seq;
+    const int64_t tiles = (max_ctx + 63) / 64;
+    // aim at two wavefronts per SIMD over the whole chip, one wavefront per (sequence, KV head, split)
+    const int64_t target_waves = int64_t(fq_host::device_cu_count()) * 8;
+    int64_t ns = (target_waves + int64_t(num_seqs) * H_KV - 1) / (int64_t(num_seqs) * H_KV);
+    if (ns > tiles) ns = tiles;
+    if (ns > 64) ns = 64;
+    if (ns < 1) ns = 1;
+    return int(ns);
+}
+
+extern "C" size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_KV, int D, int block_size,
+                                                  int max_blocks_per_seq, int num_splits) {
+    if (num_seqs <= 0 || H_Q <= 0 || H_KV <= 0 || D <= 0) return 0;
+    if (num_splits <= 0) num_splits = fq_paged_decode_auto_splits(num_seqs, H_KV, block_size, max_blocks_per_seq);
+    return fq::workspace_layout(num_seqs, H_Q, D, num_splits).total;
+}
+
+extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
+                                       const int32_t* seq_lens, const float* centroids_k,
+                                       const float* centroids_v, const float* rotation, void* out,
+                                       int num_seqs, int H_Q, int H_KV, int D, int block_size,
+                                       int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype,
+                                       int num_splits, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace fq;
+    if (num_seqs < 0 || H_Q <= 0 || H_KV <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0 || num_splits < 0)
+        return FQ_ERR_BAD_SHAPE;
+    if (H_Q % H_KV != 0 || H_Q / H_KV > 16) return FQ_ERR_BAD_SHAPE;
+    if (num_blocks > 0x7fffffffLL || num_seqs > 65535 || (H_KV + 7) / 8 > 65535) return FQ_ERR_BAD_SHAPE;
+    if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
+    if (block_size != 8 && block_size != 16 && block_size != 32) return FQ_ERR_UNSUPPORTED_BLOCK;
+    if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
+    if (num_seqs == 0) return FQ_OK;
+    if (!q || !kv_cache || !block_table || !seq_lens || !centroids_k || !centroids_v || !out)
+        return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16) || !fq_host::aligned(kv_cache, 16) ||
+        (rotation && !fq_host::aligned(rotation, 16)))
+        return FQ_ERR_MISALIGNED;
+    if (num_splits == 0) num_splits = fq_paged_decode_auto_splits(num_seqs, H_KV, block_size, max_blocks_per_seq);
+    if (num_splits > 65535) return FQ_ERR_BAD_SHAPE;
+    const size_t need = workspace_layout(num_seqs, H_Q, D, num_splits).total;
+    if (!workspace || workspace_bytes < need) return FQ_ERR_WORKSPACE;
+    if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;
+
+    DecodeLaunch a{q, kv_cache, block_table, seq_lens, centroids_k, centroids_v, rotation, out,
+                   num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, num_splits,
+                   static_cast<uint8_t*>(workspace), static_cast<hipStream_t>(stream)};
+#define FQ_DECODE_D(DD)                                                                       \
+    case DD: return dtype == FQ_F16 ? launch_decode<DD, FQ_F16>(a) : launch_decode<DD, FQ_BF16>(a);
+    switch (D) {
+        FQ_DECODE_D(64)
+        FQ_DECODE_D(128)
+        FQ_DECODE_D(256)
+        default: return FQ_ERR_UNSUPPORTED_DIM;
+    }
+#undef FQ_DECODE_D
+}

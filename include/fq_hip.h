@@ -1,0 +1,135 @@
+/*
+ * fq_hip.h - C ABI of libfq_hip.so, the MI355X (gfx950) implementation of the
+ * TurboQuant TQ4 KV-cache kernels.
+ *
+ * Every entry point takes plain device pointers, sizes and an opaque HIP
+ * stream (hipStream_t passed as void*; NULL is the default stream), launches
+ * asynchronously on that stream, allocates nothing, never synchronises and
+ * never aborts: it returns an fq_status code.  All buffers are owned by the
+ * caller.  Entry points whose kernels need scratch memory take a caller-owned
+ * workspace whose size comes from the matching *_workspace_bytes() function.
+ *
+ * Each declaration cites the launcher of the reference (paths relative to the
+ * reference checkout) whose role it takes, or the Python call site that
+ * defines the operator where the reference has no working launcher.
+ */
+#ifndef FQ_HIP_H
+#define FQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FQ_ABI_VERSION 1
+
+typedef enum fq_status {
+    FQ_OK = 0,
+    FQ_ERR_NULL_POINTER = 1,      /* a required pointer argument is NULL           */
+    FQ_ERR_UNSUPPORTED_DIM = 2,   /* head_dim not in {64, 128, 256}                */
+    FQ_ERR_UNSUPPORTED_BLOCK = 3, /* page size not in {8, 16, 32}                  */
+    FQ_ERR_UNSUPPORTED_DTYPE = 4, /* dtype code not accepted by this entry point   */
+    FQ_ERR_BAD_SHAPE = 5,         /* negative size, H_Q not a multiple of H_KV ... */
+    FQ_ERR_MISALIGNED = 6,        /* a pointer or stride breaks the stated alignment */
+    FQ_ERR_WORKSPACE = 7,         /* workspace missing or too small                */
+    FQ_ERR_LAUNCH = 8             /* the HIP runtime refused the launch            */
+} fq_status;
+
+typedef enum fq_dtype {
+    FQ_F16 = 0,
+    FQ_BF16 = 1,
+    FQ_F32 = 2
+} fq_dtype;
+
+/* Library identification and error text. */
+int fq_abi_version(void);
+const char* fq_status_string(int status);
+/* Text of the last HIP runtime error seen by this thread ("" if none). */
+const char* fq_last_hip_error(void);
+
+/*
+ * TQ4 compress.  Takes the role of tq4_compress_cuda
+ * (csrc/cuda/compress.cuh:38-48); operator defined by compress_reference
+ * (src/flashquant/kernels/cpu_reference.py:22-61).
+ *
+ *   x           (M, D) fp16 or bf16 rows, contiguous, 16-byte aligned
+ *   rot_T_even  (D, D/2) float32 = rotation.T[:, 0::2], contiguous
+ *   rot_T_odd   (D, D/2) float32 = rotation.T[:, 1::2], contiguous
+ *   boundaries  (15,) float32, ascending
+ *   packed      (M, D/2) uint8 out, 16-byte aligned: byte j = idx[2j]<<4 | idx[2j+1]
+ *   norms       (M,) float32 out
+ * D in {64, 128, 256}.  M == 0 is a no-op.
+ */
+int fq_tq4_compress(const void* x, int x_dtype,
+                    const float* rot_T_even, const float* rot_T_odd,
+                    const float* boundaries,
+                    uint8_t* packed, float* norms,
+                    int64_t M, int D, void* stream);
+
+/*
+ * TQ4 decompress.  Takes the role of tq4_decompress_cuda
+ * (csrc/cuda/decompress.cuh:40-48); operator defined by decompress_reference
+ * (src/flashquant/kernels/cpu_reference.py:64-94) followed by the cast of
+ * src/flashquant/kernels/decompress.py:80-81.
+ *
+ *   packed     (M, D/2) uint8, 4-byte aligned
+ *   norms      (M,) float32
+ *   centroids  (16,) float32
+ *   out        (M, D) fp16 / bf16 / float32, 16-byte aligned; rotated space,
+ *              out[2j] from the high nibble of byte j, out[2j+1] from the low
+ */
+int fq_tq4_decompress(const uint8_t* packed, const float* norms,
+                      const float* centroids,
+                      void* out, int out_dtype,
+                      int64_t M, int D, void* stream);
+
+/*
+ * Split-K paged decode from the packed TQ4 cache, un-rotated query in,
+ * original-space output out.  Takes the roles of paged_tq4_decode_cuda
+ * (csrc/cuda/paged_decode.cu:346-368) and split_k_reduce_cuda
+ * (csrc/cuda/split_k_reduce.cu:145-154) together with the query pre-rotation
+ * and output post-rotation of src/flashquant/kernels/paged_decode.py:112-128;
+ * operator defined by paged_decode_reference
+ * (src/flashquant/kernels/cpu_reference.py:230-368).
+ *
+ *   q            (S, H_Q, D) fp16/bf16, contiguous
+ *   kv_cache     (num_blocks, block_size, H_KV*(D+8)) uint8, 16-byte aligned
+ *   block_table  (S, max_blocks_per_seq) int32
+ *   seq_lens     (S,) int32; a length of 0 gives a zero output row
+ *   centroids_k, centroids_v  (16,) float32
+ *   rotation     (D, D) float32, or NULL: q is taken as already rotated and
+ *                out is left in rotated space
+ *   out          (S, H_Q, D) same dtype as q
+ *   num_splits   >= 1, or 0 to let the library choose
+ *   workspace    fq_paged_decode_workspace_bytes(...) bytes, 256-byte aligned
+ * D in {64, 128, 256}; block_size in {8, 16, 32}; H_Q a multiple of H_KV with
+ * H_Q / H_KV <= 16.
+ */
+int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
+                            const int32_t* block_table, const int32_t* seq_lens,
+                            const float* centroids_k, const float* centroids_v,
+                            const float* rotation, void* out,
+                            int num_seqs, int H_Q, int H_KV, int D,
+                            int block_size, int max_blocks_per_seq,
+                            int64_t num_blocks, float sm_scale, int dtype,
+                            int num_splits,
+                            void* workspace, size_t workspace_bytes,
+                            void* stream);
+
+/* Number of splits fq_split_k_paged_decode uses when num_splits == 0
+ * (counterpart of paged_tq4_decode_num_splits, csrc/cuda/paged_decode.cu:424-426,
+ * which is a constant 4 there). */
+int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_size,
+                                int max_blocks_per_seq);
+
+/* Bytes of workspace for the given launch; num_splits == 0 means "auto". */
+size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_KV, int D,
+                                       int block_size, int max_blocks_per_seq,
+                                       int num_splits);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FQ_HIP_H */
