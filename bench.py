@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the TQ4 KV-cache hot path on one MI355X.
+
+Headline (one JSON line on stdout): split-K paged TQ4 decode at the
+Llama-3-8B single-layer shape of BASELINE.json configs[2] (32 query heads over
+8 KV heads, d=128, batch 32, 4096 tokens of context, 16-token pages, seeded
+random block tables, bf16 queries).  A step is one decode call for the whole
+batch: query rotation + split-K decode + split reduce and output rotation.
+`value` is the algorithmic KV bytes of a step (context tokens x KV heads x 136)
+divided by the step time, with a different cache every step so that the 256 MB
+last-level cache cannot serve it (the "cold" figure).  The same line carries
+the roofline of the dominant kernel, the CPU baseline (the oracle timed on the
+host cores) and, under "extra", the standalone compress / decompress figures
+of configs[1].
+
+    python bench.py --gpus 1 --steps 50 --warmup 5
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published peak
+H_Q, H_KV, D, BS = 32, 8, 128, 16
+BATCH, CTX = 32, 4096
+ROW_BYTES = H_KV * (D + 8)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def outlier_rows(n, h, d, seed, device, dtype=torch.bfloat16):
+    """N(0,1) rows, 4 channels per head scaled x10 (the benchmark's outlier rule)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    x = torch.randn(n, h, d, generator=g, device=device, dtype=torch.float32)
+    gc = torch.Generator(device="cpu").manual_seed(seed)
+    for head in range(h):
+        ch = torch.randperm(d, generator=gc)[:4].to(device)
+        x[:, head, ch] *= 10.0
+    return x.to(dtype)
+
+
+def build_cache(K, book, seed, device):
+    """One packed paged cache for the decode workload, filled through the HIP
+    compress kernel, with a seeded random block table."""
+    cent, bnd, rot = book
+    n_tok = BATCH * CTX
+    pages_per_seq = CTX // BS
+    n_pages = BATCH * pages_per_seq
+    k = outlier_rows(n_tok, H_KV, D, seed, device)
+    v = outlier_rows(n_tok, H_KV, D, seed + 1, device)
+    kp, kn = K.tq4_compress(k, rot, bnd)
+    vp, vn = K.tq4_compress(v, rot, bnd)
+    del k, v
+    row = torch.empty(n_tok, ROW_BYTES, dtype=torch.uint8, device=device)
+    o1 = H_KV * (D // 2)
+    o2 = o1 + 4 * H_KV
+    o3 = o2 + H_KV * (D // 2)
+    row[:, :o1] = kp.reshape(n_tok, -1)
+    row[:, o1:o2] = kn.reshape(n_tok, H_KV).contiguous().view(torch.uint8)
+    row[:, o2:o3] = vp.reshape(n_tok, -1)
+    row[:, o3:] = vn.reshape(n_tok, H_KV).contiguous().view(torch.uint8)
+    g = torch.Generator(device="cpu").manual_seed(2002 + seed)
+    table = torch.randperm(n_pages, generator=g).reshape(BATCH, pages_per_seq).to(torch.int32)
+    cache = torch.empty(n_pages, BS, ROW_BYTES, dtype=torch.uint8, device=device)
+    t = torch.arange(CTX)
+    slots = (table.long()[:, t // BS] * BS + (t % BS)).reshape(-1).to(device)   # token (s, t) -> slot
+    cache.view(-1, ROW_BYTES)[slots] = row
+    return cache, table.to(device)
+
+
+def time_events(fn, iters):
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(iters):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters   # ms per call
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--skip-extra", action="store_true", help="omit the compress / decompress legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this benchmark runs on exactly one GPU (the path has no collectives); use --gpus 1")
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible")
+        sys.exit(3)
+
+    from flashquant_amd import kernels as K
+    from flashquant_amd import load_native
+    from oracle import tq_oracle as O
+
+    C = load_native()
+    dev = torch.device("cuda:0")
+    cent, bnd = O.lloyd_max_gaussian(D, 4)
+    rot = O.haar_orthogonal(D, 42)
+    book = (cent.to(dev), bnd.to(dev), rot.to(dev))
+    cent_d, _, rot_d = book
+    scale = 1.0 / math.sqrt(D)
+
+    # ---- decode workload -----------------------------------------------------------
+    n_caches = 4                      # 4 x 143 MB > 256 MB last-level cache
+    caches = [build_cache(K, book, 1100 + 10 * i, dev) for i in range(n_caches)]
+    gq = torch.Generator(device="cpu").manual_seed(1002)
+    q = torch.randn(BATCH, H_Q, D, generator=gq).to(torch.bfloat16).to(dev)
+    lens = torch.full((BATCH,), CTX, dtype=torch.int32, device=dev)
+    out = torch.empty_like(q)
+    kv_bytes = BATCH * CTX * ROW_BYTES
+    n_splits = C.paged_decode_auto_splits(BATCH, H_KV, BS, CTX // BS)
+
+    def step(i):
+        cache, table = caches[i % n_caches]
+        K.split_k_paged_decode(q, cache, table, lens, cent_d, cent_d, rot_d, H_KV, D, BS,
+                               sm_scale=scale, out=out)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ev_ms = time_events(step, args.steps)
+    step_ms = min(wall_ms, ev_ms) if ev_ms > 0 else wall_ms
+    warm_ms = time_events(lambda i: step(0), args.steps)
+
+    # ---- dominant kernel alone (the split-K decode), cold ----------------------------
+    q_rot = C.rotate_query(q, rot_d)
+    parts = (torch.empty(BATCH, H_Q, n_splits, D, device=dev), torch.empty(BATCH, H_Q, n_splits, device=dev),
+             torch.empty(BATCH, H_Q, n_splits, device=dev))
+
+    def decode_only(i):
+        cache, table = caches[i % n_caches]
+        C.paged_tq4_decode_partials(q_rot, cache, table, lens, cent_d, cent_d, H_KV, D, BS, scale, n_splits, parts)
+
+    for i in range(args.warmup):
+        decode_only(i)
+    kern_ms = time_events(decode_only, args.steps)
+    achieved = kv_bytes / (kern_ms * 1e-3) / 1e9
+
+    extra = {
+        "decode_tokens_per_s": BATCH / (step_ms * 1e-3),
+        "decode_step_us_cold": step_ms * 1e3,
+        "decode_step_us_warm": warm_ms * 1e3,
+        "decode_step_us_wallclock": wall_ms * 1e3,
+        "decode_gbps_warm": kv_bytes / (warm_ms * 1e-3) / 1e9,
+        "decode_pct_hbm_peak_cold": 100.0 * kv_bytes / (step_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "decode_kernel_us_cold": kern_ms * 1e3,
+        "num_splits": n_splits,
+        "kv_bytes_per_step": kv_bytes,
+    }
+
+    # ---- CPU baseline: the oracle on the host cores, bounded sample ---------------------
+    cpu = None
+    if not args.skip_cpu:
+        cache_h = caches[0][0].cpu()
+        table_h = caches[0][1].cpu()
+        q_h = q.cpu()
+        lens_h = lens.cpu()
+        done, spent = 0, 0.0
+        while done < BATCH and spent < 15.0:
+            t1 = time.perf_counter()
+            O.split_k_paged_decode(q_h[done:done + 1], cache_h, table_h[done:done + 1], lens_h[done:done + 1],
+                                   cent, cent, rot, H_KV, D, BS, sm_scale=scale)
+            spent += time.perf_counter() - t1
+            done += 1
+        cpu = {
+            "value": done * CTX * ROW_BYTES / spent / 1e9,
+            "unit": "GB/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{done} of {BATCH} sequences of the same workload (vectorised-gather form of the "
+                      f"reference's CPU fallback), {spent:.1f} s",
+        }
+        del cache_h
+
+    # ---- standalone compress / decompress (configs[1]) -----------------------------------
+    if not args.skip_extra:
+        del caches
+        torch.cuda.empty_cache()
+        rows_tok = 32 * 65536
+        x = outlier_rows(rows_tok, H_KV, D, 1001, dev)
+        packed = torch.empty(rows_tok, H_KV, D // 2, dtype=torch.uint8, device=dev)
+        norms = torch.empty(rows_tok, H_KV, 1, device=dev)
+        ev, od = O.split_rotation(rot)
+        ev, od = ev.to(dev), od.to(dev)
+        bnd_d = book[1]
+        for _ in range(2):
+            K.tq4_compress(x, rot_d, bnd_d, rotation_T_even=ev, rotation_T_odd=od, out=(packed, norms))
+        c_ms = time_events(lambda i: K.tq4_compress(x, rot_d, bnd_d, rotation_T_even=ev, rotation_T_odd=od,
+                                                    out=(packed, norms)), 5)
+        nrows = rows_tok * H_KV
+        extra.update({
+            "compress_rows": nrows,
+            "compress_ms": c_ms,
+            "compress_mrows_per_s": nrows / (c_ms * 1e-3) / 1e6,
+            "compress_mtok_per_s": rows_tok / (c_ms * 1e-3) / 1e6,
+            "compress_gbps": nrows * 324 / (c_ms * 1e-3) / 1e9,
+            "compress_pct_hbm_peak": 100.0 * nrows * 324 / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "compress_tflops_fp16_mfma": nrows * 2 * 2 * D * D / (c_ms * 1e-3) / 1e12,
+        })
+        del x
+        torch.cuda.empty_cache()
+        y = torch.empty(rows_tok, H_KV, D, dtype=torch.bfloat16, device=dev)
+        for _ in range(2):
+            K.tq4_decompress(packed, norms, cent_d, torch.bfloat16, out=y)
+        d_ms = time_events(lambda i: K.tq4_decompress(packed, norms, cent_d, torch.bfloat16, out=y), 5)
+        extra.update({
+            "decompress_ms": d_ms,
+            "decompress_gbps": nrows * 324 / (d_ms * 1e-3) / 1e9,
+            "decompress_pct_hbm_peak": 100.0 * nrows * 324 / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        })
+
+    value = kv_bytes / (step_ms * 1e-3) / 1e9
+    line = {
+        "metric": "tq4_paged_decode_hbm_gbps",
+        "value": value,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": step_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[2]: split-K paged TQ4 decode, Llama-3-8B layer shape",
+            "batch": BATCH, "context": CTX, "q_heads": H_Q, "kv_heads": H_KV, "head_dim": D,
+            "page_tokens": BS, "query_dtype": "bf16", "cache": "cold (4 caches of 143 MB in rotation)",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": None,
+            "kernel": "paged_decode_kernel<128,4,4,bf16>",
+        },
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -158,6 +158,91 @@ at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache,
     return result;
 }
 
+at::Tensor rotate_query(const at::Tensor& q, const at::Tensor& rotation) {
+    fqbind::require_gpu(q, "q");
+    require(q.dim() == 3 && (q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16),
+            "q must be float16/bfloat16 of shape (num_seqs, H_Q, D)");
+    require(rotation.dim() == 2 && rotation.size(0) == q.size(2) && rotation.size(1) == q.size(2) &&
+                rotation.scalar_type() == at::kFloat,
+            "rotation must be float32 of shape (D, D)");
+    c10::DeviceGuard guard(q.device());
+    const at::Tensor qc = q.contiguous();
+    const at::Tensor rot = rotation.to(q.device()).contiguous();
+    at::Tensor out = at::empty_like(qc);
+    const int st = fq_rotate_query(qc.data_ptr(), rot.data_ptr<float>(), out.data_ptr(), q.size(0), int(q.size(1)),
+                                   int(q.size(2)), fqbind::dtype_code(q.scalar_type(), "rotate_query"),
+                                   fqbind::current_stream(q));
+    fqbind::raise_on_error(st, "rotate_query");
+    return out;
+}
+
+using OptTriple = std::optional<std::tuple<at::Tensor, at::Tensor, at::Tensor>>;
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor> paged_tq4_decode_partials(
+    const at::Tensor& q_rot, const at::Tensor& kv_cache, const at::Tensor& block_table, const at::Tensor& seq_lens,
+    const at::Tensor& centroids_k, const at::Tensor& centroids_v, int64_t num_kv_heads, int64_t head_dim,
+    int64_t block_size, double sm_scale, int64_t num_splits, const OptTriple& out) {
+    fqbind::require_gpu(q_rot, "q_rot");
+    fqbind::require_gpu(kv_cache, "kv_cache");
+    require(q_rot.dim() == 3 && q_rot.size(2) == head_dim && q_rot.is_contiguous(), "q_rot must be contiguous (S, H_Q, D)");
+    require(kv_cache.dim() == 3 && kv_cache.scalar_type() == at::kByte && kv_cache.is_contiguous() &&
+                kv_cache.size(1) == block_size && kv_cache.size(2) == num_kv_heads * (head_dim + 8),
+            "kv_cache must be contiguous uint8 (num_blocks, block_size, num_kv_heads * (head_dim + 8))");
+    require(block_table.is_cuda() && block_table.is_contiguous() && block_table.scalar_type() == at::kInt &&
+                block_table.dim() == 2 && block_table.size(0) == q_rot.size(0),
+            "block_table must be a contiguous int32 GPU tensor (S, max_blocks)");
+    require(seq_lens.is_cuda() && seq_lens.is_contiguous() && seq_lens.scalar_type() == at::kInt &&
+                seq_lens.numel() == q_rot.size(0),
+            "seq_lens must be a contiguous int32 GPU tensor (S,)");
+    require(centroids_k.is_cuda() && centroids_v.is_cuda() && centroids_k.numel() == 16 && centroids_v.numel() == 16 &&
+                centroids_k.scalar_type() == at::kFloat && centroids_v.scalar_type() == at::kFloat,
+            "centroids must be 16 float32 values on the GPU");
+    require(num_splits >= 1, "num_splits must be >= 1");
+    c10::DeviceGuard guard(q_rot.device());
+    const int64_t S = q_rot.size(0), HQ = q_rot.size(1);
+    at::Tensor acc, m, l;
+    if (out.has_value()) {
+        acc = std::get<0>(*out); m = std::get<1>(*out); l = std::get<2>(*out);
+        require(acc.is_cuda() && acc.is_contiguous() && acc.scalar_type() == at::kFloat &&
+                    acc.numel() == S * HQ * num_splits * head_dim && m.is_cuda() && m.is_contiguous() &&
+                    m.scalar_type() == at::kFloat && m.numel() == S * HQ * num_splits && l.is_cuda() &&
+                    l.is_contiguous() && l.scalar_type() == at::kFloat && l.numel() == S * HQ * num_splits,
+                "out must be float32 GPU tensors (S, H_Q, splits, D), (S, H_Q, splits), (S, H_Q, splits)");
+    } else {
+        acc = at::empty({S, HQ, num_splits, head_dim}, q_rot.options().dtype(at::kFloat));
+        m = at::empty({S, HQ, num_splits}, q_rot.options().dtype(at::kFloat));
+        l = at::empty({S, HQ, num_splits}, q_rot.options().dtype(at::kFloat));
+    }
+    const int st = fq_paged_tq4_decode(
+        q_rot.data_ptr(), kv_cache.data_ptr<uint8_t>(), block_table.data_ptr<int32_t>(), seq_lens.data_ptr<int32_t>(),
+        centroids_k.data_ptr<float>(), centroids_v.data_ptr<float>(), acc.data_ptr<float>(), m.data_ptr<float>(),
+        l.data_ptr<float>(), int(S), int(HQ), int(num_kv_heads), int(head_dim), int(block_size),
+        int(block_table.size(1)), kv_cache.size(0), float(sm_scale),
+        fqbind::dtype_code(q_rot.scalar_type(), "paged_tq4_decode_partials"), int(num_splits),
+        fqbind::current_stream(q_rot));
+    fqbind::raise_on_error(st, "paged_tq4_decode_partials");
+    return {acc, m, l};
+}
+
+at::Tensor split_k_reduce(const at::Tensor& acc, const at::Tensor& m, const at::Tensor& l,
+                          const std::optional<at::Tensor>& rotation, at::ScalarType dtype) {
+    fqbind::require_gpu(acc, "partial_acc");
+    require(acc.dim() == 4 && acc.is_contiguous() && acc.scalar_type() == at::kFloat && m.is_contiguous() &&
+                l.is_contiguous() && m.is_cuda() && l.is_cuda() && m.scalar_type() == at::kFloat &&
+                l.scalar_type() == at::kFloat && m.numel() == acc.numel() / acc.size(3) && l.numel() == m.numel(),
+            "partials must be contiguous float32 GPU tensors (S, H_Q, splits, D), (S, H_Q, splits) x2");
+    c10::DeviceGuard guard(acc.device());
+    at::Tensor rot;
+    if (rotation.has_value()) rot = rotation->to(acc.device()).contiguous();
+    at::Tensor out = at::empty({acc.size(0), acc.size(1), acc.size(3)}, acc.options().dtype(dtype));
+    const int st = fq_split_k_reduce(acc.data_ptr<float>(), m.data_ptr<float>(), l.data_ptr<float>(),
+                                     rot.defined() ? rot.data_ptr<float>() : nullptr, out.data_ptr(), int(acc.size(0)),
+                                     int(acc.size(1)), int(acc.size(3)), fqbind::dtype_code(dtype, "split_k_reduce"),
+                                     int(acc.size(2)), fqbind::current_stream(acc));
+    fqbind::raise_on_error(st, "split_k_reduce");
+    return out;
+}
+
 }  // namespace
 
 void bind_kernels(py::module_& m) {
@@ -179,6 +264,15 @@ void bind_kernels(py::module_& m) {
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),
           py::arg("out") = py::none(), py::arg("num_splits") = 0,
           "Alias of split_k_paged_decode.");
+    m.def("rotate_query", &rotate_query, py::arg("q"), py::arg("rotation"),
+          "q_rot = (q @ rotation.T) rounded to q's dtype.");
+    m.def("paged_tq4_decode_partials", &paged_tq4_decode_partials, py::arg("q_rot"), py::arg("kv_cache"),
+          py::arg("block_table"), py::arg("seq_lens"), py::arg("centroids_k"), py::arg("centroids_v"),
+          py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale"),
+          py::arg("num_splits"), py::arg("out") = py::none(),
+          "Split partials (acc, m, l) of the paged decode for a pre-rotated query.");
+    m.def("split_k_reduce", &split_k_reduce, py::arg("partial_acc"), py::arg("partial_m"), py::arg("partial_l"),
+          py::arg("rotation"), py::arg("dtype"), "Log-sum-exp combine of split partials, optional post-rotation.");
     m.def("paged_decode_auto_splits", &fq_paged_decode_auto_splits, py::arg("num_seqs"), py::arg("num_kv_heads"),
           py::arg("block_size"), py::arg("max_blocks_per_seq"));
 }

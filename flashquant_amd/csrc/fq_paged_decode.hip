@@ -505,13 +505,6 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
     }
 }
 
-struct DecodeLaunch {
-    const void* q; const uint8_t* cache; const int32_t* bt; const int32_t* lens;
-    const float* ck; const float* cv; const float* R; void* out;
-    int S, H_Q, H_KV, D, BS, max_blocks; int64_t num_blocks; float sm_scale; int NS;
-    uint8_t* ws; hipStream_t stream;
-};
-
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct WorkspaceLayout {
@@ -529,48 +522,65 @@ inline WorkspaceLayout workspace_layout(int S, int H_Q, int D, int NS) {
 }
 
 template <int D, int DT>
-int launch_decode(const DecodeLaunch& a) {
-    const WorkspaceLayout w = workspace_layout(a.S, a.H_Q, D, a.NS);
-    const int G = a.H_Q / a.H_KV;
-    const void* q_rot = a.q;
-    if (a.R) {
-        uint16_t* qr = reinterpret_cast<uint16_t*>(a.ws + w.qrot);
-        hipLaunchKernelGGL((rotate_q_kernel<D, DT>), dim3(a.S, (a.H_Q + 7) / 8), dim3(256), 0, a.stream,
-                           reinterpret_cast<const uint16_t*>(a.q), a.R, qr, a.H_Q);
-        q_rot = qr;
-    }
-    DecodeParams p;
-    p.q_rot = q_rot; p.cache = a.cache; p.block_table = a.bt; p.seq_lens = a.lens;
-    p.centroids_k = a.ck; p.centroids_v = a.cv;
-    p.part_acc = reinterpret_cast<float*>(a.ws + w.acc);
-    p.part_m = reinterpret_cast<float*>(a.ws + w.m);
-    p.part_l = reinterpret_cast<float*>(a.ws + w.l);
-    p.H_Q = a.H_Q; p.H_KV = a.H_KV; p.G = G; p.max_blocks = a.max_blocks;
-    p.num_blocks = int(a.num_blocks); p.num_splits = a.NS;
-    p.two_tables = a.ck != a.cv ? 1 : 0;
-    p.scale_log2e = a.sm_scale * kLog2e;
-
-    const int waves = a.H_KV < 8 ? a.H_KV : 8;
-    const dim3 grid(a.NS, a.S, (a.H_KV + waves - 1) / waves), block(64 * waves);
+int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
+    const int waves = p.H_KV < 8 ? p.H_KV : 8;
+    const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
     const size_t lds = size_t(p.two_tables ? 2 : 1) * kLutWords * sizeof(uint32_t);
 #define FQ_DECODE_GP(BSL, GPV) \
-    hipLaunchKernelGGL((paged_decode_kernel<D, BSL, GPV, DT>), grid, block, lds, a.stream, p)
-#define FQ_DECODE_BS(BSL)                       \
-    do {                                        \
-        if (G <= 4) FQ_DECODE_GP(BSL, 4);       \
-        else if (G <= 8) FQ_DECODE_GP(BSL, 8);  \
-        else FQ_DECODE_GP(BSL, 16);             \
+    hipLaunchKernelGGL((paged_decode_kernel<D, BSL, GPV, DT>), grid, block, lds, stream, p)
+#define FQ_DECODE_BS(BSL)                        \
+    do {                                         \
+        if (p.G <= 4) FQ_DECODE_GP(BSL, 4);      \
+        else if (p.G <= 8) FQ_DECODE_GP(BSL, 8); \
+        else FQ_DECODE_GP(BSL, 16);              \
     } while (0)
-    switch (a.BS) {
+    switch (BS) {
         case 8: FQ_DECODE_BS(3); break;
         case 16: FQ_DECODE_BS(4); break;
         default: FQ_DECODE_BS(5); break;
     }
 #undef FQ_DECODE_BS
 #undef FQ_DECODE_GP
-    hipLaunchKernelGGL((reduce_rotate_kernel<D, DT>), dim3(a.S, (a.H_Q + 7) / 8), dim3(256), 0, a.stream,
-                       p.part_acc, p.part_m, p.part_l, a.R, reinterpret_cast<uint16_t*>(a.out), a.H_Q, a.NS);
     return fq_host::check_launch();
+}
+
+template <int DT>
+int launch_rotate(const void* q, const float* R, void* q_rot, int S, int H_Q, int D, hipStream_t stream) {
+    const dim3 grid(S, (H_Q + 7) / 8), block(256);
+    const uint16_t* src = reinterpret_cast<const uint16_t*>(q);
+    uint16_t* dst = reinterpret_cast<uint16_t*>(q_rot);
+    switch (D) {
+        case 64: hipLaunchKernelGGL((rotate_q_kernel<64, DT>), grid, block, 0, stream, src, R, dst, H_Q); break;
+        case 128: hipLaunchKernelGGL((rotate_q_kernel<128, DT>), grid, block, 0, stream, src, R, dst, H_Q); break;
+        default: hipLaunchKernelGGL((rotate_q_kernel<256, DT>), grid, block, 0, stream, src, R, dst, H_Q); break;
+    }
+    return fq_host::check_launch();
+}
+
+template <int DT>
+int launch_reduce(const float* acc, const float* m, const float* l, const float* R, void* out, int S, int H_Q,
+                  int D, int NS, hipStream_t stream) {
+    const dim3 grid(S, (H_Q + 7) / 8), block(256);
+    uint16_t* dst = reinterpret_cast<uint16_t*>(out);
+    switch (D) {
+        case 64: hipLaunchKernelGGL((reduce_rotate_kernel<64, DT>), grid, block, 0, stream, acc, m, l, R, dst, H_Q, NS); break;
+        case 128: hipLaunchKernelGGL((reduce_rotate_kernel<128, DT>), grid, block, 0, stream, acc, m, l, R, dst, H_Q, NS); break;
+        default: hipLaunchKernelGGL((reduce_rotate_kernel<256, DT>), grid, block, 0, stream, acc, m, l, R, dst, H_Q, NS); break;
+    }
+    return fq_host::check_launch();
+}
+
+inline int check_decode_shape(int num_seqs, int H_Q, int H_KV, int D, int block_size, int max_blocks_per_seq,
+                              int64_t num_blocks, int dtype, int num_splits) {
+    if (num_seqs < 0 || H_Q <= 0 || H_KV <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0 || num_splits < 0)
+        return FQ_ERR_BAD_SHAPE;
+    if (H_Q % H_KV != 0 || H_Q / H_KV > 16) return FQ_ERR_BAD_SHAPE;
+    if (num_blocks > 0x7fffffffLL || num_seqs > 65535 || (H_KV + 7) / 8 > 65535 || num_splits > 65535)
+        return FQ_ERR_BAD_SHAPE;
+    if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
+    if (block_size != 8 && block_size != 16 && block_size != 32) return FQ_ERR_UNSUPPORTED_BLOCK;
+    if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
+    return FQ_OK;
 }
 
 }  // namespace fq
@@ -599,37 +609,50 @@ extern "C" size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_K
     return fq::workspace_layout(num_seqs, H_Q, D, num_splits).total;
 }
 
-extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
-                                       const int32_t* seq_lens, const float* centroids_k,
-                                       const float* centroids_v, const float* rotation, void* out,
-                                       int num_seqs, int H_Q, int H_KV, int D, int block_size,
-                                       int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype,
-                                       int num_splits, void* workspace, size_t workspace_bytes, void* stream) {
+extern "C" int fq_rotate_query(const void* q, const float* rotation, void* q_rot, int64_t num_seqs, int H_Q,
+                               int D, int dtype, void* stream) {
     using namespace fq;
-    if (num_seqs < 0 || H_Q <= 0 || H_KV <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0 || num_splits < 0)
-        return FQ_ERR_BAD_SHAPE;
-    if (H_Q % H_KV != 0 || H_Q / H_KV > 16) return FQ_ERR_BAD_SHAPE;
-    if (num_blocks > 0x7fffffffLL || num_seqs > 65535 || (H_KV + 7) / 8 > 65535) return FQ_ERR_BAD_SHAPE;
+    if (num_seqs < 0 || num_seqs > 65535 || H_Q <= 0) return FQ_ERR_BAD_SHAPE;
     if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
-    if (block_size != 8 && block_size != 16 && block_size != 32) return FQ_ERR_UNSUPPORTED_BLOCK;
     if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
     if (num_seqs == 0) return FQ_OK;
-    if (!q || !kv_cache || !block_table || !seq_lens || !centroids_k || !centroids_v || !out)
-        return FQ_ERR_NULL_POINTER;
-    if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16) || !fq_host::aligned(kv_cache, 16) ||
-        (rotation && !fq_host::aligned(rotation, 16)))
+    if (!q || !rotation || !q_rot) return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(rotation, 16) || !fq_host::aligned(q, 2) || !fq_host::aligned(q_rot, 2))
         return FQ_ERR_MISALIGNED;
-    if (num_splits == 0) num_splits = fq_paged_decode_auto_splits(num_seqs, H_KV, block_size, max_blocks_per_seq);
-    if (num_splits > 65535) return FQ_ERR_BAD_SHAPE;
-    const size_t need = workspace_layout(num_seqs, H_Q, D, num_splits).total;
-    if (!workspace || workspace_bytes < need) return FQ_ERR_WORKSPACE;
-    if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == FQ_F16 ? launch_rotate<FQ_F16>(q, rotation, q_rot, int(num_seqs), H_Q, D, s)
+                           : launch_rotate<FQ_BF16>(q, rotation, q_rot, int(num_seqs), H_Q, D, s);
+}
 
-    DecodeLaunch a{q, kv_cache, block_table, seq_lens, centroids_k, centroids_v, rotation, out,
-                   num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, num_splits,
-                   static_cast<uint8_t*>(workspace), static_cast<hipStream_t>(stream)};
-#define FQ_DECODE_D(DD)                                                                       \
-    case DD: return dtype == FQ_F16 ? launch_decode<DD, FQ_F16>(a) : launch_decode<DD, FQ_BF16>(a);
+extern "C" int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache, const int32_t* block_table,
+                                   const int32_t* seq_lens, const float* centroids_k, const float* centroids_v,
+                                   float* partial_acc, float* partial_m, float* partial_l, int num_seqs, int H_Q,
+                                   int H_KV, int D, int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                                   float sm_scale, int dtype, int num_splits, void* stream) {
+    using namespace fq;
+    const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
+                                       num_splits);
+    if (bad != FQ_OK) return bad;
+    if (num_splits < 1) return FQ_ERR_BAD_SHAPE;
+    if (num_seqs == 0) return FQ_OK;
+    if (!q_rot || !kv_cache || !block_table || !seq_lens || !centroids_k || !centroids_v || !partial_acc ||
+        !partial_m || !partial_l)
+        return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(q_rot, 16) || !fq_host::aligned(kv_cache, 16) || !fq_host::aligned(partial_acc, 16))
+        return FQ_ERR_MISALIGNED;
+    DecodeParams p;
+    p.q_rot = q_rot; p.cache = kv_cache; p.block_table = block_table; p.seq_lens = seq_lens;
+    p.centroids_k = centroids_k; p.centroids_v = centroids_v;
+    p.part_acc = partial_acc; p.part_m = partial_m; p.part_l = partial_l;
+    p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.max_blocks = max_blocks_per_seq;
+    p.num_blocks = int(num_blocks); p.num_splits = num_splits;
+    p.two_tables = centroids_k != centroids_v ? 1 : 0;
+    p.scale_log2e = sm_scale * kLog2e;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define FQ_DECODE_D(DD)                                                                 \
+    case DD:                                                                            \
+        return dtype == FQ_F16 ? launch_partials<DD, FQ_F16>(p, num_seqs, block_size, s) \
+                               : launch_partials<DD, FQ_BF16>(p, num_seqs, block_size, s);
     switch (D) {
         FQ_DECODE_D(64)
         FQ_DECODE_D(128)
@@ -637,4 +660,53 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
         default: return FQ_ERR_UNSUPPORTED_DIM;
     }
 #undef FQ_DECODE_D
+}
+
+extern "C" int fq_split_k_reduce(const float* partial_acc, const float* partial_m, const float* partial_l,
+                                 const float* rotation, void* out, int num_seqs, int H_Q, int D, int dtype,
+                                 int num_splits, void* stream) {
+    using namespace fq;
+    if (num_seqs < 0 || num_seqs > 65535 || H_Q <= 0 || num_splits < 1) return FQ_ERR_BAD_SHAPE;
+    if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
+    if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
+    if (num_seqs == 0) return FQ_OK;
+    if (!partial_acc || !partial_m || !partial_l || !out) return FQ_ERR_NULL_POINTER;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == FQ_F16
+               ? launch_reduce<FQ_F16>(partial_acc, partial_m, partial_l, rotation, out, num_seqs, H_Q, D, num_splits, s)
+               : launch_reduce<FQ_BF16>(partial_acc, partial_m, partial_l, rotation, out, num_seqs, H_Q, D, num_splits, s);
+}
+
+extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
+                                       const int32_t* seq_lens, const float* centroids_k,
+                                       const float* centroids_v, const float* rotation, void* out,
+                                       int num_seqs, int H_Q, int H_KV, int D, int block_size,
+                                       int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype,
+                                       int num_splits, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace fq;
+    const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
+                                       num_splits);
+    if (bad != FQ_OK) return bad;
+    if (num_seqs == 0) return FQ_OK;
+    if (!q || !out) return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16)) return FQ_ERR_MISALIGNED;
+    if (num_splits == 0) num_splits = fq_paged_decode_auto_splits(num_seqs, H_KV, block_size, max_blocks_per_seq);
+    const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_splits);
+    if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
+    if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    float* acc = reinterpret_cast<float*>(ws + w.acc);
+    float* m = reinterpret_cast<float*>(ws + w.m);
+    float* l = reinterpret_cast<float*>(ws + w.l);
+    const void* q_rot = q;
+    if (rotation) {
+        const int st = fq_rotate_query(q, rotation, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
+        if (st != FQ_OK) return st;
+        q_rot = ws + w.qrot;
+    }
+    int st = fq_paged_tq4_decode(q_rot, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m, l,
+                                 num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
+                                 num_splits, stream);
+    if (st != FQ_OK) return st;
+    return fq_split_k_reduce(acc, m, l, rotation, out, num_seqs, H_Q, D, dtype, num_splits, stream);
 }

@@ -118,6 +118,38 @@ int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
                             void* workspace, size_t workspace_bytes,
                             void* stream);
 
+/*
+ * The three stages of fq_split_k_paged_decode as separate launches, for callers
+ * that hold the rotated query or want the partials (the reference exposes its
+ * decode at this level: paged_tq4_decode_cuda, csrc/cuda/paged_decode.cu:346-368,
+ * and split_k_reduce_cuda, csrc/cuda/split_k_reduce.cu:145-154).
+ *
+ * fq_rotate_query:     q_rot = (q @ rotation.T) rounded to dtype
+ *                      (src/flashquant/kernels/paged_decode.py:113); q, q_rot (num_seqs, H_Q, D).
+ * fq_paged_tq4_decode: q_rot pre-rotated; writes un-normalised float32 partials
+ *                      partial_acc (num_seqs, H_Q, num_splits, D) and the base-2 running
+ *                      maximum / denominator partial_m, partial_l (num_seqs, H_Q, num_splits);
+ *                      an empty split has m = -inf.  num_splits >= 1.
+ * fq_split_k_reduce:   out = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*), rounded to
+ *                      dtype; if rotation is not NULL the rounded value is multiplied by
+ *                      rotation in float32 and rounded again (paged_decode.py:123).
+ */
+int fq_rotate_query(const void* q, const float* rotation, void* q_rot,
+                    int64_t num_seqs, int H_Q, int D, int dtype, void* stream);
+
+int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache,
+                        const int32_t* block_table, const int32_t* seq_lens,
+                        const float* centroids_k, const float* centroids_v,
+                        float* partial_acc, float* partial_m, float* partial_l,
+                        int num_seqs, int H_Q, int H_KV, int D,
+                        int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                        float sm_scale, int dtype, int num_splits, void* stream);
+
+int fq_split_k_reduce(const float* partial_acc, const float* partial_m,
+                      const float* partial_l, const float* rotation, void* out,
+                      int num_seqs, int H_Q, int D, int dtype, int num_splits,
+                      void* stream);
+
 /* Number of splits fq_split_k_paged_decode uses when num_splits == 0
  * (counterpart of paged_tq4_decode_num_splits, csrc/cuda/paged_decode.cu:424-426,
  * which is a constant 4 there). */
