@@ -72,7 +72,32 @@ struct DecodeParams {
 
 __device__ __forceinline__ uint32_t byte_of(uint32_t w, int b) { return (w >> (8 * b)) & 0xffu; }
 
-template <int D, int BSL, int GP, int DT>
+// Cross-lane helpers that stay in the VALU (no LDS round trip).
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+// max over lanes l and l ^ 16 (rows of 16 lanes swapped pairwise)
+__device__ __forceinline__ float max_xor16(float v) {
+    const uint32_t u = float_to_bits(v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return __builtin_fmaxf(bits_to_float(r[0]), bits_to_float(r[1]));
+}
+// max over lanes l and l ^ 32
+__device__ __forceinline__ float max_xor32(float v) {
+    const uint32_t u = float_to_bits(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_fmaxf(bits_to_float(r[0]), bits_to_float(r[1]));
+}
+// max over all lanes that share lane % GP
+template <int GP>
+__device__ __forceinline__ float max_same_head(float v) {
+    if (GP <= 4) v = __builtin_fmaxf(v, dpp_mov<0x124>(v));   // row_ror:4
+    if (GP <= 8) v = __builtin_fmaxf(v, dpp_mov<0x128>(v));   // row_ror:8
+    return max_xor32(max_xor16(v));
+}
+
+template <int D, int BSL, int GP, int DT, int PVR>
 __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p) {
     constexpr int BS = 1 << BSL;
     constexpr int KS = D / 32;            // k-steps of the score product
@@ -81,7 +106,6 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     constexpr int VW = DPL > 8 ? 2 : 1;   // V dwords per lane per token
     constexpr int NB = 16 / GP;           // block classes
     constexpr int NC = 4 / NB;            // kept blocks per lane per tile
-    constexpr int PAGES = 64 / BS;        // pages per tile
     constexpr int ROW_HALF = D / 2;
 
     extern __shared__ uint32_t lut[];
@@ -178,43 +202,63 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 
     const uint8_t* cache = p.cache;
     const int max_page = p.num_blocks - 1;
+    const int64_t page_bytes = int64_t(BS) * row_bytes;
 
-    auto load_tile = [&](int t0, Tile& t) {
-        // the pages of this tile (wave-uniform)
-        int pg[PAGES];
-        const int p0 = t0 >> BSL;
+    // Lane-constant byte offsets from the base of a block's page: the K operand
+    // reads row n (quarter g of the head's index bytes), the V operand and the
+    // norms read rows 4g + 0..3.  With 8-token pages a 16-token block spans two
+    // pages and rows 8..15 live in the second one (k_hi / r_hi).
+    constexpr bool SMALL_PAGES = BSL == 3;
+    const bool k_hi = SMALL_PAGES && (n & 8);
+    const bool r_hi = SMALL_PAGES && (g & 2);
+    const uint32_t k_off = uint32_t((SMALL_PAGES ? (n & 7) : n) * row_bytes + h * ROW_HALF + g * (D / 8));
+    uint32_t v_off[4], n_off[4];
 #pragma unroll
-        for (int i = 0; i < PAGES; ++i) {
-            int idx = p0 + i;
-            idx = idx > last_page_idx ? last_page_idx : idx;
-            int v = bt[idx];
-            v = v < 0 ? 0 : (v > max_page ? max_page : v);
-            pg[i] = v;
+    for (int i = 0; i < 4; ++i) {
+        const int r = SMALL_PAGES ? ((4 * g + i) & 7) : 4 * g + i;
+        v_off[i] = uint32_t(r * row_bytes + v_idx_off + n * (DPL / 2));
+        n_off[i] = uint32_t(r * row_bytes + k_norm_off);
+    }
+    const uint32_t vn_delta = uint32_t(v_norm_off - k_norm_off);
+
+    // Page ids of this split, fetched once: lane i of register r holds the page of
+    // split-local page index 64 r + i (clamped to the sequence's last page and to the
+    // cache size, so every address formed from them stays inside the cache).  A tile
+    // then gets its pages with v_readlane, with no memory access on its critical path.
+    int pv[PVR];
+    const int split_p0 = begin >> BSL;
+#pragma unroll
+    for (int r = 0; r < PVR; ++r) {
+        int idx = split_p0 + 64 * r + lane;
+        idx = idx > last_page_idx ? last_page_idx : idx;
+        int pg = bt[idx];
+        pv[r] = pg < 0 ? 0 : (pg > max_page ? max_page : pg);
+    }
+    auto page_id = [&](int rel) -> int {   // rel: split-local page index, wave-uniform
+        int v = __builtin_amdgcn_readlane(pv[0], rel & 63);
+#pragma unroll
+        for (int r = 1; r < PVR; ++r) {
+            const int vr = __builtin_amdgcn_readlane(pv[r], rel & 63);
+            v = (rel >> 6) == r ? vr : v;
         }
-        // byte offset of the row of tile-local token u (0..63); tokens at or past
-        // `end` read the last valid token of the split instead
-        auto row_off = [&](int blk, int r) -> int64_t {
-            int u = 16 * blk + r;
-            const int lim = end - 1 - t0;
-            int page;
-            if (u > lim) {
-                u = lim;
-                // u is now a run-time value: pick its page by comparison
-                page = pg[0];
-#pragma unroll
-                for (int i = 1; i < PAGES; ++i) page = (u >> BSL) >= i ? pg[i] : page;
-            } else if (BSL == 4) {
-                page = pg[blk];
-            } else if (BSL == 5) {
-                page = pg[blk >> 1];
-            } else {
-                page = (r & 8) ? pg[2 * blk + 1] : pg[2 * blk];
-            }
-            return (int64_t(page) * BS + ((t0 + u) & (BS - 1))) * row_bytes;
-        };
+        return v;
+    };
+
+    // Loads one tile.  Tokens at or past `end` are not clamped: their values are
+    // masked later.
+    auto load_tile = [&](int t0, Tile& t) {
+        const uint8_t* lo[4];
+        const uint8_t* hi[4];
+        const int p0 = (t0 >> BSL) - split_p0;
 #pragma unroll
         for (int blk = 0; blk < 4; ++blk) {
-            const uint8_t* src = cache + row_off(blk, n) + h * ROW_HALF + g * (D / 8);
+            const int rel = BSL == 4 ? blk : (BSL == 5 ? (blk >> 1) : 2 * blk);
+            lo[blk] = cache + int64_t(page_id(p0 + rel)) * page_bytes + ((BSL == 5 && (blk & 1)) ? 16 * row_bytes : 0);
+            hi[blk] = SMALL_PAGES ? cache + int64_t(page_id(p0 + rel + 1)) * page_bytes : lo[blk];
+        }
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            const uint8_t* src = (k_hi ? hi[blk] : lo[blk]) + k_off;
             if (KW == 4) {
                 const uint4v w = *reinterpret_cast<const uint4v*>(src);
                 t.k[blk][0] = w.x; t.k[blk][1] = w.y; t.k[blk][2] = w.z; t.k[blk][3] = w.w;
@@ -234,7 +278,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
         for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const uint8_t* src = cache + row_off(2 * ks + j / 4, 4 * g + j % 4) + v_idx_off + n * (DPL / 2);
+                const int blk = 2 * ks + j / 4;
+                const uint8_t* src = (r_hi ? hi[blk] : lo[blk]) + v_off[j % 4];
                 if (DPL == 4) {
                     t.v[ks][j][0] = *reinterpret_cast<const uint16_t*>(src);
                 } else if (DPL == 8) {
@@ -248,19 +293,13 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
         }
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
+            const uint8_t* base = r_hi ? hi[c * NB] : lo[c * NB];
+#pragma unroll
+            for (int bc = 1; bc < NB; ++bc) base = bc_lane == bc ? (r_hi ? hi[c * NB + bc] : lo[c * NB + bc]) : base;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                // block c*NB + bc_lane is a run-time block: go through the generic path
-                const int blk = c * NB + bc_lane;
-                int u = 16 * blk + 4 * g + i;
-                const int lim = end - 1 - t0;
-                u = u > lim ? lim : u;
-                int page = pg[0];
-#pragma unroll
-                for (int q = 1; q < PAGES; ++q) page = (u >> BSL) >= q ? pg[q] : page;
-                const uint8_t* row = cache + (int64_t(page) * BS + ((t0 + u) & (BS - 1))) * row_bytes;
-                t.kn[c][i] = *reinterpret_cast<const float*>(row + k_norm_off);
-                t.vn[c][i] = *reinterpret_cast<const float*>(row + v_norm_off);
+                t.kn[c][i] = *reinterpret_cast<const float*>(base + n_off[i]);
+                t.vn[c][i] = *reinterpret_cast<const float*>(base + n_off[i] + vn_delta);
             }
         }
     };
@@ -272,50 +311,87 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     float M = -__builtin_inff();
     float lsum = 0.0f;
 
-    Tile cur;
-    load_tile(begin, cur);
+    // One operand (8 fp16 values) from 4 packed bytes: 4 conflict-free LDS reads.
+    auto lookup4 = [&](const uint32_t* tab, uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) -> uint4v {
+        uint4v r;
+        r.x = tab[b0 * kLutCopies];
+        r.y = tab[b1 * kLutCopies];
+        r.z = tab[b2 * kLutCopies];
+        r.w = tab[b3 * kLutCopies];
+        return r;
+    };
+    constexpr int VG = DPL / 4;      // groups of four coordinate blocks per k-step of P.V
 
-    for (int t0 = begin; t0 < end; t0 += 64) {
-        Tile nxt;
-        const bool more = t0 + 64 < end;
-        if (more) load_tile(t0 + 64, nxt);
-
-        // ---- scores --------------------------------------------------------------
-        float4v sacc[4];
-#pragma unroll
-        for (int blk = 0; blk < 4; ++blk) {
-            sacc[blk] = float4v{0.f, 0.f, 0.f, 0.f};
+    auto compute_tile = [&](int t0, const Tile& cur) {
+        // The LDS lookups of one group of operands are issued before the MFMAs of the
+        // previous group, so that the LDS latency overlaps matrix work; the scheduling
+        // fences keep the compiler from serialising lookup -> wait -> MFMA again.
+        uint4v ka[2][KS];
+        auto k_group = [&](int blk, uint4v (&dst)[KS]) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const uint32_t w = cur.k[blk][ks];
-                uint4v a;
-                a.x = lut_k[byte_of(w, 0) * kLutCopies];
-                a.y = lut_k[byte_of(w, 1) * kLutCopies];
-                a.z = lut_k[byte_of(w, 2) * kLutCopies];
-                a.w = lut_k[byte_of(w, 3) * kLutCopies];
-                sacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), qh[ks], sacc[blk], 0, 0, 0);
+                dst[ks] = lookup4(lut_k, byte_of(w, 0), byte_of(w, 1), byte_of(w, 2), byte_of(w, 3));
             }
+        };
+        // nibble transposes of the V token pairs (all of them: 2 k-steps x 4 pairs)
+        uint32_t X[2][4][VW], Y[2][4][VW];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int jp = 0; jp < 4; ++jp)
+#pragma unroll
+                for (int wv = 0; wv < VW; ++wv) {
+                    const uint32_t A = cur.v[ks][2 * jp][wv], B = cur.v[ks][2 * jp + 1][wv];
+                    X[ks][jp][wv] = (A & 0xF0F0F0F0u) | ((B >> 4) & 0x0F0F0F0Fu);
+                    Y[ks][jp][wv] = ((A << 4) & 0xF0F0F0F0u) | (B & 0x0F0F0F0Fu);
+                }
+        uint4v vb[2][4];
+        auto v_group = [&](int grp, uint4v (&dst)[4]) {   // grp = ks * VG + quarter
+            const int ks = grp / VG, q4 = grp % VG;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int db = 4 * q4 + e, bi = db / 2;
+                const uint32_t (&src)[4][VW] = (db & 1) ? Y[ks] : X[ks];
+                dst[e] = lookup4(lut_v, byte_of(src[0][bi / 4], bi % 4), byte_of(src[1][bi / 4], bi % 4),
+                                 byte_of(src[2][bi / 4], bi % 4), byte_of(src[3][bi / 4], bi % 4));
+            }
+        };
+
+        // ---- scores --------------------------------------------------------------
+        float s_[NC][4];
+        k_group(0, ka[0]);
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            if (blk < 3) k_group(blk + 1, ka[(blk + 1) & 1]);
+            else v_group(0, vb[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            float4v acc = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ka[blk & 1][ks]), qh[ks], acc, 0, 0, 0);
+            const int c = blk / NB, bc = blk % NB;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_[c][i] = (bc == 0 || bc_lane == bc) ? acc[i] : s_[c][i];
+            __builtin_amdgcn_sched_barrier(0);
         }
+
         float a_[NC][4], rv[NC][4];
         float tmax = -__builtin_inff();
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float s = sacc[c * NB][i];
-#pragma unroll
-                for (int bc = 1; bc < NB; ++bc) s = bc_lane == bc ? sacc[c * NB + bc][i] : s;
-                const float vn = __builtin_fmaxf(cur.vn[c][i], kTinyNorm);
-                rv[c][i] = __builtin_amdgcn_rcpf(vn);
-                float a = __builtin_fmaf(s * cur.kn[c][i], qscale, __builtin_amdgcn_logf(vn));
                 const int tok = t0 + 16 * (c * NB + bc_lane) + 4 * g + i;
-                a = tok < end ? a : -__builtin_inff();
-                a_[c][i] = a;
-                tmax = __builtin_fmaxf(tmax, a);
+                const bool live = tok < end;
+                const float vn = __builtin_fmaxf(cur.vn[c][i], kTinyNorm);
+                rv[c][i] = live ? __builtin_amdgcn_rcpf(vn) : 0.0f;
+                const float a = __builtin_fmaf(s_[c][i] * cur.kn[c][i], qscale, __builtin_amdgcn_logf(vn));
+                a_[c][i] = live ? a : -__builtin_inff();
+                tmax = __builtin_fmaxf(tmax, a_[c][i]);
             }
         }
-#pragma unroll
-        for (int mask = GP; mask < 64; mask <<= 1) tmax = __builtin_fmaxf(tmax, xor_shuffle(tmax, mask));
+        tmax = max_same_head<GP>(tmax);
         const float Mnew = __builtin_fmaxf(M, tmax);
         const float Ms = Mnew == -__builtin_inff() ? 0.0f : Mnew;
         const float alpha = __builtin_amdgcn_exp2f(M - Ms);
@@ -337,8 +413,16 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
         // ---- rescale the accumulators when a maximum moved --------------------------
         if (__any(alpha != 1.0f)) {
             float ar[4];
+            if (GP == 4) {
+                // row 4g + i belongs to head i, held by the lane at position i of this lane's quad
+                ar[0] = dpp_mov<0x00>(alpha);
+                ar[1] = dpp_mov<0x55>(alpha);
+                ar[2] = dpp_mov<0xAA>(alpha);
+                ar[3] = dpp_mov<0xFF>(alpha);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * g + i, kWave);
+                for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * g + i, kWave);
+            }
 #pragma unroll
             for (int db = 0; db < DPL; ++db)
 #pragma unroll
@@ -360,34 +444,44 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             }
         }
 
-        // ---- O += P . V ---------------------------------------------------------------
+        // ---- O += P . V, lookups of the next group in flight during the MFMAs ------------
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            uint32_t X[4][VW], Y[4][VW];
+        for (int grp = 0; grp < 2 * VG; ++grp) {
+            if (grp + 1 < 2 * VG) v_group(grp + 1, vb[(grp + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            const int ks = grp / VG, q4 = grp % VG;
 #pragma unroll
-            for (int jp = 0; jp < 4; ++jp) {
-#pragma unroll
-                for (int wv = 0; wv < VW; ++wv) {
-                    const uint32_t A = cur.v[ks][2 * jp][wv], B = cur.v[ks][2 * jp + 1][wv];
-                    X[jp][wv] = (A & 0xF0F0F0F0u) | ((B >> 4) & 0x0F0F0F0Fu);
-                    Y[jp][wv] = ((A << 4) & 0xF0F0F0F0u) | (B & 0x0F0F0F0Fu);
-                }
-            }
-#pragma unroll
-            for (int db = 0; db < DPL; ++db) {
-                const int bi = db / 2;
-                uint4v b;
-                uint32_t src[4];
-#pragma unroll
-                for (int jp = 0; jp < 4; ++jp) src[jp] = (db & 1) ? Y[jp][bi / 4] : X[jp][bi / 4];
-                b.x = lut_v[byte_of(src[0], bi % 4) * kLutCopies];
-                b.y = lut_v[byte_of(src[1], bi % 4) * kLutCopies];
-                b.z = lut_v[byte_of(src[2], bi % 4) * kLutCopies];
-                b.w = lut_v[byte_of(src[3], bi % 4) * kLutCopies];
-                O[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[ks], __builtin_bit_cast(half8, b), O[db], 0, 0, 0);
-            }
+            for (int e = 0; e < 4; ++e)
+                O[4 * q4 + e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[ks], __builtin_bit_cast(half8, vb[grp & 1][e]),
+                                                                      O[4 * q4 + e], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (more) cur = nxt;
+    };
+
+    // ---- tiles of the split, two register images in ping-pong ------------------------
+    // The prefetch of the next tile is unconditional (past the last tile it reloads
+    // the last one): a branch around it would make the compiler wait for every
+    // outstanding load where the paths merge, which serialises load and compute.
+    // The workgroup barrier keeps the wavefronts (one per KV head) on the same tile,
+    // so that the halves of a cache line that two heads share are asked for together.
+    {
+        Tile ta, tb;
+        int t0 = begin;
+        const int last_t0 = begin + ((end - begin - 1) & ~63);
+        load_tile(t0, ta);
+        while (true) {
+            __builtin_amdgcn_s_barrier();
+            load_tile(t0 + 64 < last_t0 ? t0 + 64 : last_t0, tb);
+            compute_tile(t0, ta);
+            t0 += 64;
+            if (t0 >= end) break;
+            __builtin_amdgcn_s_barrier();
+            load_tile(t0 + 64 < last_t0 ? t0 + 64 : last_t0, ta);
+            compute_tile(t0, tb);
+            t0 += 64;
+            if (t0 >= end) break;
+        }
     }
 
     // ---- publish the partial of this split --------------------------------------------
@@ -526,8 +620,15 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
     const int waves = p.H_KV < 8 ? p.H_KV : 8;
     const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
     const size_t lds = size_t(p.two_tables ? 2 : 1) * kLutWords * sizeof(uint32_t);
-#define FQ_DECODE_GP(BSL, GPV) \
-    hipLaunchKernelGGL((paged_decode_kernel<D, BSL, GPV, DT>), grid, block, lds, stream, p)
+    // pages a split can span: its tokens are ceil(max_ctx / splits) rounded up to a tile
+    const int64_t max_ctx = int64_t(p.max_blocks) * BS;
+    const int64_t chunk = (((max_ctx + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
+    const bool wide = chunk / BS > 64;   // begin is a multiple of 64 tokens, hence page aligned
+#define FQ_DECODE_GP(BSL, GPV)                                                                              \
+    do {                                                                                                    \
+        if (wide) hipLaunchKernelGGL((paged_decode_kernel<D, BSL, GPV, DT, 4>), grid, block, lds, stream, p); \
+        else hipLaunchKernelGGL((paged_decode_kernel<D, BSL, GPV, DT, 1>), grid, block, lds, stream, p);      \
+    } while (0)
 #define FQ_DECODE_BS(BSL)                        \
     do {                                         \
         if (p.G <= 4) FQ_DECODE_GP(BSL, 4);      \
@@ -570,6 +671,8 @@ int launch_reduce(const float* acc, const float* m, const float* l, const float*
     return fq_host::check_launch();
 }
 
+int effective_splits(int num_splits, int num_seqs, int H_KV, int block_size, int max_blocks_per_seq);
+
 inline int check_decode_shape(int num_seqs, int H_Q, int H_KV, int D, int block_size, int max_blocks_per_seq,
                               int64_t num_blocks, int dtype, int num_splits) {
     if (num_seqs < 0 || H_Q <= 0 || H_KV <= 0 || max_blocks_per_seq <= 0 || num_blocks <= 0 || num_splits < 0)
@@ -589,6 +692,16 @@ namespace fq_host {
 int device_cu_count();
 }
 
+// A split keeps its page ids in at most 4 registers of 64 lanes: it may span at most
+// 256 pages, which bounds the split count from below for long contexts.
+extern "C" int fq_paged_decode_min_splits(int block_size, int max_blocks_per_seq) {
+    if (block_size <= 0 || max_blocks_per_seq <= 0) return 1;
+    const int64_t max_ctx = int64_t(block_size) * max_blocks_per_seq;
+    const int64_t cap = 256 * int64_t(block_size);      // tokens per split, a multiple of 64
+    const int64_t ns = (max_ctx + cap - 1) / cap;
+    return int(ns < 1 ? 1 : ns);
+}
+
 extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_size, int max_blocks_per_seq) {
     if (num_seqs <= 0 || H_KV <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 1;
     const int64_t max_ctx = int64_t(block_size) * max_blocks_per_seq;
@@ -598,14 +711,22 @@ extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_siz
     int64_t ns = (target_waves + int64_t(num_seqs) * H_KV - 1) / (int64_t(num_seqs) * H_KV);
     if (ns > tiles) ns = tiles;
     if (ns > 64) ns = 64;
+    const int64_t floor_ns = fq_paged_decode_min_splits(block_size, max_blocks_per_seq);
+    if (ns < floor_ns) ns = floor_ns;
     if (ns < 1) ns = 1;
     return int(ns);
+}
+
+int fq::effective_splits(int num_splits, int num_seqs, int H_KV, int block_size, int max_blocks_per_seq) {
+    if (num_splits <= 0) return fq_paged_decode_auto_splits(num_seqs, H_KV, block_size, max_blocks_per_seq);
+    const int floor_ns = fq_paged_decode_min_splits(block_size, max_blocks_per_seq);
+    return num_splits < floor_ns ? floor_ns : num_splits;
 }
 
 extern "C" size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_KV, int D, int block_size,
                                                   int max_blocks_per_seq, int num_splits) {
     if (num_seqs <= 0 || H_Q <= 0 || H_KV <= 0 || D <= 0) return 0;
-    if (num_splits <= 0) num_splits = fq_paged_decode_auto_splits(num_seqs, H_KV, block_size, max_blocks_per_seq);
+    num_splits = fq::effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
     return fq::workspace_layout(num_seqs, H_Q, D, num_splits).total;
 }
 
@@ -633,7 +754,7 @@ extern "C" int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache, c
     const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
                                        num_splits);
     if (bad != FQ_OK) return bad;
-    if (num_splits < 1) return FQ_ERR_BAD_SHAPE;
+    if (num_splits < fq_paged_decode_min_splits(block_size, max_blocks_per_seq)) return FQ_ERR_BAD_SHAPE;
     if (num_seqs == 0) return FQ_OK;
     if (!q_rot || !kv_cache || !block_table || !seq_lens || !centroids_k || !centroids_v || !partial_acc ||
         !partial_m || !partial_l)
@@ -690,7 +811,7 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     if (num_seqs == 0) return FQ_OK;
     if (!q || !out) return FQ_ERR_NULL_POINTER;
     if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16)) return FQ_ERR_MISALIGNED;
-    if (num_splits == 0) num_splits = fq_paged_decode_auto_splits(num_seqs, H_KV, block_size, max_blocks_per_seq);
+    num_splits = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
     const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_splits);
     if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
     if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;

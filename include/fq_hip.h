@@ -156,6 +156,11 @@ int fq_split_k_reduce(const float* partial_acc, const float* partial_m,
 int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_size,
                                 int max_blocks_per_seq);
 
+/* Smallest split count the decode kernel accepts for this context length: a
+ * split may span at most 256 pages.  fq_split_k_paged_decode raises a smaller
+ * request to this value; fq_paged_tq4_decode rejects it (FQ_ERR_BAD_SHAPE). */
+int fq_paged_decode_min_splits(int block_size, int max_blocks_per_seq);
+
 /* Bytes of workspace for the given launch; num_splits == 0 means "auto". */
 size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_KV, int D,
                                        int block_size, int max_blocks_per_seq,
