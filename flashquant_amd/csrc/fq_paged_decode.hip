@@ -43,14 +43,26 @@
 //            2x2 nibble transpose of token pairs makes each byte hold the same
 //            coordinate of two consecutive tokens: again one lookup per byte.
 
+#include <cstdlib>
+
 #include "fq_common.hpp"
+
+#ifndef FQ_STAGED_DEBUG_MODE
+#define FQ_STAGED_DEBUG_MODE 0   // 1: copy only, 2: compute only (timing experiments; never shipped)
+#endif
+
+namespace fq_host {
+// FQ_DECODE_DIRECT=1 in the environment routes every shape to the direct kernel
+// (both kernels are kept tested).
+bool force_direct_decode();
+}
 
 namespace fq {
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kTinyNorm = 1e-30f;
-constexpr int kLutCopies = 32;
-constexpr int kLutWords = 256 * kLutCopies;   // per table
+constexpr int kLutCopies = 64;                // one copy per lane: entry stride 256 bytes
+constexpr int kLutWords = 256 * kLutCopies;   // per table (64 KB)
+constexpr float kHalfMax = 65504.0f;
 
 struct DecodeParams {
     const void* q_rot;          // (S, H_Q, D) query dtype, rotated space
@@ -71,6 +83,51 @@ struct DecodeParams {
 };
 
 __device__ __forceinline__ uint32_t byte_of(uint32_t w, int b) { return (w >> (8 * b)) & 0xffu; }
+
+// LDS byte address of table entry `byte K of w` in the copy of this lane: the entry
+// stride is 256 bytes and lane_off = 4 * lane < 256, so the address is the two bytes
+// (byte K of w, lane_off) side by side: one v_perm_b32 instead of extract, shift and add.
+template <int K>
+__device__ __forceinline__ uint32_t lut_addr(uint32_t w, uint32_t lane_off) {
+    return __builtin_amdgcn_perm(w, lane_off, 0x0C0C0000u | ((4u + K) << 8));
+}
+__device__ __forceinline__ uint32_t lds_word(const uint8_t* table, uint32_t addr) {
+    return *reinterpret_cast<const uint32_t*>(table + addr);
+}
+// the four fp16 pairs of the four bytes of w
+__device__ __forceinline__ uint4v lookup_word(const uint8_t* table, uint32_t w, uint32_t lane_off) {
+    uint4v r;
+    r.x = lds_word(table, lut_addr<0>(w, lane_off));
+    r.y = lds_word(table, lut_addr<1>(w, lane_off));
+    r.z = lds_word(table, lut_addr<2>(w, lane_off));
+    r.w = lds_word(table, lut_addr<3>(w, lane_off));
+    return r;
+}
+// byte BI of each of four words
+template <int BI>
+__device__ __forceinline__ uint4v lookup_column(const uint8_t* table, const uint32_t (&src)[4], uint32_t lane_off) {
+    uint4v r;
+    r.x = lds_word(table, lut_addr<BI>(src[0], lane_off));
+    r.y = lds_word(table, lut_addr<BI>(src[1], lane_off));
+    r.z = lds_word(table, lut_addr<BI>(src[2], lane_off));
+    r.w = lds_word(table, lut_addr<BI>(src[3], lane_off));
+    return r;
+}
+
+// Fills a 64-copy byte table: entry (byte, copy) = fp16 pair (centroid[byte >> 4],
+// centroid[byte & 15]).  The 16 centroids are fetched once (lane l holds centroid
+// l % 16); a wavefront then writes one byte's 64 copies per step, picking the two
+// values with v_readlane, so the build is a short LDS-write loop with no memory
+// latency inside it.
+__device__ __forceinline__ void build_byte_table(uint32_t* table, const float* __restrict__ centroids, int wave,
+                                                 int waves, int lane) {
+    const float mine = centroids[lane & 15];
+    for (int byte = wave; byte < 256; byte += waves) {
+        const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), byte >> 4));
+        const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), byte & 15));
+        table[byte * kLutCopies + lane] = pack_h2(_Float16(hi), _Float16(lo));
+    }
+}
 
 // Cross-lane helpers that stay in the VALU (no LDS round trip).
 template <int CTRL>
@@ -108,7 +165,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     constexpr int NC = 4 / NB;            // kept blocks per lane per tile
     constexpr int ROW_HALF = D / 2;
 
-    extern __shared__ uint32_t lut[];
+    __shared__ __attribute__((aligned(256))) uint32_t lut[kLutWords];   // K table (static: constant LDS address)
+    extern __shared__ uint32_t lut2[];                                  // V table when it differs
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -122,18 +180,13 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     const int h = blockIdx.z * waves + wave;
 
     // ---- byte -> (fp16, fp16) tables, one copy per LDS bank ----------------------
-    {
-        const int tables = p.two_tables ? 2 : 1;
-        for (int e = threadIdx.x; e < tables * kLutWords; e += blockDim.x) {
-            const float* c = e >= kLutWords ? p.centroids_v : p.centroids_k;
-            const int byte = (e % kLutWords) / kLutCopies;
-            lut[e] = pack_h2(_Float16(c[byte >> 4]), _Float16(c[byte & 15]));
-        }
-    }
+    build_byte_table(lut, p.centroids_k, wave, waves, lane);
+    if (p.two_tables) build_byte_table(lut2, p.centroids_v, wave, waves, lane);
     __syncthreads();
     if (h >= p.H_KV) return;
-    const uint32_t* lut_k = lut + (lane & 31);
-    const uint32_t* lut_v = lut_k + (p.two_tables ? kLutWords : 0);
+    const uint8_t* lut_k = reinterpret_cast<const uint8_t*>(lut);
+    const uint8_t* lut_v = p.two_tables ? reinterpret_cast<const uint8_t*>(lut2) : lut_k;
+    const uint32_t lane_off = 4u * lane;
 
     int L = p.seq_lens[seq];
     L = L < 0 ? 0 : L;
@@ -311,15 +364,6 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     float M = -__builtin_inff();
     float lsum = 0.0f;
 
-    // One operand (8 fp16 values) from 4 packed bytes: 4 conflict-free LDS reads.
-    auto lookup4 = [&](const uint32_t* tab, uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) -> uint4v {
-        uint4v r;
-        r.x = tab[b0 * kLutCopies];
-        r.y = tab[b1 * kLutCopies];
-        r.z = tab[b2 * kLutCopies];
-        r.w = tab[b3 * kLutCopies];
-        return r;
-    };
     constexpr int VG = DPL / 4;      // groups of four coordinate blocks per k-step of P.V
 
     auto compute_tile = [&](int t0, const Tile& cur) {
@@ -331,7 +375,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const uint32_t w = cur.k[blk][ks];
-                dst[ks] = lookup4(lut_k, byte_of(w, 0), byte_of(w, 1), byte_of(w, 2), byte_of(w, 3));
+                dst[ks] = lookup_word(lut_k, w, lane_off);
             }
         };
         // nibble transposes of the V token pairs (all of them: 2 k-steps x 4 pairs)
@@ -353,8 +397,11 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             for (int e = 0; e < 4; ++e) {
                 const int db = 4 * q4 + e, bi = db / 2;
                 const uint32_t (&src)[4][VW] = (db & 1) ? Y[ks] : X[ks];
-                dst[e] = lookup4(lut_v, byte_of(src[0][bi / 4], bi % 4), byte_of(src[1][bi / 4], bi % 4),
-                                 byte_of(src[2][bi / 4], bi % 4), byte_of(src[3][bi / 4], bi % 4));
+                const uint32_t col[4] = {src[0][bi / 4], src[1][bi / 4], src[2][bi / 4], src[3][bi / 4]};
+                dst[e] = (bi % 4 == 0) ? lookup_column<0>(lut_v, col, lane_off)
+                       : (bi % 4 == 1) ? lookup_column<1>(lut_v, col, lane_off)
+                       : (bi % 4 == 2) ? lookup_column<2>(lut_v, col, lane_off)
+                                       : lookup_column<3>(lut_v, col, lane_off);
             }
         };
 
@@ -376,7 +423,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        float a_[NC][4], rv[NC][4];
+        float a_[NC][4], rv[NC][4];   // rv: value norm of a live token, 0 for a masked one
         float tmax = -__builtin_inff();
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
@@ -384,10 +431,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
             for (int i = 0; i < 4; ++i) {
                 const int tok = t0 + 16 * (c * NB + bc_lane) + 4 * g + i;
                 const bool live = tok < end;
-                const float vn = __builtin_fmaxf(cur.vn[c][i], kTinyNorm);
-                rv[c][i] = live ? __builtin_amdgcn_rcpf(vn) : 0.0f;
-                const float a = __builtin_fmaf(s_[c][i] * cur.kn[c][i], qscale, __builtin_amdgcn_logf(vn));
-                a_[c][i] = live ? a : -__builtin_inff();
+                rv[c][i] = live ? cur.vn[c][i] : 0.0f;
+                a_[c][i] = live ? s_[c][i] * cur.kn[c][i] * qscale : -__builtin_inff();
                 tmax = __builtin_fmaxf(tmax, a_[c][i]);
             }
         }
@@ -404,8 +449,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float w = __builtin_amdgcn_exp2f(a_[c][i] - Ms);
-                psum = __builtin_fmaf(w, rv[c][i], psum);
-                wh[c][i] = _Float16(w);
+                psum += w;
+                wh[c][i] = _Float16(__builtin_fminf(w * rv[c][i], kHalfMax));
             }
         }
         lsum = __builtin_fmaf(lsum, alpha, psum);
@@ -517,85 +562,587 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     }
 }
 
-// q_rot[s, h, j] = sum_k q[s, h, k] * R[j, k], rounded to the query dtype
-// (src/flashquant/kernels/paged_decode.py:113).  One workgroup per (sequence, 8 heads).
-template <int D, int DT>
-__global__ __launch_bounds__(256) void rotate_q_kernel(const uint16_t* __restrict__ q, const float* __restrict__ R,
-                                                       uint16_t* __restrict__ q_rot, int H_Q) {
-    constexpr int HB = 8;
-    __shared__ float qs[HB][D];
-    const int seq = blockIdx.x, h0 = blockIdx.y * HB;
-    const int heads = H_Q - h0 < HB ? H_Q - h0 : HB;
-    for (int i = threadIdx.x; i < heads * D; i += 256)
-        qs[i / D][i % D] = load_elem<DT>(q[(int64_t(seq) * H_Q + h0) * D + i]);
-    __syncthreads();
-    for (int j = threadIdx.x; j < D; j += 256) {
-        float acc[HB];
+// ---------------------------------------------------------------------------------------
+// Staged variant for 8 KV heads of dimension 128 (the common GQA layout).
+//
+// The direct kernel above lets every wavefront fetch its own head's bytes, which are
+// 64-byte halves of cache lines it shares with the neighbouring head and 4-byte norms
+// inside 32-byte strips shared by all heads: the vector L1 then spends its time on
+// requests for lines that are already in flight.  Here the workgroup (8 wavefronts, one
+// per KV head) copies whole token rows: thread t moves the 16-byte chunks t, t + 512, ...
+// of a 32-token tile, so every wavefront request covers eight complete cache lines and
+// each line is asked for exactly once.  The chunks land in LDS in a swizzled layout from
+// which the wavefronts read their MFMA operands without bank conflicts:
+//
+//   stage (16 tokens) = [K idx 8 KB | V idx 8 KB | K norms 512 B | V norms 512 B]
+//   16-byte slot of (head h, row r, quarter q) = 64 h + 4 p + (q ^ ((p >> 1) & 3)),
+//   p = r ^ ((r >> 2) & 1) ^ (h & 1)
+//
+// (rows r and r + 4, read together by the P.V operand loads, fall in different halves of
+// the banks; the eight rows read together by a K operand load fall in eight different
+// 16-byte bank groups; the eight chunks a quarter-wave writes together do too).
+//
+// Pipeline, one workgroup barrier per tile: at iteration i the registers holding tile
+// i + 1 (loaded during iteration i - 1) are written to the LDS slot that tile i - 1 has
+// just vacated, the loads of tile i + 2 are issued, and tile i is consumed from LDS.
+// A tile is 32 tokens: two 16-token blocks; with 4 query heads per KV head the 16 MFMA
+// columns carry (head, block, half of the block's rows), so that all lanes own distinct
+// (head, token) scores.
+// ---------------------------------------------------------------------------------------
+
+constexpr int kStageBytes = 17408;            // 16 rows x 8 heads x 136 bytes
+constexpr int kTileBytes = 2 * kStageBytes;   // 32 tokens
+constexpr int kStageKnOff = 16384;
+constexpr int kStageVnOff = 16896;
+constexpr int kChunksPerRow = 68;
+constexpr int kChunksPerTile = 32 * kChunksPerRow;   // 2176
+
+__host__ __device__ constexpr int staged_slot(int h, int r, int q) {
+    const int pp = (r ^ ((r >> 2) & 1) ^ (h & 1)) & 15;
+    return 64 * h + 4 * pp + (q ^ ((pp >> 1) & 3));
+}
+
+// LDS byte offset (inside a tile slot) of the 16-byte chunk `ci` of tile row `row` (0..31).
+__device__ __forceinline__ int staged_chunk_dst(int row, int ci) {
+    const int stage = row >> 4, r = row & 15;
+    int off;
+    if (ci < 32) {
+        off = 16 * staged_slot(ci >> 2, r, ci & 3);
+    } else if (ci < 34) {
+        off = kStageKnOff + 32 * r + 16 * (ci - 32);
+    } else if (ci < 66) {
+        off = 8192 + 16 * staged_slot((ci - 34) >> 2, r, (ci - 34) & 3);
+    } else {
+        off = kStageVnOff + 32 * r + 16 * (ci - 66);
+    }
+    return stage * kStageBytes + off;
+}
+
+template <int BSL, int GP, int DT, int PVR>
+__global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodeParams p) {
+    constexpr int D = 128;
+    constexpr int BS = 1 << BSL;
+    constexpr int KS = 4;                 // k-steps of the score product
+    constexpr int DPL = 8;                // V coordinates per lane
+    constexpr int NSC = GP / 2;           // scores per lane per tile
+    constexpr int H = 8;
+    constexpr int ROWB = H * (D + 8);     // 1088
+    constexpr int PPT = BS >= 32 ? 1 : 32 / BS;   // pages per tile
+
+    // The table is a static array so that its LDS address is a compile-time constant
+    // that folds into the offset field of every lookup; the tile slots are dynamic.
+    __shared__ __attribute__((aligned(256))) uint32_t lut[kLutWords];
+    extern __shared__ __attribute__((aligned(16))) uint8_t slots[];   // two tile slots
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int h = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront = KV head
+    const int n = lane & 15;
+    const int g = lane >> 4;
+    const int hd = n % GP;
+    const int cls = n / GP;               // column class: GP=4 -> 2*block + half, GP=8 -> block, GP=16 -> 0
+    const int split = blockIdx.x;
+    const int seq = blockIdx.y;
+
+    build_byte_table(lut, p.centroids_k, h, 8, lane);
+    const uint8_t* lut_k = reinterpret_cast<const uint8_t*>(lut);
+    const uint8_t* lut_v = lut_k;          // this kernel is used when K and V share the codebook
+    const uint32_t lane_off = 4u * lane;
+
+    int L = p.seq_lens[seq];
+    L = L < 0 ? 0 : L;
+    L = L > p.max_blocks * BS ? p.max_blocks * BS : L;
+    const int NS = p.num_splits;
+    const int chunk = (((L + NS - 1) / NS) + 63) & ~63;
+    const int begin = split * chunk;
+    const int end = L < begin + chunk ? L : begin + chunk;
+    const int hq_lane = h * p.G + n;
+    if (begin >= end) {   // uniform over the workgroup
+        if (g == 0 && n < p.G) {
+            const int64_t o = (int64_t(seq) * p.H_Q + hq_lane) * NS + split;
+            p.part_m[o] = -__builtin_inff();
+            p.part_l[o] = 0.0f;
+        }
+        return;
+    }
+    const int32_t* bt = p.block_table + int64_t(seq) * p.max_blocks;
+    const int last_page_idx = (L - 1) >> BSL;
+    const int max_page = p.num_blocks - 1;
+    const uint8_t* cache = p.cache;
+    constexpr int64_t page_bytes = int64_t(BS) * ROWB;
+
+    // ---- query operand (same as the direct kernel) -----------------------------------
+    half8 qh[KS];
+    float qscale;
+    {
+        float qf[KS][8];
+        float mx = 0.0f;
+        const bool live = hd < p.G;
+        const uint16_t* qsrc = reinterpret_cast<const uint16_t*>(p.q_rot) +
+                               (int64_t(seq) * p.H_Q + h * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
-        for (int hh = 0; hh < HB; ++hh) acc[hh] = 0.0f;
-        const float4v* row = reinterpret_cast<const float4v*>(R + int64_t(j) * D);
-        for (int k4 = 0; k4 < D / 4; ++k4) {
-            const float4v r = row[k4];
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint4v raw = *reinterpret_cast<const uint4v*>(qsrc + 8 * ks);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-            for (int hh = 0; hh < HB; ++hh) {
-                acc[hh] = __builtin_fmaf(qs[hh][4 * k4], r.x, acc[hh]);
-                acc[hh] = __builtin_fmaf(qs[hh][4 * k4 + 1], r.y, acc[hh]);
-                acc[hh] = __builtin_fmaf(qs[hh][4 * k4 + 2], r.z, acc[hh]);
-                acc[hh] = __builtin_fmaf(qs[hh][4 * k4 + 3], r.w, acc[hh]);
+            for (int i = 0; i < 4; ++i) {
+                qf[ks][2 * i] = live ? load_elem<DT>(uint16_t(w[i] & 0xffffu)) : 0.0f;
+                qf[ks][2 * i + 1] = live ? load_elem<DT>(uint16_t(w[i] >> 16)) : 0.0f;
+                mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(qf[ks][2 * i]), __builtin_fabsf(qf[ks][2 * i + 1])));
             }
         }
-        for (int hh = 0; hh < heads; ++hh)
-            q_rot[(int64_t(seq) * H_Q + h0 + hh) * D + j] = store_elem<DT>(acc[hh]);
+        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 16));
+        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 32));
+        int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+        if (ex < -100 || ex > 100) ex = 0;
+        const float down = bits_to_float(uint32_t(127 - ex) << 23);
+        qscale = p.scale_log2e * bits_to_float(uint32_t(127 + ex) << 23);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qh[ks][e] = _Float16(qf[ks][e] * down);
+    }
+
+    // ---- page ids of the split in registers (see the direct kernel) ---------------------
+    int pv[PVR];
+    const int split_p0 = begin >> BSL;
+#pragma unroll
+    for (int r = 0; r < PVR; ++r) {
+        int idx = split_p0 + 64 * r + lane;
+        idx = idx > last_page_idx ? last_page_idx : idx;
+        int pg = bt[idx];
+        pv[r] = pg < 0 ? 0 : (pg > max_page ? max_page : pg);
+    }
+    auto page_id = [&](int rel) -> int {
+        int v = __builtin_amdgcn_readlane(pv[0], rel & 63);
+#pragma unroll
+        for (int r = 1; r < PVR; ++r) {
+            const int vr = __builtin_amdgcn_readlane(pv[r], rel & 63);
+            v = (rel >> 6) == r ? vr : v;
+        }
+        return v;
+    };
+
+    // ---- copy plan: chunk c = tid + 512 k of the tile, k = 0..4 (the last round only
+    // for the first 128 threads) -----------------------------------------------------------
+    constexpr int ROUNDS = 5;
+    uint32_t src_off[ROUNDS];    // byte offset from the base of the chunk's page
+    int src_page[ROUNDS];        // which of the tile's pages (lane constant)
+    int dst_off[ROUNDS];         // byte offset inside the LDS tile slot
+#pragma unroll
+    for (int k = 0; k < ROUNDS; ++k) {
+        int c = tid + 512 * k;
+        c = c < kChunksPerTile ? c : kChunksPerTile - 1;
+        const int row = c / kChunksPerRow, ci = c % kChunksPerRow;
+        src_page[k] = BS >= 32 ? 0 : row >> BSL;
+        src_off[k] = uint32_t((row & (BS - 1)) * ROWB + ci * 16);
+        dst_off[k] = staged_chunk_dst(row, ci);
+    }
+    const bool has_round4 = tid < kChunksPerTile - 4 * 512;   // 128 threads, whole wavefronts
+
+    uint4v stage_reg[ROUNDS];
+    auto issue_loads = [&](int t0) {
+        const uint8_t* base[PPT];
+        const int p0 = (t0 >> BSL) - split_p0;
+#pragma unroll
+        for (int i = 0; i < PPT; ++i) base[i] = cache + int64_t(page_id(p0 + i)) * page_bytes;
+        const uint32_t in_page = BS >= 32 ? uint32_t((t0 & (BS - 1)) * ROWB) : 0u;
+#pragma unroll
+        for (int k = 0; k < ROUNDS; ++k) {
+            const uint8_t* b = base[0];
+#pragma unroll
+            for (int i = 1; i < PPT; ++i) b = src_page[k] == i ? base[i] : b;
+            if (k < 4 || has_round4) stage_reg[k] = *reinterpret_cast<const uint4v*>(b + in_page + src_off[k]);
+        }
+    };
+    auto write_slot = [&](int slot) {
+        uint8_t* dst = slots + slot * kTileBytes;
+#pragma unroll
+        for (int k = 0; k < ROUNDS; ++k)
+            if (k < 4 || has_round4) *reinterpret_cast<uint4v*>(dst + dst_off[k]) = stage_reg[k];
+    };
+
+    // ---- lane-constant LDS read offsets (inside a tile slot) -------------------------------
+    int k_rd[2];                // K operand of block b: 16 bytes of row n, quarter g
+    int v_rd[2][4];             // V operand: dword n of rows 4g + i of block b
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        k_rd[b] = b * kStageBytes + 16 * staged_slot(h, n, g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            v_rd[b][i] = b * kStageBytes + 8192 + 16 * staged_slot(h, 4 * g + i, n >> 2) + 4 * (n & 3);
+    }
+    // the (block, row) of this lane's scores, and the slot of each score in the P operand
+    int sc_tok[NSC];            // token offset inside the tile
+    int n_rd[NSC];              // K norm offset; the V norm is 512 bytes further
+#pragma unroll
+    for (int e = 0; e < NSC; ++e) {
+        int blk, row;
+        if (GP == 4) { blk = cls >> 1; row = 4 * g + 2 * (cls & 1) + e; }
+        else if (GP == 8) { blk = cls; row = 4 * g + e; }
+        else { blk = e >> 2; row = 4 * g + (e & 3); }
+        sc_tok[e] = 16 * blk + row;
+        n_rd[e] = blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
+    }
+
+    // ---- running state ---------------------------------------------------------------------
+    float4v O[DPL];
+#pragma unroll
+    for (int db = 0; db < DPL; ++db) O[db] = float4v{0.f, 0.f, 0.f, 0.f};
+    float M = -__builtin_inff();
+    float lsum = 0.0f;
+
+    auto compute_tile = [&](int t0, int slot) {
+        const uint8_t* tile = slots + slot * kTileBytes;
+        // operands of this lane, raw
+        uint4v kraw[2];
+        uint32_t vraw[2][4];
+        float kn[NSC], vn[NSC];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) kraw[b] = *reinterpret_cast<const uint4v*>(tile + k_rd[b]);
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vraw[b][i] = *reinterpret_cast<const uint32_t*>(tile + v_rd[b][i]);
+#pragma unroll
+        for (int e = 0; e < NSC; ++e) {
+            kn[e] = *reinterpret_cast<const float*>(tile + n_rd[e]);
+            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageVnOff - kStageKnOff));
+        }
+
+        // ---- scores: lookups of block 1 in flight during the MFMAs of block 0 ----------------
+        uint4v ka[2][KS];
+        const uint32_t kw[2][4] = {{kraw[0].x, kraw[0].y, kraw[0].z, kraw[0].w}, {kraw[1].x, kraw[1].y, kraw[1].z, kraw[1].w}};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) ka[0][ks] = lookup_word(lut_k, kw[0][ks], lane_off);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) ka[1][ks] = lookup_word(lut_k, kw[1][ks], lane_off);
+        // nibble transposes of the V token pairs: pair jp = rows (2 jp', 2 jp' + 1) of block jp / 2
+        uint32_t X[4], Y[4];
+#pragma unroll
+        for (int jp = 0; jp < 4; ++jp) {
+            const uint32_t A = vraw[jp >> 1][2 * (jp & 1)], B = vraw[jp >> 1][2 * (jp & 1) + 1];
+            X[jp] = (A & 0xF0F0F0F0u) | ((B >> 4) & 0x0F0F0F0Fu);
+            Y[jp] = ((A << 4) & 0xF0F0F0F0u) | (B & 0x0F0F0F0Fu);
+        }
+        uint4v vb[2][4];
+        auto v_group = [&](int grp, uint4v (&dst)[4]) {   // coordinate blocks 4 grp .. 4 grp + 3
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int db = 4 * grp + e, bi = db / 2;
+                const uint32_t (&src)[4] = (db & 1) ? Y : X;
+                dst[e] = (bi == 0) ? lookup_column<0>(lut_v, src, lane_off)
+                       : (bi == 1) ? lookup_column<1>(lut_v, src, lane_off)
+                       : (bi == 2) ? lookup_column<2>(lut_v, src, lane_off)
+                                   : lookup_column<3>(lut_v, src, lane_off);
+            }
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        float4v acc[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            acc[b] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ka[b][ks]), qh[ks], acc[b], 0, 0, 0);
+            if (b == 0) v_group(0, vb[0]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // ---- this lane's scores ------------------------------------------------------------------
+        float a_[NSC], rv[NSC];
+        float tmax = -__builtin_inff();
+#pragma unroll
+        for (int e = 0; e < NSC; ++e) {
+            float s;
+            if (GP == 4) {
+                const float s0 = (cls & 1) ? acc[0][2 + e] : acc[0][e];
+                const float s1 = (cls & 1) ? acc[1][2 + e] : acc[1][e];
+                s = (cls >> 1) ? s1 : s0;
+            } else if (GP == 8) {
+                s = cls ? acc[1][e] : acc[0][e];
+            } else {
+                s = acc[e >> 2][e & 3];
+            }
+            const bool live = t0 + sc_tok[e] < end;
+            rv[e] = live ? vn[e] : 0.0f;
+            a_[e] = live ? s * kn[e] * qscale : -__builtin_inff();
+            tmax = __builtin_fmaxf(tmax, a_[e]);
+        }
+        tmax = max_same_head<GP>(tmax);
+        const float Mnew = __builtin_fmaxf(M, tmax);
+        const float Ms = Mnew == -__builtin_inff() ? 0.0f : Mnew;
+        const float alpha = __builtin_amdgcn_exp2f(M - Ms);
+        M = Mnew;
+        _Float16 wh[NSC];
+        float psum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < NSC; ++e) {
+            const float w = __builtin_amdgcn_exp2f(a_[e] - Ms);
+            psum += w;
+            wh[e] = _Float16(__builtin_fminf(w * rv[e], kHalfMax));
+        }
+        lsum = __builtin_fmaf(lsum, alpha, psum);
+
+        if (__any(alpha != 1.0f)) {
+            float ar[4];
+            if (GP == 4) {
+                ar[0] = dpp_mov<0x00>(alpha);
+                ar[1] = dpp_mov<0x55>(alpha);
+                ar[2] = dpp_mov<0xAA>(alpha);
+                ar[3] = dpp_mov<0xFF>(alpha);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * g + i, kWave);
+            }
+#pragma unroll
+            for (int db = 0; db < DPL; ++db)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) O[db][i] *= ar[i];
+        }
+
+        // ---- weights as the A operand: slot j <-> (block j / 4, row 4g + j % 4) -------------------
+        half8 pa;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            constexpr _Float16 zero = _Float16(0.0f);
+            if (GP == 4) pa[j] = ((j >> 2) == (cls >> 1) && ((j >> 1) & 1) == (cls & 1)) ? wh[j & 1] : zero;
+            else if (GP == 8) pa[j] = ((j >> 2) == cls) ? wh[(j & 3) % NSC] : zero;
+            else pa[j] = wh[j % NSC];
+        }
+
+        // ---- O += P . V ------------------------------------------------------------------------------
+        __builtin_amdgcn_sched_barrier(0);
+        v_group(1, vb[1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            O[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(half8, vb[0][e]), O[e], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            O[4 + e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(half8, vb[1][e]), O[4 + e], 0, 0, 0);
+    };
+
+    // ---- tiles ------------------------------------------------------------------------------------
+    {
+        const int last_t0 = begin + ((end - begin - 1) & ~31);
+        auto clamp_t0 = [&](int t) { return t < last_t0 ? t : last_t0; };
+        issue_loads(begin);
+        write_slot(0);
+        issue_loads(clamp_t0(begin + 32));
+        int i = 0;
+        for (int t0 = begin; t0 < (FQ_STAGED_DEBUG_MODE == 3 ? begin : end); t0 += 32, ++i) {
+#ifndef FQ_STAGED_NO_BARRIER
+            __syncthreads();                      // tile i is in LDS; slot of tile i - 1 is free
+#endif
+#if FQ_STAGED_DEBUG_MODE != 2
+            write_slot((i + 1) & 1);              // tile i + 1 (its loads ran during tile i - 1)
+            issue_loads(clamp_t0(t0 + 64));       // tile i + 2
+#endif
+#if FQ_STAGED_DEBUG_MODE != 1
+            compute_tile(t0, i & 1);
+#endif
+        }
+    }
+
+    // ---- publish the partial of this split (as in the direct kernel) -----------------------------
+#pragma unroll
+    for (int mask = GP; mask < 64; mask <<= 1) lsum += xor_shuffle(lsum, mask);
+#pragma unroll
+    for (int db = 0; db < DPL; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = O[db][i];
+#pragma unroll
+            for (int mask = 4 * GP; mask < 64; mask <<= 1) v += xor_shuffle(v, mask);
+            O[db][i] = v;
+        }
+    if (g == 0 && n < p.G) {
+        const int64_t o = (int64_t(seq) * p.H_Q + hq_lane) * NS + split;
+        p.part_m[o] = M;
+        p.part_l[o] = lsum;
+    }
+    if (g < GP / 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int head = 4 * g + i;
+            if (head < p.G) {
+                float* dst = p.part_acc + ((int64_t(seq) * p.H_Q + h * p.G + head) * NS + split) * D + n * DPL;
+#pragma unroll
+                for (int q4 = 0; q4 < DPL / 4; ++q4) {
+                    const float4v v = {O[4 * q4][i], O[4 * q4 + 1][i], O[4 * q4 + 2][i], O[4 * q4 + 3][i]};
+                    *reinterpret_cast<float4v*>(dst + 4 * q4) = v;
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Head rotations: rows of D elements times the D x D rotation, float32 throughout, on the
+// float32 MFMA (v_mfma_f32_16x16x4_f32), so that no splitting of the matrix is needed and
+// the result matches a float32 matmul to rounding.  A workgroup (4 wavefronts) owns 16
+// rows; wavefront w produces the 16-column blocks w, w + 4, ...
+//
+// The contraction index is permuted so that operands load as contiguous runs: MFMA step
+// (j, e) with lane group g uses k = 32 j + 8 g + e, hence lane (m, g) holds the 8-element
+// runs k = 32 j + 8 g .. + 7 of row m (A side) and of the matrix (B side).
+// ---------------------------------------------------------------------------------------
+
+constexpr int kRotRows = 16;
+
+// B operand values of one 16-column block.  TRANSPOSED: out = x @ R.T (B[k][n] = R[col+n][k],
+// contiguous in k); otherwise out = x @ R (B[k][n] = R[k][col+n], 16 lanes contiguous in n).
+template <int D, bool TRANSPOSED>
+__device__ __forceinline__ void load_rotation_block(const float* __restrict__ R, int col, int n, int g,
+                                                    float (&b)[D / 32][8]) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+        if (TRANSPOSED) {
+            const float4v* src = reinterpret_cast<const float4v*>(R + int64_t(col + n) * D + 32 * j + 8 * g);
+            const float4v lo = src[0], hi = src[1];
+            b[j][0] = lo.x; b[j][1] = lo.y; b[j][2] = lo.z; b[j][3] = lo.w;
+            b[j][4] = hi.x; b[j][5] = hi.y; b[j][6] = hi.z; b[j][7] = hi.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) b[j][e] = R[int64_t(32 * j + 8 * g + e) * D + col + n];
+        }
+    }
+}
+
+template <int D>
+__device__ __forceinline__ float4v rotate_block(const float (&a)[D / 32][8], const float (&b)[D / 32][8]) {
+    // four independent partial sums: a single accumulator would chain D/4 dependent MFMAs
+    float4v acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            acc[e & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j][e], b[j][e], acc[e & 3], 0, 0, 0);
+    return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+}
+
+// q_rot[row, j] = sum_k q[row, k] * R[j, k], rounded to the query dtype
+// (src/flashquant/kernels/paged_decode.py:113).  rows = num_seqs * H_Q.
+template <int D, int DT>
+__global__ __launch_bounds__(256) void rotate_q_kernel(const uint16_t* __restrict__ q, const float* __restrict__ R,
+                                                       uint16_t* __restrict__ q_rot, int64_t rows) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int64_t row0 = int64_t(blockIdx.x) * kRotRows;
+    const int64_t my_row = row0 + n < rows ? row0 + n : rows - 1;
+    float a[D / 32][8];
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+        const uint4v raw = *reinterpret_cast<const uint4v*>(q + my_row * D + 32 * j + 8 * g);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a[j][2 * i] = load_elem<DT>(uint16_t(w[i] & 0xffffu));
+            a[j][2 * i + 1] = load_elem<DT>(uint16_t(w[i] >> 16));
+        }
+    }
+    for (int cb = wave; cb < D / 16; cb += 4) {
+        float b[D / 32][8];
+        load_rotation_block<D, true>(R, 16 * cb, n, g, b);
+        const float4v acc = rotate_block<D>(a, b);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t row = row0 + 4 * g + i;
+            if (row < rows) q_rot[row * D + 16 * cb + n] = store_elem<DT>(acc[i]);
+        }
     }
 }
 
 // Combine of the split partials: out_rot = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
 // (0 when every split is empty), rounded to the query dtype as the reference's
-// rotated-space result is (cpu_reference.py:366), then multiplied by R in float32
-// and rounded again (paged_decode.py:123).  One workgroup per (sequence, 8 heads).
+// rotated-space result is (cpu_reference.py:366), then multiplied by R in float32 and
+// rounded again (paged_decode.py:123).  rows = num_seqs * H_Q; a workgroup owns 16 rows:
+// each wavefront combines 4 of them into LDS, then all rotate from there.
 template <int D, int DT>
 __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restrict__ part_acc,
                                                             const float* __restrict__ part_m,
                                                             const float* __restrict__ part_l,
                                                             const float* __restrict__ R, uint16_t* __restrict__ out,
-                                                            int H_Q, int NS) {
-    constexpr int HB = 8;
-    __shared__ float os[HB][D];
-    const int seq = blockIdx.x, h0 = blockIdx.y * HB;
-    const int heads = H_Q - h0 < HB ? H_Q - h0 : HB;
-    for (int i = threadIdx.x; i < heads * D; i += 256) {
-        const int hh = i / D, d = i % D;
-        const int64_t base = (int64_t(seq) * H_Q + h0 + hh) * NS;
+                                                            int64_t rows, int NS) {
+    __shared__ float os[kRotRows][D + 4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int64_t row0 = int64_t(blockIdx.x) * kRotRows;
+    // ---- combine: thread t handles 8 consecutive coordinates of row t / 16; splits are taken
+    // eight at a time so that their loads are all in flight together ------------------------------
+    {
+        const int r = threadIdx.x >> 4;
+        const int64_t row = row0 + r < rows ? row0 + r : rows - 1;
+        const int64_t base = row * NS;
         float mstar = -__builtin_inff();
-        for (int s = 0; s < NS; ++s) mstar = __builtin_fmaxf(mstar, part_m[base + s]);
-        float num = 0.0f, den = 0.0f;
-        for (int s = 0; s < NS; ++s) {
-            const float m = part_m[base + s];
-            if (m == -__builtin_inff()) continue;
-            const float w = __builtin_amdgcn_exp2f(m - mstar);
-            num = __builtin_fmaf(part_acc[(base + s) * D + d], w, num);
-            den = __builtin_fmaf(part_l[base + s], w, den);
+        for (int s0 = 0; s0 < NS; s0 += 8) {
+            float mv[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) mv[k] = part_m[base + (s0 + k < NS ? s0 + k : NS - 1)];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) mstar = __builtin_fmaxf(mstar, mv[k]);
         }
-        const float v = den > 0.0f ? num / den : 0.0f;
-        os[hh][d] = load_elem<DT>(store_elem<DT>(v));
+        for (int c0 = 8 * (threadIdx.x & 15); c0 < D; c0 += 128) {
+            float num[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) num[e] = 0.0f;
+            float den = 0.0f;
+            for (int s0 = 0; s0 < NS; s0 += 8) {
+                float mv[8], lv[8];
+                float4v lo[8], hi[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int sidx = s0 + k < NS ? s0 + k : NS - 1;
+                    mv[k] = part_m[base + sidx];
+                    lv[k] = part_l[base + sidx];
+                    // an empty split (m = -inf) never wrote its accumulator: do not read it
+                    const bool use = s0 + k < NS && mv[k] != -__builtin_inff();
+                    const float4v* src = reinterpret_cast<const float4v*>(part_acc + (base + sidx) * D + c0);
+                    lo[k] = use ? src[0] : float4v{0.f, 0.f, 0.f, 0.f};
+                    hi[k] = use ? src[1] : float4v{0.f, 0.f, 0.f, 0.f};
+                    mv[k] = use ? mv[k] : -__builtin_inff();
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const float w = mv[k] == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(mv[k] - mstar);
+                    den = __builtin_fmaf(lv[k], w, den);
+                    num[0] = __builtin_fmaf(lo[k].x, w, num[0]); num[1] = __builtin_fmaf(lo[k].y, w, num[1]);
+                    num[2] = __builtin_fmaf(lo[k].z, w, num[2]); num[3] = __builtin_fmaf(lo[k].w, w, num[3]);
+                    num[4] = __builtin_fmaf(hi[k].x, w, num[4]); num[5] = __builtin_fmaf(hi[k].y, w, num[5]);
+                    num[6] = __builtin_fmaf(hi[k].z, w, num[6]); num[7] = __builtin_fmaf(hi[k].w, w, num[7]);
+                }
+            }
+            const bool live = row0 + r < rows && den > 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) os[r][c0 + e] = live ? load_elem<DT>(store_elem<DT>(num[e] / den)) : 0.0f;
+        }
     }
     __syncthreads();
     if (R == nullptr) {
-        for (int i = threadIdx.x; i < heads * D; i += 256)
-            out[(int64_t(seq) * H_Q + h0) * D + i] = store_elem<DT>(os[i / D][i % D]);
+        for (int i = threadIdx.x; i < kRotRows * D; i += 256) {
+            const int64_t row = row0 + i / D;
+            if (row < rows) out[row * D + i % D] = store_elem<DT>(os[i / D][i % D]);
+        }
         return;
     }
-    for (int j = threadIdx.x; j < D; j += 256) {
-        float acc[HB];
+    float a[D / 32][8];
 #pragma unroll
-        for (int hh = 0; hh < HB; ++hh) acc[hh] = 0.0f;
-        for (int d = 0; d < D; ++d) {
-            const float r = R[int64_t(d) * D + j];
+    for (int j = 0; j < D / 32; ++j)
 #pragma unroll
-            for (int hh = 0; hh < HB; ++hh) acc[hh] = __builtin_fmaf(os[hh][d], r, acc[hh]);
+        for (int e = 0; e < 8; ++e) a[j][e] = os[n][32 * j + 8 * g + e];
+    for (int cb = wave; cb < D / 16; cb += 4) {
+        float b[D / 32][8];
+        load_rotation_block<D, false>(R, 16 * cb, n, g, b);
+        const float4v acc = rotate_block<D>(a, b);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t row = row0 + 4 * g + i;
+            if (row < rows) out[row * D + 16 * cb + n] = store_elem<DT>(acc[i]);
         }
-        for (int hh = 0; hh < heads; ++hh)
-            out[(int64_t(seq) * H_Q + h0 + hh) * D + j] = store_elem<DT>(acc[hh]);
     }
 }
 
@@ -615,25 +1162,63 @@ inline WorkspaceLayout workspace_layout(int S, int H_Q, int D, int NS) {
     return w;
 }
 
+// Launch with `lds` bytes of dynamic LDS; more than 64 KB per workgroup has to be
+// allowed per kernel function first.
+template <typename K>
+int launch_with_lds(K kernel, const DecodeParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
+    if (lds > 32768 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
+        fq_host::note_hip_error(hipGetLastError());
+        return FQ_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
+    return fq_host::check_launch();
+}
+
+template <typename K>
+int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream) {
+    // dynamic part only; the 64 KB table is static
+    const size_t lds = 2 * size_t(kTileBytes);
+    return launch_with_lds(kernel, p, dim3(p.num_splits, S, 1), dim3(512), lds, stream);
+}
+
 template <int D, int DT>
 int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
-    const int waves = p.H_KV < 8 ? p.H_KV : 8;
-    const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
-    const size_t lds = size_t(p.two_tables ? 2 : 1) * kLutWords * sizeof(uint32_t);
     // pages a split can span: its tokens are ceil(max_ctx / splits) rounded up to a tile
     const int64_t max_ctx = int64_t(p.max_blocks) * BS;
     const int64_t chunk = (((max_ctx + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
     const bool wide = chunk / BS > 64;   // begin is a multiple of 64 tokens, hence page aligned
-#define FQ_DECODE_GP(BSL, GPV)                                                                              \
-    do {                                                                                                    \
-        if (wide) hipLaunchKernelGGL((paged_decode_kernel<D, BSL, GPV, DT, 4>), grid, block, lds, stream, p); \
-        else hipLaunchKernelGGL((paged_decode_kernel<D, BSL, GPV, DT, 1>), grid, block, lds, stream, p);      \
+
+    if (D == 128 && p.H_KV == 8 && !p.two_tables && !fq_host::force_direct_decode()) {
+#define FQ_STAGED_GP(BSL, GPV)                                                                      \
+    return wide ? launch_staged(paged_decode_staged_kernel<BSL, GPV, DT, 4>, p, S, stream)         \
+                : launch_staged(paged_decode_staged_kernel<BSL, GPV, DT, 1>, p, S, stream)
+#define FQ_STAGED_BS(BSL)                         \
+    do {                                          \
+        if (p.G <= 4) { FQ_STAGED_GP(BSL, 4); }   \
+        else if (p.G <= 8) { FQ_STAGED_GP(BSL, 8); } \
+        else { FQ_STAGED_GP(BSL, 16); }           \
     } while (0)
-#define FQ_DECODE_BS(BSL)                        \
-    do {                                         \
-        if (p.G <= 4) FQ_DECODE_GP(BSL, 4);      \
-        else if (p.G <= 8) FQ_DECODE_GP(BSL, 8); \
-        else FQ_DECODE_GP(BSL, 16);              \
+        switch (BS) {
+            case 8: FQ_STAGED_BS(3); break;
+            case 16: FQ_STAGED_BS(4); break;
+            default: FQ_STAGED_BS(5); break;
+        }
+#undef FQ_STAGED_BS
+#undef FQ_STAGED_GP
+    }
+
+    const int waves = p.H_KV < 8 ? p.H_KV : 8;
+    const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
+    const size_t lds = p.two_tables ? size_t(kLutWords) * sizeof(uint32_t) : 0;   // the K table is static
+#define FQ_DECODE_GP(BSL, GPV)                                                                  \
+    return wide ? launch_with_lds(paged_decode_kernel<D, BSL, GPV, DT, 4>, p, grid, block, lds, stream) \
+                : launch_with_lds(paged_decode_kernel<D, BSL, GPV, DT, 1>, p, grid, block, lds, stream)
+#define FQ_DECODE_BS(BSL)                             \
+    do {                                              \
+        if (p.G <= 4) { FQ_DECODE_GP(BSL, 4); }       \
+        else if (p.G <= 8) { FQ_DECODE_GP(BSL, 8); }  \
+        else { FQ_DECODE_GP(BSL, 16); }               \
     } while (0)
     switch (BS) {
         case 8: FQ_DECODE_BS(3); break;
@@ -647,13 +1232,14 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
 
 template <int DT>
 int launch_rotate(const void* q, const float* R, void* q_rot, int S, int H_Q, int D, hipStream_t stream) {
-    const dim3 grid(S, (H_Q + 7) / 8), block(256);
+    const int64_t rows = int64_t(S) * H_Q;
+    const dim3 grid(unsigned((rows + kRotRows - 1) / kRotRows)), block(256);
     const uint16_t* src = reinterpret_cast<const uint16_t*>(q);
     uint16_t* dst = reinterpret_cast<uint16_t*>(q_rot);
     switch (D) {
-        case 64: hipLaunchKernelGGL((rotate_q_kernel<64, DT>), grid, block, 0, stream, src, R, dst, H_Q); break;
-        case 128: hipLaunchKernelGGL((rotate_q_kernel<128, DT>), grid, block, 0, stream, src, R, dst, H_Q); break;
-        default: hipLaunchKernelGGL((rotate_q_kernel<256, DT>), grid, block, 0, stream, src, R, dst, H_Q); break;
+        case 64: hipLaunchKernelGGL((rotate_q_kernel<64, DT>), grid, block, 0, stream, src, R, dst, rows); break;
+        case 128: hipLaunchKernelGGL((rotate_q_kernel<128, DT>), grid, block, 0, stream, src, R, dst, rows); break;
+        default: hipLaunchKernelGGL((rotate_q_kernel<256, DT>), grid, block, 0, stream, src, R, dst, rows); break;
     }
     return fq_host::check_launch();
 }
@@ -661,12 +1247,13 @@ int launch_rotate(const void* q, const float* R, void* q_rot, int S, int H_Q, in
 template <int DT>
 int launch_reduce(const float* acc, const float* m, const float* l, const float* R, void* out, int S, int H_Q,
                   int D, int NS, hipStream_t stream) {
-    const dim3 grid(S, (H_Q + 7) / 8), block(256);
+    const int64_t rows = int64_t(S) * H_Q;
+    const dim3 grid(unsigned((rows + kRotRows - 1) / kRotRows)), block(256);
     uint16_t* dst = reinterpret_cast<uint16_t*>(out);
     switch (D) {
-        case 64: hipLaunchKernelGGL((reduce_rotate_kernel<64, DT>), grid, block, 0, stream, acc, m, l, R, dst, H_Q, NS); break;
-        case 128: hipLaunchKernelGGL((reduce_rotate_kernel<128, DT>), grid, block, 0, stream, acc, m, l, R, dst, H_Q, NS); break;
-        default: hipLaunchKernelGGL((reduce_rotate_kernel<256, DT>), grid, block, 0, stream, acc, m, l, R, dst, H_Q, NS); break;
+        case 64: hipLaunchKernelGGL((reduce_rotate_kernel<64, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS); break;
+        case 128: hipLaunchKernelGGL((reduce_rotate_kernel<128, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS); break;
+        default: hipLaunchKernelGGL((reduce_rotate_kernel<256, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS); break;
     }
     return fq_host::check_launch();
 }
@@ -690,6 +1277,10 @@ inline int check_decode_shape(int num_seqs, int H_Q, int H_KV, int D, int block_
 
 namespace fq_host {
 int device_cu_count();
+bool force_direct_decode() {
+    const char* v = getenv("FQ_DECODE_DIRECT");
+    return v && v[0] == '1';
+}
 }
 
 // A split keeps its page ids in at most 4 registers of 64 lanes: it may span at most
@@ -738,7 +1329,7 @@ extern "C" int fq_rotate_query(const void* q, const float* rotation, void* q_rot
     if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
     if (num_seqs == 0) return FQ_OK;
     if (!q || !rotation || !q_rot) return FQ_ERR_NULL_POINTER;
-    if (!fq_host::aligned(rotation, 16) || !fq_host::aligned(q, 2) || !fq_host::aligned(q_rot, 2))
+    if (!fq_host::aligned(rotation, 16) || !fq_host::aligned(q, 16) || !fq_host::aligned(q_rot, 2))
         return FQ_ERR_MISALIGNED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dtype == FQ_F16 ? launch_rotate<FQ_F16>(q, rotation, q_rot, int(num_seqs), H_Q, D, s)
