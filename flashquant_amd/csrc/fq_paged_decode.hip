@@ -51,6 +51,12 @@
 #define FQ_STAGED_DEBUG_MODE 0   // 1: copy only, 2: compute only (timing experiments; never shipped)
 #endif
 
+#ifdef FQ_DBG_TIMING
+#define FQ_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x == 3 && blockIdx.y == 5) tmark[i] = wall_clock64(); } while (0)
+#else
+#define FQ_MARK(i)
+#endif
+
 namespace fq_host {
 // FQ_DECODE_DIRECT=1 in the environment routes every shape to the direct kernel
 // (both kernels are kept tested).
@@ -65,7 +71,8 @@ constexpr int kLutWords = 256 * kLutCopies;   // per table (64 KB)
 constexpr float kHalfMax = 65504.0f;
 
 struct DecodeParams {
-    const void* q_rot;          // (S, H_Q, D) query dtype, rotated space
+    const void* q_rot;          // (S, H_Q, D) query dtype: rotated, or un-rotated when `rotation` is set
+    const float* rotation;      // staged kernel only: rotate the query in the prologue (NULL: already rotated)
     const uint8_t* cache;       // (num_blocks, BS, H_KV*(D+8))
     const int32_t* block_table; // (S, max_blocks)
     const int32_t* seq_lens;    // (S,)
@@ -119,14 +126,16 @@ __device__ __forceinline__ uint4v lookup_column(const uint8_t* table, const uint
 // l % 16); a wavefront then writes one byte's 64 copies per step, picking the two
 // values with v_readlane, so the build is a short LDS-write loop with no memory
 // latency inside it.
-__device__ __forceinline__ void build_byte_table(uint32_t* table, const float* __restrict__ centroids, int wave,
-                                                 int waves, int lane) {
-    const float mine = centroids[lane & 15];
+__device__ __forceinline__ void fill_byte_table(uint32_t* table, float mine, int wave, int waves, int lane) {
     for (int byte = wave; byte < 256; byte += waves) {
         const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), byte >> 4));
         const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), byte & 15));
         table[byte * kLutCopies + lane] = pack_h2(_Float16(hi), _Float16(lo));
     }
+}
+__device__ __forceinline__ void build_byte_table(uint32_t* table, const float* __restrict__ centroids, int wave,
+                                                 int waves, int lane) {
+    fill_byte_table(table, centroids[lane & 15], wave, waves, lane);
 }
 
 // Cross-lane helpers that stay in the VALU (no LDS round trip).
@@ -152,6 +161,52 @@ __device__ __forceinline__ float max_same_head(float v) {
     if (GP <= 4) v = __builtin_fmaxf(v, dpp_mov<0x124>(v));   // row_ror:4
     if (GP <= 8) v = __builtin_fmaxf(v, dpp_mov<0x128>(v));   // row_ror:8
     return max_xor32(max_xor16(v));
+}
+
+// ---------------------------------------------------------------------------------------
+// Head rotations: rows of D elements times the D x D rotation, float32 throughout, on the
+// float32 MFMA (v_mfma_f32_16x16x4_f32), so that no splitting of the matrix is needed and
+// the result matches a float32 matmul to rounding.  A workgroup (4 wavefronts) owns 16
+// rows; wavefront w produces the 16-column blocks w, w + 4, ...
+//
+// The contraction index is permuted so that operands load as contiguous runs: MFMA step
+// (j, e) with lane group g uses k = 32 j + 8 g + e, hence lane (m, g) holds the 8-element
+// runs k = 32 j + 8 g .. + 7 of row m (A side) and of the matrix (B side).
+// ---------------------------------------------------------------------------------------
+
+constexpr int kRotRows = 16;
+
+// B operand values of one 16-column block.  TRANSPOSED: out = x @ R.T (B[k][n] = R[col+n][k],
+// contiguous in k); otherwise out = x @ R (B[k][n] = R[k][col+n], 16 lanes contiguous in n).
+template <int D, bool TRANSPOSED>
+__device__ __forceinline__ void load_rotation_block(const float* __restrict__ R, int col, int n, int g,
+                                                    float (&b)[D / 32][8]) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+        if (TRANSPOSED) {
+            const float4v* src = reinterpret_cast<const float4v*>(R + int64_t(col + n) * D + 32 * j + 8 * g);
+            const float4v lo = src[0], hi = src[1];
+            b[j][0] = lo.x; b[j][1] = lo.y; b[j][2] = lo.z; b[j][3] = lo.w;
+            b[j][4] = hi.x; b[j][5] = hi.y; b[j][6] = hi.z; b[j][7] = hi.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) b[j][e] = R[int64_t(32 * j + 8 * g + e) * D + col + n];
+        }
+    }
+}
+
+template <int D>
+__device__ __forceinline__ float4v rotate_block(const float (&a)[D / 32][8], const float (&b)[D / 32][8]) {
+    // four independent partial sums: a single accumulator would chain D/4 dependent MFMAs
+    float4v acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            acc[e & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j][e], b[j][e], acc[e & 3], 0, 0, 0);
+    return (acc[0] + acc[1]) + (acc[2] + acc[3]);
 }
 
 template <int D, int BSL, int GP, int DT, int PVR>
@@ -634,6 +689,10 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     __shared__ __attribute__((aligned(256))) uint32_t lut[kLutWords];
     extern __shared__ __attribute__((aligned(16))) uint8_t slots[];   // two tile slots
 
+#ifdef FQ_DBG_TIMING
+    unsigned long long tmark[12] = {};
+#endif
+    FQ_MARK(0);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int h = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront = KV head
@@ -644,10 +703,26 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     const int split = blockIdx.x;
     const int seq = blockIdx.y;
 
-    build_byte_table(lut, p.centroids_k, h, 8, lane);
+    // Every load that depends on nothing is asked for first, so that the memory
+    // latencies of the prologue overlap instead of adding up: the centroids, the
+    // rotation columns of this wavefront and the first 32 query heads.
+    const float cent_mine = p.centroids_k[lane & 15];
     const uint8_t* lut_k = reinterpret_cast<const uint8_t*>(lut);
     const uint8_t* lut_v = lut_k;          // this kernel is used when K and V share the codebook
     const uint32_t lane_off = 4u * lane;
+    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + int64_t(seq) * p.H_Q * 128;
+    float rot_b[4][8];
+    uint4v q_pre[2][4];
+    if (p.rotation != nullptr) {
+        load_rotation_block<128, true>(p.rotation, 16 * h, n, g, rot_b);
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+            const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) q_pre[rb][j] = *reinterpret_cast<const uint4v*>(qseq + row * 128 + 32 * j + 8 * g);
+        }
+    }
+    FQ_MARK(1);
 
     int L = p.seq_lens[seq];
     L = L < 0 ? 0 : L;
@@ -671,38 +746,6 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     const uint8_t* cache = p.cache;
     constexpr int64_t page_bytes = int64_t(BS) * ROWB;
 
-    // ---- query operand (same as the direct kernel) -----------------------------------
-    half8 qh[KS];
-    float qscale;
-    {
-        float qf[KS][8];
-        float mx = 0.0f;
-        const bool live = hd < p.G;
-        const uint16_t* qsrc = reinterpret_cast<const uint16_t*>(p.q_rot) +
-                               (int64_t(seq) * p.H_Q + h * p.G + (live ? hd : 0)) * D + g * (D / 4);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const uint4v raw = *reinterpret_cast<const uint4v*>(qsrc + 8 * ks);
-            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                qf[ks][2 * i] = live ? load_elem<DT>(uint16_t(w[i] & 0xffffu)) : 0.0f;
-                qf[ks][2 * i + 1] = live ? load_elem<DT>(uint16_t(w[i] >> 16)) : 0.0f;
-                mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(qf[ks][2 * i]), __builtin_fabsf(qf[ks][2 * i + 1])));
-            }
-        }
-        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 16));
-        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 32));
-        int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
-        if (ex < -100 || ex > 100) ex = 0;
-        const float down = bits_to_float(uint32_t(127 - ex) << 23);
-        qscale = p.scale_log2e * bits_to_float(uint32_t(127 + ex) << 23);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) qh[ks][e] = _Float16(qf[ks][e] * down);
-    }
-
     // ---- page ids of the split in registers (see the direct kernel) ---------------------
     int pv[PVR];
     const int split_p0 = begin >> BSL;
@@ -722,6 +765,8 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         }
         return v;
     };
+    // the table is filled while the page ids are on their way
+    fill_byte_table(lut, cent_mine, h, 8, lane);
 
     // ---- copy plan: chunk c = tid + 512 k of the tile, k = 0..4 (the last round only
     // for the first 128 threads) -----------------------------------------------------------
@@ -761,6 +806,88 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         for (int k = 0; k < ROUNDS; ++k)
             if (k < 4 || has_round4) *reinterpret_cast<uint4v*>(dst + dst_off[k]) = stage_reg[k];
     };
+
+    FQ_MARK(2);
+    // the loads of the first tile fly while the query is prepared
+    issue_loads(begin);
+    FQ_MARK(3);
+
+    // ---- query operand ------------------------------------------------------------------
+    // With a rotation matrix the workgroup first rotates all query heads of its sequence:
+    // wavefront h produces columns 16h .. 16h+15 of q_rot = (q @ R.T) on the float32 MFMA,
+    // rounded to the query dtype as the reference rounds it, and the heads are exchanged
+    // through LDS (the tile slots are not in use yet).
+    half8 qh[KS];
+    float qscale;
+    {
+        float qf[KS][8];
+        float mx = 0.0f;
+        const bool live = hd < p.G;
+        if (p.rotation != nullptr) {
+            float* qs = reinterpret_cast<float*>(slots);   // (H_Q, D) float32, H_Q <= 128
+            for (int rb = 0; 16 * rb < p.H_Q; ++rb) {
+                const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
+                float a[KS][8];
+#pragma unroll
+                for (int j = 0; j < KS; ++j) {
+                    const uint4v raw = rb < 2 ? q_pre[rb & 1][j]
+                                              : *reinterpret_cast<const uint4v*>(qseq + row * D + 32 * j + 8 * g);
+                    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        a[j][2 * i] = load_elem<DT>(uint16_t(w[i] & 0xffffu));
+                        a[j][2 * i + 1] = load_elem<DT>(uint16_t(w[i] >> 16));
+                    }
+                }
+#ifdef FQ_DBG_NO_ROT_MFMA
+                const float4v acc = {a[0][0] + rot_b[0][0], a[1][1] + rot_b[1][1], a[2][2], a[3][3]};
+#else
+                const float4v acc = rotate_block<D>(a, rot_b);
+#endif
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int head = 16 * rb + 4 * g + i;
+                    if (head < p.H_Q) qs[head * D + 16 * h + n] = load_elem<DT>(store_elem<DT>(acc[i]));
+                }
+            }
+            FQ_MARK(4);
+            __syncthreads();
+            FQ_MARK(5);
+            const float* src = qs + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    qf[ks][e] = live ? src[8 * ks + e] : 0.0f;
+                    mx = __builtin_fmaxf(mx, __builtin_fabsf(qf[ks][e]));
+                }
+            FQ_MARK(6);
+            __syncthreads();   // the slots are about to receive tiles
+        } else {
+            const uint16_t* qsrc = qseq + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const uint4v raw = *reinterpret_cast<const uint4v*>(qsrc + 8 * ks);
+                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    qf[ks][2 * i] = live ? load_elem<DT>(uint16_t(w[i] & 0xffffu)) : 0.0f;
+                    qf[ks][2 * i + 1] = live ? load_elem<DT>(uint16_t(w[i] >> 16)) : 0.0f;
+                    mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(qf[ks][2 * i]), __builtin_fabsf(qf[ks][2 * i + 1])));
+                }
+            }
+        }
+        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 16));
+        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 32));
+        int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+        if (ex < -100 || ex > 100) ex = 0;
+        const float down = bits_to_float(uint32_t(127 - ex) << 23);
+        qscale = p.scale_log2e * bits_to_float(uint32_t(127 + ex) << 23);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qh[ks][e] = _Float16(qf[ks][e] * down);
+    }
 
     // ---- lane-constant LDS read offsets (inside a tile slot) -------------------------------
     int k_rd[2];                // K operand of block b: 16 bytes of row n, quarter g
@@ -928,8 +1055,8 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     {
         const int last_t0 = begin + ((end - begin - 1) & ~31);
         auto clamp_t0 = [&](int t) { return t < last_t0 ? t : last_t0; };
-        issue_loads(begin);
-        write_slot(0);
+        FQ_MARK(7);
+        write_slot(0);                            // tile 0, loaded before the query was prepared
         issue_loads(clamp_t0(begin + 32));
         int i = 0;
         for (int t0 = begin; t0 < (FQ_STAGED_DEBUG_MODE == 3 ? begin : end); t0 += 32, ++i) {
@@ -946,6 +1073,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         }
     }
 
+    FQ_MARK(8);
     // ---- publish the partial of this split (as in the direct kernel) -----------------------------
 #pragma unroll
     for (int mask = GP; mask < 64; mask <<= 1) lsum += xor_shuffle(lsum, mask);
@@ -977,52 +1105,12 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             }
         }
     }
-}
-
-// ---------------------------------------------------------------------------------------
-// Head rotations: rows of D elements times the D x D rotation, float32 throughout, on the
-// float32 MFMA (v_mfma_f32_16x16x4_f32), so that no splitting of the matrix is needed and
-// the result matches a float32 matmul to rounding.  A workgroup (4 wavefronts) owns 16
-// rows; wavefront w produces the 16-column blocks w, w + 4, ...
-//
-// The contraction index is permuted so that operands load as contiguous runs: MFMA step
-// (j, e) with lane group g uses k = 32 j + 8 g + e, hence lane (m, g) holds the 8-element
-// runs k = 32 j + 8 g .. + 7 of row m (A side) and of the matrix (B side).
-// ---------------------------------------------------------------------------------------
-
-constexpr int kRotRows = 16;
-
-// B operand values of one 16-column block.  TRANSPOSED: out = x @ R.T (B[k][n] = R[col+n][k],
-// contiguous in k); otherwise out = x @ R (B[k][n] = R[k][col+n], 16 lanes contiguous in n).
-template <int D, bool TRANSPOSED>
-__device__ __forceinline__ void load_rotation_block(const float* __restrict__ R, int col, int n, int g,
-                                                    float (&b)[D / 32][8]) {
-#pragma unroll
-    for (int j = 0; j < D / 32; ++j) {
-        if (TRANSPOSED) {
-            const float4v* src = reinterpret_cast<const float4v*>(R + int64_t(col + n) * D + 32 * j + 8 * g);
-            const float4v lo = src[0], hi = src[1];
-            b[j][0] = lo.x; b[j][1] = lo.y; b[j][2] = lo.z; b[j][3] = lo.w;
-            b[j][4] = hi.x; b[j][5] = hi.y; b[j][6] = hi.z; b[j][7] = hi.w;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) b[j][e] = R[int64_t(32 * j + 8 * g + e) * D + col + n];
-        }
-    }
-}
-
-template <int D>
-__device__ __forceinline__ float4v rotate_block(const float (&a)[D / 32][8], const float (&b)[D / 32][8]) {
-    // four independent partial sums: a single accumulator would chain D/4 dependent MFMAs
-    float4v acc[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] = float4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int j = 0; j < D / 32; ++j)
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-            acc[e & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j][e], b[j][e], acc[e & 3], 0, 0, 0);
-    return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+#ifdef FQ_DBG_TIMING
+    FQ_MARK(9);
+    if (threadIdx.x == 0 && blockIdx.x == 3 && blockIdx.y == 5)
+        printf("marks(100MHz ticks): start->lut %llu ->split %llu ->issue0 %llu ->rot %llu ->bar %llu ->qf %llu ->loop %llu ->tiles %llu ->end %llu\n",
+               tmark[1]-tmark[0], tmark[2]-tmark[1], tmark[3]-tmark[2], tmark[4]-tmark[3], tmark[5]-tmark[4], tmark[6]-tmark[5], tmark[7]-tmark[6], tmark[8]-tmark[7], tmark[9]-tmark[8]);
+#endif
 }
 
 // q_rot[row, j] = sum_k q[row, k] * R[j, k], rounded to the query dtype
@@ -1175,6 +1263,11 @@ int launch_with_lds(K kernel, const DecodeParams& p, dim3 grid, dim3 block, size
     return fq_host::check_launch();
 }
 
+// The staged kernel covers 8 KV heads of dimension 128 sharing one codebook.
+inline bool staged_applies(int D, int H_KV, bool two_tables) {
+    return D == 128 && H_KV == 8 && !two_tables && !fq_host::force_direct_decode();
+}
+
 template <typename K>
 int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream) {
     // dynamic part only; the 64 KB table is static
@@ -1189,7 +1282,7 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
     const int64_t chunk = (((max_ctx + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
     const bool wide = chunk / BS > 64;   // begin is a multiple of 64 tokens, hence page aligned
 
-    if (D == 128 && p.H_KV == 8 && !p.two_tables && !fq_host::force_direct_decode()) {
+    if (staged_applies(D, p.H_KV, p.two_tables != 0)) {
 #define FQ_STAGED_GP(BSL, GPV)                                                                      \
     return wide ? launch_staged(paged_decode_staged_kernel<BSL, GPV, DT, 4>, p, S, stream)         \
                 : launch_staged(paged_decode_staged_kernel<BSL, GPV, DT, 1>, p, S, stream)
@@ -1336,24 +1429,27 @@ extern "C" int fq_rotate_query(const void* q, const float* rotation, void* q_rot
                            : launch_rotate<FQ_BF16>(q, rotation, q_rot, int(num_seqs), H_Q, D, s);
 }
 
-extern "C" int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache, const int32_t* block_table,
-                                   const int32_t* seq_lens, const float* centroids_k, const float* centroids_v,
-                                   float* partial_acc, float* partial_m, float* partial_l, int num_seqs, int H_Q,
-                                   int H_KV, int D, int block_size, int max_blocks_per_seq, int64_t num_blocks,
-                                   float sm_scale, int dtype, int num_splits, void* stream) {
-    using namespace fq;
+namespace fq {
+// Partials of the split-K decode.  `rotation` may be non-NULL only when the staged kernel
+// applies: it then rotates the (un-rotated) query itself.
+int decode_partials(const void* q, const float* rotation, const uint8_t* kv_cache, const int32_t* block_table,
+                    const int32_t* seq_lens, const float* centroids_k, const float* centroids_v, float* partial_acc,
+                    float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D, int block_size,
+                    int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype, int num_splits,
+                    void* stream) {
     const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
                                        num_splits);
     if (bad != FQ_OK) return bad;
     if (num_splits < fq_paged_decode_min_splits(block_size, max_blocks_per_seq)) return FQ_ERR_BAD_SHAPE;
     if (num_seqs == 0) return FQ_OK;
-    if (!q_rot || !kv_cache || !block_table || !seq_lens || !centroids_k || !centroids_v || !partial_acc ||
+    if (!q || !kv_cache || !block_table || !seq_lens || !centroids_k || !centroids_v || !partial_acc ||
         !partial_m || !partial_l)
         return FQ_ERR_NULL_POINTER;
-    if (!fq_host::aligned(q_rot, 16) || !fq_host::aligned(kv_cache, 16) || !fq_host::aligned(partial_acc, 16))
+    if (!fq_host::aligned(q, 16) || !fq_host::aligned(kv_cache, 16) || !fq_host::aligned(partial_acc, 16) ||
+        (rotation && !fq_host::aligned(rotation, 16)))
         return FQ_ERR_MISALIGNED;
     DecodeParams p;
-    p.q_rot = q_rot; p.cache = kv_cache; p.block_table = block_table; p.seq_lens = seq_lens;
+    p.q_rot = q; p.rotation = rotation; p.cache = kv_cache; p.block_table = block_table; p.seq_lens = seq_lens;
     p.centroids_k = centroids_k; p.centroids_v = centroids_v;
     p.part_acc = partial_acc; p.part_m = partial_m; p.part_l = partial_l;
     p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.max_blocks = max_blocks_per_seq;
@@ -1372,6 +1468,17 @@ extern "C" int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache, c
         default: return FQ_ERR_UNSUPPORTED_DIM;
     }
 #undef FQ_DECODE_D
+}
+}  // namespace fq
+
+extern "C" int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache, const int32_t* block_table,
+                                   const int32_t* seq_lens, const float* centroids_k, const float* centroids_v,
+                                   float* partial_acc, float* partial_m, float* partial_l, int num_seqs, int H_Q,
+                                   int H_KV, int D, int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                                   float sm_scale, int dtype, int num_splits, void* stream) {
+    return fq::decode_partials(q_rot, nullptr, kv_cache, block_table, seq_lens, centroids_k, centroids_v, partial_acc,
+                               partial_m, partial_l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq,
+                               num_blocks, sm_scale, dtype, num_splits, stream);
 }
 
 extern "C" int fq_split_k_reduce(const float* partial_acc, const float* partial_m, const float* partial_l,
@@ -1410,15 +1517,20 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     float* acc = reinterpret_cast<float*>(ws + w.acc);
     float* m = reinterpret_cast<float*>(ws + w.m);
     float* l = reinterpret_cast<float*>(ws + w.l);
-    const void* q_rot = q;
+    const void* q_in = q;
+    const float* fused_rotation = nullptr;
     if (rotation) {
-        const int st = fq_rotate_query(q, rotation, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
-        if (st != FQ_OK) return st;
-        q_rot = ws + w.qrot;
+        if (centroids_k && staged_applies(D, H_KV, centroids_k != centroids_v)) {
+            fused_rotation = rotation;       // the staged kernel rotates the query in its prologue
+        } else {
+            const int st = fq_rotate_query(q, rotation, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
+            if (st != FQ_OK) return st;
+            q_in = ws + w.qrot;
+        }
     }
-    int st = fq_paged_tq4_decode(q_rot, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m, l,
-                                 num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
-                                 num_splits, stream);
+    int st = decode_partials(q_in, fused_rotation, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m,
+                             l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
+                             num_splits, stream);
     if (st != FQ_OK) return st;
     return fq_split_k_reduce(acc, m, l, rotation, out, num_seqs, H_Q, D, dtype, num_splits, stream);
 }
