@@ -24,6 +24,26 @@ void* current_stream(const at::Tensor& like) {
 
 namespace {
 
+// A (D, D) float32 rotation on the right device as the C ABI wants it: row-major, or
+// column-major when the transpose is the contiguous one (no copy in either case).
+struct RotationArg {
+    at::Tensor keep;
+    const float* ptr = nullptr;
+    int col_major = 0;
+};
+RotationArg rotation_arg(const at::Tensor& rotation, const c10::Device& dev, int64_t D) {
+    require(rotation.dim() == 2 && rotation.size(0) == D && rotation.size(1) == D && rotation.scalar_type() == at::kFloat,
+            "rotation must be float32 of shape (D, D)");
+    RotationArg r;
+    r.keep = rotation.to(dev);
+    if (!r.keep.is_contiguous()) {
+        if (r.keep.t().is_contiguous()) r.col_major = 1;
+        else r.keep = r.keep.contiguous();
+    }
+    r.ptr = r.keep.data_ptr<float>();
+    return r;
+}
+
 using OptPair = std::optional<std::tuple<at::Tensor, at::Tensor>>;
 
 std::tuple<at::Tensor, at::Tensor> tq4_compress(const at::Tensor& x, const at::Tensor& rot_T_even,
@@ -128,13 +148,8 @@ at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache,
     const bool same = centroids_v.is_same(centroids_k) ||
                       (centroids_v.device() == centroids_k.device() && centroids_v.data_ptr() == centroids_k.data_ptr());
     const at::Tensor cv = same ? ck : centroids_v.to(q.device()).contiguous();
-    at::Tensor rot;
-    if (rotation.has_value()) {
-        require(rotation->dim() == 2 && rotation->size(0) == D && rotation->size(1) == D &&
-                    rotation->scalar_type() == at::kFloat,
-                "rotation must be float32 of shape (D, D)");
-        rot = rotation->to(q.device()).contiguous();
-    }
+    RotationArg rot;
+    if (rotation.has_value()) rot = rotation_arg(*rotation, q.device(), D);
     at::Tensor result;
     if (out.has_value()) {
         result = *out;
@@ -150,7 +165,7 @@ at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache,
     at::Tensor ws = at::empty({int64_t(ws_bytes)}, q.options().dtype(at::kByte));
     const int st = fq_split_k_paged_decode(
         qc.data_ptr(), kv_cache.data_ptr<uint8_t>(), bt.data_ptr<int32_t>(), sl.data_ptr<int32_t>(),
-        ck.data_ptr<float>(), cv.data_ptr<float>(), rot.defined() ? rot.data_ptr<float>() : nullptr, result.data_ptr(),
+        ck.data_ptr<float>(), cv.data_ptr<float>(), rot.ptr, rot.col_major, result.data_ptr(),
         S, HQ, int(num_kv_heads), D, int(block_size), max_blocks, kv_cache.size(0), float(scale),
         fqbind::dtype_code(q.scalar_type(), "split_k_paged_decode"), int(num_splits), ws.data_ptr(), ws_bytes,
         fqbind::current_stream(q));
@@ -162,14 +177,11 @@ at::Tensor rotate_query(const at::Tensor& q, const at::Tensor& rotation) {
     fqbind::require_gpu(q, "q");
     require(q.dim() == 3 && (q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16),
             "q must be float16/bfloat16 of shape (num_seqs, H_Q, D)");
-    require(rotation.dim() == 2 && rotation.size(0) == q.size(2) && rotation.size(1) == q.size(2) &&
-                rotation.scalar_type() == at::kFloat,
-            "rotation must be float32 of shape (D, D)");
     c10::DeviceGuard guard(q.device());
     const at::Tensor qc = q.contiguous();
-    const at::Tensor rot = rotation.to(q.device()).contiguous();
+    const RotationArg rot = rotation_arg(rotation, q.device(), q.size(2));
     at::Tensor out = at::empty_like(qc);
-    const int st = fq_rotate_query(qc.data_ptr(), rot.data_ptr<float>(), out.data_ptr(), q.size(0), int(q.size(1)),
+    const int st = fq_rotate_query(qc.data_ptr(), rot.ptr, rot.col_major, out.data_ptr(), q.size(0), int(q.size(1)),
                                    int(q.size(2)), fqbind::dtype_code(q.scalar_type(), "rotate_query"),
                                    fqbind::current_stream(q));
     fqbind::raise_on_error(st, "rotate_query");
@@ -232,11 +244,11 @@ at::Tensor split_k_reduce(const at::Tensor& acc, const at::Tensor& m, const at::
                 l.scalar_type() == at::kFloat && m.numel() == acc.numel() / acc.size(3) && l.numel() == m.numel(),
             "partials must be contiguous float32 GPU tensors (S, H_Q, splits, D), (S, H_Q, splits) x2");
     c10::DeviceGuard guard(acc.device());
-    at::Tensor rot;
-    if (rotation.has_value()) rot = rotation->to(acc.device()).contiguous();
+    RotationArg rot;
+    if (rotation.has_value()) rot = rotation_arg(*rotation, acc.device(), acc.size(3));
     at::Tensor out = at::empty({acc.size(0), acc.size(1), acc.size(3)}, acc.options().dtype(dtype));
     const int st = fq_split_k_reduce(acc.data_ptr<float>(), m.data_ptr<float>(), l.data_ptr<float>(),
-                                     rot.defined() ? rot.data_ptr<float>() : nullptr, out.data_ptr(), int(acc.size(0)),
+                                     rot.ptr, rot.col_major, out.data_ptr(), int(acc.size(0)),
                                      int(acc.size(1)), int(acc.size(3)), fqbind::dtype_code(dtype, "split_k_reduce"),
                                      int(acc.size(2)), fqbind::current_stream(acc));
     fqbind::raise_on_error(st, "split_k_reduce");

@@ -44,6 +44,9 @@
 //            coordinate of two consecutive tokens: again one lookup per byte.
 
 #include <cstdlib>
+#include <map>
+#include <mutex>
+#include <utility>
 
 #include "fq_common.hpp"
 
@@ -61,6 +64,8 @@ namespace fq_host {
 // FQ_DECODE_DIRECT=1 in the environment routes every shape to the direct kernel
 // (both kernels are kept tested).
 bool force_direct_decode();
+// Raises the dynamic-LDS limit of a kernel function once per (function, device); later calls are a lookup.
+bool lds_limit_raised(const void* kernel, size_t bytes);
 }
 
 namespace fq {
@@ -72,6 +77,7 @@ constexpr float kHalfMax = 65504.0f;
 
 struct DecodeParams {
     const void* q_rot;          // (S, H_Q, D) query dtype: rotated, or un-rotated when `rotation` is set
+    int rot_col_major;          // layout of `rotation` / of the matrix given to the side kernels
     const float* rotation;      // staged kernel only: rotate the query in the prologue (NULL: already rotated)
     const uint8_t* cache;       // (num_blocks, BS, H_KV*(D+8))
     const int32_t* block_table; // (S, max_blocks)
@@ -193,6 +199,17 @@ __device__ __forceinline__ void load_rotation_block(const float* __restrict__ R,
             for (int e = 0; e < 8; ++e) b[j][e] = R[int64_t(32 * j + 8 * g + e) * D + col + n];
         }
     }
+}
+
+// Rotation matrix given either row-major (element (i, j) at i*D + j) or column-major
+// (at i + j*D, i.e. the transpose is the contiguous one, which is what a QR factor
+// moved to the GPU looks like).  `x_times_Rt` selects out = x @ R.T, else out = x @ R.
+template <int D>
+__device__ __forceinline__ void load_rotation_any(const float* __restrict__ R, bool col_major, bool x_times_Rt,
+                                                  int col, int n, int g, float (&b)[D / 32][8]) {
+    // x @ R.T on a column-major R reads the same addresses as x @ R on a row-major one
+    if (x_times_Rt != col_major) load_rotation_block<D, true>(R, col, n, g, b);
+    else load_rotation_block<D, false>(R, col, n, g, b);
 }
 
 template <int D>
@@ -714,7 +731,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     float rot_b[4][8];
     uint4v q_pre[2][4];
     if (p.rotation != nullptr) {
-        load_rotation_block<128, true>(p.rotation, 16 * h, n, g, rot_b);
+        load_rotation_any<128>(p.rotation, p.rot_col_major != 0, true, 16 * h, n, g, rot_b);
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
@@ -1117,7 +1134,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
 // (src/flashquant/kernels/paged_decode.py:113).  rows = num_seqs * H_Q.
 template <int D, int DT>
 __global__ __launch_bounds__(256) void rotate_q_kernel(const uint16_t* __restrict__ q, const float* __restrict__ R,
-                                                       uint16_t* __restrict__ q_rot, int64_t rows) {
+                                                       uint16_t* __restrict__ q_rot, int64_t rows, int col_major) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int64_t row0 = int64_t(blockIdx.x) * kRotRows;
@@ -1135,7 +1152,7 @@ __global__ __launch_bounds__(256) void rotate_q_kernel(const uint16_t* __restric
     }
     for (int cb = wave; cb < D / 16; cb += 4) {
         float b[D / 32][8];
-        load_rotation_block<D, true>(R, 16 * cb, n, g, b);
+        load_rotation_any<D>(R, col_major != 0, true, 16 * cb, n, g, b);
         const float4v acc = rotate_block<D>(a, b);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -1155,7 +1172,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
                                                             const float* __restrict__ part_m,
                                                             const float* __restrict__ part_l,
                                                             const float* __restrict__ R, uint16_t* __restrict__ out,
-                                                            int64_t rows, int NS) {
+                                                            int64_t rows, int NS, int col_major) {
     __shared__ float os[kRotRows][D + 4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
@@ -1224,7 +1241,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
         for (int e = 0; e < 8; ++e) a[j][e] = os[n][32 * j + 8 * g + e];
     for (int cb = wave; cb < D / 16; cb += 4) {
         float b[D / 32][8];
-        load_rotation_block<D, false>(R, 16 * cb, n, g, b);
+        load_rotation_any<D>(R, col_major != 0, false, 16 * cb, n, g, b);
         const float4v acc = rotate_block<D>(a, b);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -1254,11 +1271,7 @@ inline WorkspaceLayout workspace_layout(int S, int H_Q, int D, int NS) {
 // allowed per kernel function first.
 template <typename K>
 int launch_with_lds(K kernel, const DecodeParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
-    if (lds > 32768 &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
-        fq_host::note_hip_error(hipGetLastError());
-        return FQ_ERR_LAUNCH;
-    }
+    if (lds > 32768 && !fq_host::lds_limit_raised(reinterpret_cast<const void*>(kernel), lds)) return FQ_ERR_LAUNCH;
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
     return fq_host::check_launch();
 }
@@ -1324,29 +1337,29 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
 }
 
 template <int DT>
-int launch_rotate(const void* q, const float* R, void* q_rot, int S, int H_Q, int D, hipStream_t stream) {
+int launch_rotate(const void* q, const float* R, int col_major, void* q_rot, int S, int H_Q, int D, hipStream_t stream) {
     const int64_t rows = int64_t(S) * H_Q;
     const dim3 grid(unsigned((rows + kRotRows - 1) / kRotRows)), block(256);
     const uint16_t* src = reinterpret_cast<const uint16_t*>(q);
     uint16_t* dst = reinterpret_cast<uint16_t*>(q_rot);
     switch (D) {
-        case 64: hipLaunchKernelGGL((rotate_q_kernel<64, DT>), grid, block, 0, stream, src, R, dst, rows); break;
-        case 128: hipLaunchKernelGGL((rotate_q_kernel<128, DT>), grid, block, 0, stream, src, R, dst, rows); break;
-        default: hipLaunchKernelGGL((rotate_q_kernel<256, DT>), grid, block, 0, stream, src, R, dst, rows); break;
+        case 64: hipLaunchKernelGGL((rotate_q_kernel<64, DT>), grid, block, 0, stream, src, R, dst, rows, col_major); break;
+        case 128: hipLaunchKernelGGL((rotate_q_kernel<128, DT>), grid, block, 0, stream, src, R, dst, rows, col_major); break;
+        default: hipLaunchKernelGGL((rotate_q_kernel<256, DT>), grid, block, 0, stream, src, R, dst, rows, col_major); break;
     }
     return fq_host::check_launch();
 }
 
 template <int DT>
-int launch_reduce(const float* acc, const float* m, const float* l, const float* R, void* out, int S, int H_Q,
+int launch_reduce(const float* acc, const float* m, const float* l, const float* R, int col_major, void* out, int S, int H_Q,
                   int D, int NS, hipStream_t stream) {
     const int64_t rows = int64_t(S) * H_Q;
     const dim3 grid(unsigned((rows + kRotRows - 1) / kRotRows)), block(256);
     uint16_t* dst = reinterpret_cast<uint16_t*>(out);
     switch (D) {
-        case 64: hipLaunchKernelGGL((reduce_rotate_kernel<64, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS); break;
-        case 128: hipLaunchKernelGGL((reduce_rotate_kernel<128, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS); break;
-        default: hipLaunchKernelGGL((reduce_rotate_kernel<256, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS); break;
+        case 64: hipLaunchKernelGGL((reduce_rotate_kernel<64, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major); break;
+        case 128: hipLaunchKernelGGL((reduce_rotate_kernel<128, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major); break;
+        default: hipLaunchKernelGGL((reduce_rotate_kernel<256, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major); break;
     }
     return fq_host::check_launch();
 }
@@ -1370,6 +1383,21 @@ inline int check_decode_shape(int num_seqs, int H_Q, int H_KV, int D, int block_
 
 namespace fq_host {
 int device_cu_count();
+bool lds_limit_raised(const void* kernel, size_t bytes) {
+    static std::mutex mu;
+    static std::map<std::pair<const void*, int>, size_t> done;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = done.find({kernel, dev});
+    if (it != done.end() && it->second >= bytes) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes)) != hipSuccess) {
+        note_hip_error(hipGetLastError());
+        return false;
+    }
+    done[{kernel, dev}] = bytes;
+    return true;
+}
 bool force_direct_decode() {
     const char* v = getenv("FQ_DECODE_DIRECT");
     return v && v[0] == '1';
@@ -1414,7 +1442,7 @@ extern "C" size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_K
     return fq::workspace_layout(num_seqs, H_Q, D, num_splits).total;
 }
 
-extern "C" int fq_rotate_query(const void* q, const float* rotation, void* q_rot, int64_t num_seqs, int H_Q,
+extern "C" int fq_rotate_query(const void* q, const float* rotation, int rotation_col_major, void* q_rot, int64_t num_seqs, int H_Q,
                                int D, int dtype, void* stream) {
     using namespace fq;
     if (num_seqs < 0 || num_seqs > 65535 || H_Q <= 0) return FQ_ERR_BAD_SHAPE;
@@ -1425,14 +1453,14 @@ extern "C" int fq_rotate_query(const void* q, const float* rotation, void* q_rot
     if (!fq_host::aligned(rotation, 16) || !fq_host::aligned(q, 16) || !fq_host::aligned(q_rot, 2))
         return FQ_ERR_MISALIGNED;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return dtype == FQ_F16 ? launch_rotate<FQ_F16>(q, rotation, q_rot, int(num_seqs), H_Q, D, s)
-                           : launch_rotate<FQ_BF16>(q, rotation, q_rot, int(num_seqs), H_Q, D, s);
+    return dtype == FQ_F16 ? launch_rotate<FQ_F16>(q, rotation, rotation_col_major, q_rot, int(num_seqs), H_Q, D, s)
+                           : launch_rotate<FQ_BF16>(q, rotation, rotation_col_major, q_rot, int(num_seqs), H_Q, D, s);
 }
 
 namespace fq {
 // Partials of the split-K decode.  `rotation` may be non-NULL only when the staged kernel
 // applies: it then rotates the (un-rotated) query itself.
-int decode_partials(const void* q, const float* rotation, const uint8_t* kv_cache, const int32_t* block_table,
+int decode_partials(const void* q, const float* rotation, int rotation_col_major, const uint8_t* kv_cache, const int32_t* block_table,
                     const int32_t* seq_lens, const float* centroids_k, const float* centroids_v, float* partial_acc,
                     float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D, int block_size,
                     int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype, int num_splits,
@@ -1449,7 +1477,7 @@ int decode_partials(const void* q, const float* rotation, const uint8_t* kv_cach
         (rotation && !fq_host::aligned(rotation, 16)))
         return FQ_ERR_MISALIGNED;
     DecodeParams p;
-    p.q_rot = q; p.rotation = rotation; p.cache = kv_cache; p.block_table = block_table; p.seq_lens = seq_lens;
+    p.q_rot = q; p.rotation = rotation; p.rot_col_major = rotation_col_major; p.cache = kv_cache; p.block_table = block_table; p.seq_lens = seq_lens;
     p.centroids_k = centroids_k; p.centroids_v = centroids_v;
     p.part_acc = partial_acc; p.part_m = partial_m; p.part_l = partial_l;
     p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.max_blocks = max_blocks_per_seq;
@@ -1476,13 +1504,13 @@ extern "C" int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache, c
                                    float* partial_acc, float* partial_m, float* partial_l, int num_seqs, int H_Q,
                                    int H_KV, int D, int block_size, int max_blocks_per_seq, int64_t num_blocks,
                                    float sm_scale, int dtype, int num_splits, void* stream) {
-    return fq::decode_partials(q_rot, nullptr, kv_cache, block_table, seq_lens, centroids_k, centroids_v, partial_acc,
+    return fq::decode_partials(q_rot, nullptr, 0, kv_cache, block_table, seq_lens, centroids_k, centroids_v, partial_acc,
                                partial_m, partial_l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq,
                                num_blocks, sm_scale, dtype, num_splits, stream);
 }
 
 extern "C" int fq_split_k_reduce(const float* partial_acc, const float* partial_m, const float* partial_l,
-                                 const float* rotation, void* out, int num_seqs, int H_Q, int D, int dtype,
+                                 const float* rotation, int rotation_col_major, void* out, int num_seqs, int H_Q, int D, int dtype,
                                  int num_splits, void* stream) {
     using namespace fq;
     if (num_seqs < 0 || num_seqs > 65535 || H_Q <= 0 || num_splits < 1) return FQ_ERR_BAD_SHAPE;
@@ -1492,13 +1520,13 @@ extern "C" int fq_split_k_reduce(const float* partial_acc, const float* partial_
     if (!partial_acc || !partial_m || !partial_l || !out) return FQ_ERR_NULL_POINTER;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dtype == FQ_F16
-               ? launch_reduce<FQ_F16>(partial_acc, partial_m, partial_l, rotation, out, num_seqs, H_Q, D, num_splits, s)
-               : launch_reduce<FQ_BF16>(partial_acc, partial_m, partial_l, rotation, out, num_seqs, H_Q, D, num_splits, s);
+               ? launch_reduce<FQ_F16>(partial_acc, partial_m, partial_l, rotation, rotation_col_major, out, num_seqs, H_Q, D, num_splits, s)
+               : launch_reduce<FQ_BF16>(partial_acc, partial_m, partial_l, rotation, rotation_col_major, out, num_seqs, H_Q, D, num_splits, s);
 }
 
 extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
                                        const int32_t* seq_lens, const float* centroids_k,
-                                       const float* centroids_v, const float* rotation, void* out,
+                                       const float* centroids_v, const float* rotation, int rotation_col_major, void* out,
                                        int num_seqs, int H_Q, int H_KV, int D, int block_size,
                                        int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype,
                                        int num_splits, void* workspace, size_t workspace_bytes, void* stream) {
@@ -1523,14 +1551,14 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
         if (centroids_k && staged_applies(D, H_KV, centroids_k != centroids_v)) {
             fused_rotation = rotation;       // the staged kernel rotates the query in its prologue
         } else {
-            const int st = fq_rotate_query(q, rotation, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
+            const int st = fq_rotate_query(q, rotation, rotation_col_major, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
             if (st != FQ_OK) return st;
             q_in = ws + w.qrot;
         }
     }
-    int st = decode_partials(q_in, fused_rotation, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m,
+    int st = decode_partials(q_in, fused_rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m,
                              l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
                              num_splits, stream);
     if (st != FQ_OK) return st;
-    return fq_split_k_reduce(acc, m, l, rotation, out, num_seqs, H_Q, D, dtype, num_splits, stream);
+    return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_splits, stream);
 }

@@ -101,6 +101,8 @@ int fq_tq4_decompress(const uint8_t* packed, const float* norms,
  *   centroids_k, centroids_v  (16,) float32
  *   rotation     (D, D) float32, or NULL: q is taken as already rotated and
  *                out is left in rotated space
+ *   rotation_col_major  0: element (i, j) at i*D + j; 1: at i + j*D (the layout
+ *                of a LAPACK QR factor, whose transpose is the contiguous one)
  *   out          (S, H_Q, D) same dtype as q
  *   num_splits   >= 1, or 0 to let the library choose
  *   workspace    fq_paged_decode_workspace_bytes(...) bytes, 256-byte aligned
@@ -110,7 +112,7 @@ int fq_tq4_decompress(const uint8_t* packed, const float* norms,
 int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
                             const int32_t* block_table, const int32_t* seq_lens,
                             const float* centroids_k, const float* centroids_v,
-                            const float* rotation, void* out,
+                            const float* rotation, int rotation_col_major, void* out,
                             int num_seqs, int H_Q, int H_KV, int D,
                             int block_size, int max_blocks_per_seq,
                             int64_t num_blocks, float sm_scale, int dtype,
@@ -134,7 +136,7 @@ int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
  *                      dtype; if rotation is not NULL the rounded value is multiplied by
  *                      rotation in float32 and rounded again (paged_decode.py:123).
  */
-int fq_rotate_query(const void* q, const float* rotation, void* q_rot,
+int fq_rotate_query(const void* q, const float* rotation, int rotation_col_major, void* q_rot,
                     int64_t num_seqs, int H_Q, int D, int dtype, void* stream);
 
 int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache,
@@ -146,7 +148,8 @@ int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache,
                         float sm_scale, int dtype, int num_splits, void* stream);
 
 int fq_split_k_reduce(const float* partial_acc, const float* partial_m,
-                      const float* partial_l, const float* rotation, void* out,
+                      const float* partial_l, const float* rotation,
+                      int rotation_col_major, void* out,
                       int num_seqs, int H_Q, int D, int dtype, int num_splits,
                       void* stream);
 
