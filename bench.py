@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="omit the compress / decompress legs")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain device copy of one cache (142.6 MB read + 142.6 MB written): the "
+                         "reference point for scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this benchmark runs on exactly one GPU (the path has no collectives); use --gpus 1")
@@ -147,13 +150,13 @@ def main():
     warm_ms = time_events(lambda i: step(0), args.steps)
 
     # ---- dominant kernel alone (the split-K decode), cold ----------------------------
-    q_rot = C.rotate_query(q, rot_d)
     parts = (torch.empty(BATCH, H_Q, n_splits, D, device=dev), torch.empty(BATCH, H_Q, n_splits, device=dev),
              torch.empty(BATCH, H_Q, n_splits, device=dev))
 
     def decode_only(i):
         cache, table = caches[i % n_caches]
-        C.paged_tq4_decode_partials(q_rot, cache, table, lens, cent_d, cent_d, H_KV, D, BS, scale, n_splits, parts)
+        # the same launch the step makes: un-rotated query, rotation applied in the kernel's prologue
+        C.paged_tq4_decode_partials(q, cache, table, lens, cent_d, cent_d, H_KV, D, BS, scale, n_splits, parts, rot_d)
 
     for i in range(args.warmup):
         decode_only(i)
@@ -171,6 +174,13 @@ def main():
         "num_splits": n_splits,
         "kv_bytes_per_step": kv_bytes,
     }
+
+    if args.copy_probe:
+        dst = torch.empty_like(caches[0][0])
+        for i in range(4):
+            dst.copy_(caches[i % n_caches][0])
+        torch.cuda.synchronize()
+        del dst
 
     # ---- CPU baseline: the oracle on the host cores, bounded sample ---------------------
     cpu = None
@@ -259,7 +269,9 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a plain copy
+            # (profiles/paged_decode_hbm_traffic_pmc.txt); a measured constant, not read live
+            "traffic": 150.1e6,
             "kernel": "paged_decode_staged_kernel<4,4,bf16,1>",
         },
         "cpu_baseline": cpu,

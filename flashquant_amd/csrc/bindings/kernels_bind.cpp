@@ -193,7 +193,8 @@ using OptTriple = std::optional<std::tuple<at::Tensor, at::Tensor, at::Tensor>>;
 std::tuple<at::Tensor, at::Tensor, at::Tensor> paged_tq4_decode_partials(
     const at::Tensor& q_rot, const at::Tensor& kv_cache, const at::Tensor& block_table, const at::Tensor& seq_lens,
     const at::Tensor& centroids_k, const at::Tensor& centroids_v, int64_t num_kv_heads, int64_t head_dim,
-    int64_t block_size, double sm_scale, int64_t num_splits, const OptTriple& out) {
+    int64_t block_size, double sm_scale, int64_t num_splits, const OptTriple& out,
+    const std::optional<at::Tensor>& rotation) {
     fqbind::require_gpu(q_rot, "q_rot");
     fqbind::require_gpu(kv_cache, "kv_cache");
     require(q_rot.dim() == 3 && q_rot.size(2) == head_dim && q_rot.is_contiguous(), "q_rot must be contiguous (S, H_Q, D)");
@@ -225,8 +226,10 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> paged_tq4_decode_partials(
         m = at::empty({S, HQ, num_splits}, q_rot.options().dtype(at::kFloat));
         l = at::empty({S, HQ, num_splits}, q_rot.options().dtype(at::kFloat));
     }
+    RotationArg rot;
+    if (rotation.has_value()) rot = rotation_arg(*rotation, q_rot.device(), head_dim);
     const int st = fq_paged_tq4_decode(
-        q_rot.data_ptr(), kv_cache.data_ptr<uint8_t>(), block_table.data_ptr<int32_t>(), seq_lens.data_ptr<int32_t>(),
+        q_rot.data_ptr(), rot.ptr, rot.col_major, kv_cache.data_ptr<uint8_t>(), block_table.data_ptr<int32_t>(), seq_lens.data_ptr<int32_t>(),
         centroids_k.data_ptr<float>(), centroids_v.data_ptr<float>(), acc.data_ptr<float>(), m.data_ptr<float>(),
         l.data_ptr<float>(), int(S), int(HQ), int(num_kv_heads), int(head_dim), int(block_size),
         int(block_table.size(1)), kv_cache.size(0), float(sm_scale),
@@ -281,8 +284,11 @@ void bind_kernels(py::module_& m) {
     m.def("paged_tq4_decode_partials", &paged_tq4_decode_partials, py::arg("q_rot"), py::arg("kv_cache"),
           py::arg("block_table"), py::arg("seq_lens"), py::arg("centroids_k"), py::arg("centroids_v"),
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale"),
-          py::arg("num_splits"), py::arg("out") = py::none(),
-          "Split partials (acc, m, l) of the paged decode for a pre-rotated query.");
+          py::arg("num_splits"), py::arg("out") = py::none(), py::arg("rotation") = py::none(),
+          "Split partials (acc, m, l) of the paged decode; the query is pre-rotated unless `rotation` is given "
+          "(accepted only where the kernel rotates the query itself).");
+    m.def("paged_decode_fuses_rotation", &fq_paged_decode_fuses_rotation, py::arg("head_dim"),
+          py::arg("num_kv_heads"), py::arg("shared_codebook"));
     m.def("split_k_reduce", &split_k_reduce, py::arg("partial_acc"), py::arg("partial_m"), py::arg("partial_l"),
           py::arg("rotation"), py::arg("dtype"), "Log-sum-exp combine of split partials, optional post-rotation.");
     m.def("paged_decode_auto_splits", &fq_paged_decode_auto_splits, py::arg("num_seqs"), py::arg("num_kv_heads"),

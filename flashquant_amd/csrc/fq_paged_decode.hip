@@ -1499,14 +1499,20 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
 }
 }  // namespace fq
 
-extern "C" int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache, const int32_t* block_table,
-                                   const int32_t* seq_lens, const float* centroids_k, const float* centroids_v,
-                                   float* partial_acc, float* partial_m, float* partial_l, int num_seqs, int H_Q,
-                                   int H_KV, int D, int block_size, int max_blocks_per_seq, int64_t num_blocks,
-                                   float sm_scale, int dtype, int num_splits, void* stream) {
-    return fq::decode_partials(q_rot, nullptr, 0, kv_cache, block_table, seq_lens, centroids_k, centroids_v, partial_acc,
-                               partial_m, partial_l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq,
-                               num_blocks, sm_scale, dtype, num_splits, stream);
+extern "C" int fq_paged_decode_fuses_rotation(int D, int H_KV, int shared_codebook) {
+    return fq::staged_applies(D, H_KV, shared_codebook == 0) ? 1 : 0;
+}
+
+extern "C" int fq_paged_tq4_decode(const void* q, const float* rotation, int rotation_col_major,
+                                   const uint8_t* kv_cache, const int32_t* block_table, const int32_t* seq_lens,
+                                   const float* centroids_k, const float* centroids_v, float* partial_acc,
+                                   float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D,
+                                   int block_size, int max_blocks_per_seq, int64_t num_blocks, float sm_scale,
+                                   int dtype, int num_splits, void* stream) {
+    if (rotation && !fq::staged_applies(D, H_KV, centroids_k != centroids_v)) return FQ_ERR_BAD_SHAPE;
+    return fq::decode_partials(q, rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k,
+                               centroids_v, partial_acc, partial_m, partial_l, num_seqs, H_Q, H_KV, D, block_size,
+                               max_blocks_per_seq, num_blocks, sm_scale, dtype, num_splits, stream);
 }
 
 extern "C" int fq_split_k_reduce(const float* partial_acc, const float* partial_m, const float* partial_l,

@@ -128,7 +128,11 @@ int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
  *
  * fq_rotate_query:     q_rot = (q @ rotation.T) rounded to dtype
  *                      (src/flashquant/kernels/paged_decode.py:113); q, q_rot (num_seqs, H_Q, D).
- * fq_paged_tq4_decode: q_rot pre-rotated; writes un-normalised float32 partials
+ * fq_paged_tq4_decode: q pre-rotated and rotation NULL, or q un-rotated with the rotation,
+ *                      which the kernel then applies itself: allowed only where
+ *                      fq_paged_decode_fuses_rotation() returns 1 (8 KV heads of dimension
+ *                      128 sharing one codebook), FQ_ERR_BAD_SHAPE elsewhere.
+ *                      Writes un-normalised float32 partials
  *                      partial_acc (num_seqs, H_Q, num_splits, D) and the base-2 running
  *                      maximum / denominator partial_m, partial_l (num_seqs, H_Q, num_splits);
  *                      an empty split has m = -inf.  num_splits >= 1.
@@ -139,7 +143,10 @@ int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
 int fq_rotate_query(const void* q, const float* rotation, int rotation_col_major, void* q_rot,
                     int64_t num_seqs, int H_Q, int D, int dtype, void* stream);
 
-int fq_paged_tq4_decode(const void* q_rot, const uint8_t* kv_cache,
+int fq_paged_decode_fuses_rotation(int D, int H_KV, int shared_codebook);
+
+int fq_paged_tq4_decode(const void* q, const float* rotation, int rotation_col_major,
+                        const uint8_t* kv_cache,
                         const int32_t* block_table, const int32_t* seq_lens,
                         const float* centroids_k, const float* centroids_v,
                         float* partial_acc, float* partial_m, float* partial_l,

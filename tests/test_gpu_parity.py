@@ -200,6 +200,26 @@ def test_paged_decode_rotated_space_and_out_argument():
     assert (out.cpu().float() - want.float()).abs().max() <= 2e-2
 
 
+def test_paged_decode_rotation_layouts_agree():
+    """The rotation is taken row-major or column-major (a QR factor moved to the GPU
+    is column-major) without a copy; both must give the same result."""
+    c, b, r = book(128)
+    q, cache, table, sl = build_paged_case([150, 40], 32, 8)
+    cd = c.to(DEV)
+    args = (q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), cd, cd)
+    row_major = r.contiguous().to(DEV)
+    col_major = r.t().contiguous().t().to(DEV)
+    assert row_major.is_contiguous() and not col_major.is_contiguous()
+    a = K.split_k_paged_decode(*args, row_major, 8, 128, 16)
+    bb = K.split_k_paged_decode(*args, col_major, 8, 128, 16)
+    assert torch.equal(a, bb)
+    qa = load_native().rotate_query(q.to(DEV), row_major)
+    qb = load_native().rotate_query(q.to(DEV), col_major)
+    want = torch.matmul(q.float(), r.T).to(q.dtype)
+    assert torch.equal(qa, qb)
+    assert (qa.cpu().float() - want.float()).abs().max() <= 2 ** -6   # one bf16 step at |q_rot| < 4
+
+
 def test_paged_decode_distinct_value_codebook():
     c, b, r = book(128)
     q, cache, table, sl = build_paged_case([75], 8, 2)
