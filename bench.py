@@ -244,6 +244,36 @@ def main():
             "decompress_pct_hbm_peak": 100.0 * nrows * 324 / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         })
 
+        del y, packed, norms
+        torch.cuda.empty_cache()
+
+        # ---- fused TQ4 prefill (configs[3]): batch 4, 32 query heads over 8, 8192 tokens, causal ----
+        pb, pn = 4, 8192
+        gq3 = torch.Generator(device=dev).manual_seed(1003)
+        q3 = torch.randn(pb, H_Q, pn, D, generator=gq3, device=dev).to(torch.bfloat16)
+        kx = outlier_rows(pb * pn, H_KV, D, 1013, dev)            # (tokens, heads, D)
+        vx = outlier_rows(pb * pn, H_KV, D, 1023, dev)
+        kp3, kn3 = K.tq4_compress(kx, rot_d, bnd_d)
+        vp3, vn3 = K.tq4_compress(vx, rot_d, bnd_d)
+        del kx, vx
+
+        def to_bhnd(t):                                            # (B*N, H, X) -> (B, H, N, X)
+            return t.reshape(pb, pn, H_KV, -1).permute(0, 2, 1, 3).contiguous()
+
+        kp3, kn3, vp3, vn3 = (to_bhnd(t) for t in (kp3, kn3, vp3, vn3))
+        for _ in range(2):
+            K.fused_tq_attention(q3, kp3, kn3, vp3, vn3, cent_d, cent_d, rot_d, sm_scale=scale, is_causal=True)
+        p_ms = time_events(lambda i: K.fused_tq_attention(q3, kp3, kn3, vp3, vn3, cent_d, cent_d, rot_d,
+                                                          sm_scale=scale, is_causal=True), 5)
+        p_flops = 4.0 * pn * pn * D * pb * H_Q / 2.0               # causal half of QK^T and PV
+        extra.update({
+            "prefill_ms": p_ms,
+            "prefill_tflops": p_flops / (p_ms * 1e-3) / 1e12,
+            "prefill_pct_fp16_mfma_peak": 100.0 * p_flops / (p_ms * 1e-3) / 2.5e15,
+            "prefill_tokens_per_s": pb * pn / (p_ms * 1e-3),
+        })
+        del q3, kp3, kn3, vp3, vn3
+
     value = kv_bytes / (step_ms * 1e-3) / 1e9
     line = {
         "metric": "tq4_paged_decode_hbm_gbps",

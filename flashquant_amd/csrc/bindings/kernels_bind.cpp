@@ -173,6 +173,46 @@ at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache,
     return result;
 }
 
+at::Tensor fused_tq_attention(const at::Tensor& q, const at::Tensor& k_packed, const at::Tensor& k_norms,
+                              const at::Tensor& v_packed, const at::Tensor& v_norms, const at::Tensor& centroids_k,
+                              const at::Tensor& centroids_v, const at::Tensor& rotation,
+                              std::optional<double> sm_scale, bool is_causal) {
+    fqbind::require_gpu(q, "q");
+    fqbind::require_gpu(k_packed, "k_packed");
+    fqbind::require_gpu(v_packed, "v_packed");
+    require(q.dim() == 4, "q must have shape (B, H_Q, N_Q, D)");
+    require(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, "q must be float16 or bfloat16");
+    const int64_t B = q.size(0), HQ = q.size(1), NQ = q.size(2), D = q.size(3);
+    require(k_packed.dim() == 4 && k_packed.scalar_type() == at::kByte && k_packed.size(0) == B &&
+                k_packed.size(3) == D / 2,
+            "k_packed must be uint8 of shape (B, H_KV, N_KV, D/2)");
+    const int64_t HKV = k_packed.size(1), NKV = k_packed.size(2);
+    require(v_packed.scalar_type() == at::kByte && v_packed.sizes() == k_packed.sizes(),
+            "v_packed must be uint8 with the shape of k_packed");
+    require(HKV > 0 && HQ % HKV == 0, "H_Q must be a multiple of H_KV");
+    require(k_norms.scalar_type() == at::kFloat && k_norms.numel() == B * HKV * NKV &&
+                v_norms.scalar_type() == at::kFloat && v_norms.numel() == B * HKV * NKV,
+            "norms must be float32 with one value per (batch, KV head, token)");
+    require(centroids_k.numel() == 16 && centroids_v.numel() == 16 && centroids_k.scalar_type() == at::kFloat &&
+                centroids_v.scalar_type() == at::kFloat,
+            "centroids must be 16 float32 values");
+    c10::DeviceGuard guard(q.device());
+    const double scale = sm_scale.has_value() ? *sm_scale : 1.0 / std::sqrt(double(D));
+    const at::Tensor qc = q.contiguous();
+    const at::Tensor kp = k_packed.contiguous(), vp = v_packed.contiguous();
+    const at::Tensor kn = k_norms.to(q.device()).contiguous(), vn = v_norms.to(q.device()).contiguous();
+    const at::Tensor ck = centroids_k.to(q.device()).contiguous(), cv = centroids_v.to(q.device()).contiguous();
+    const RotationArg rot = rotation_arg(rotation, q.device(), D);
+    at::Tensor result = at::empty_like(qc);
+    const int st = fq_fused_tq_attention(
+        qc.data_ptr(), kp.data_ptr<uint8_t>(), kn.data_ptr<float>(), vp.data_ptr<uint8_t>(), vn.data_ptr<float>(),
+        ck.data_ptr<float>(), cv.data_ptr<float>(), rot.ptr, rot.col_major, result.data_ptr(),
+        int(B), int(HQ), int(HKV), int(NQ), int(NKV), int(D), float(scale), is_causal ? 1 : 0,
+        fqbind::dtype_code(q.scalar_type(), "fused_tq_attention"), fqbind::current_stream(q));
+    fqbind::raise_on_error(st, "fused_tq_attention");
+    return result;
+}
+
 at::Tensor rotate_query(const at::Tensor& q, const at::Tensor& rotation) {
     fqbind::require_gpu(q, "q");
     require(q.dim() == 3 && (q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16),
@@ -279,6 +319,10 @@ void bind_kernels(py::module_& m) {
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),
           py::arg("out") = py::none(), py::arg("num_splits") = 0,
           "Alias of split_k_paged_decode.");
+    m.def("fused_tq_attention", &fused_tq_attention, py::arg("q"), py::arg("k_packed"), py::arg("k_norms"),
+          py::arg("v_packed"), py::arg("v_norms"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),
+          py::arg("sm_scale") = py::none(), py::arg("is_causal") = false,
+          "Fused TQ4 attention: un-rotated q (B, H_Q, N_Q, D) over packed K/V, original-space output");
     m.def("rotate_query", &rotate_query, py::arg("q"), py::arg("rotation"),
           "q_rot = (q @ rotation.T) rounded to q's dtype.");
     m.def("paged_tq4_decode_partials", &paged_tq4_decode_partials, py::arg("q_rot"), py::arg("kv_cache"),

@@ -1,0 +1,146 @@
+// Device helpers shared by the attention kernels: the byte -> (fp16, fp16) centroid
+// table in LDS, cross-lane reductions that stay in the VALU, and the float32-MFMA
+// head rotation.
+#pragma once
+
+#include "fq_common.hpp"
+
+namespace fq {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kLutCopies = 64;                // one copy per lane: entry stride 256 bytes
+constexpr int kLutWords = 256 * kLutCopies;   // per table (64 KB)
+constexpr float kHalfMax = 65504.0f;
+
+__device__ __forceinline__ uint32_t byte_of(uint32_t w, int b) { return (w >> (8 * b)) & 0xffu; }
+
+// LDS byte address of table entry `byte K of w` in the copy of this lane: the entry
+// stride is 256 bytes and lane_off = 4 * lane < 256, so the address is the two bytes
+// (byte K of w, lane_off) side by side: one v_perm_b32 instead of extract, shift and add.
+template <int K>
+__device__ __forceinline__ uint32_t lut_addr(uint32_t w, uint32_t lane_off) {
+    return __builtin_amdgcn_perm(w, lane_off, 0x0C0C0000u | ((4u + K) << 8));
+}
+__device__ __forceinline__ uint32_t lds_word(const uint8_t* table, uint32_t addr) {
+    return *reinterpret_cast<const uint32_t*>(table + addr);
+}
+// the four fp16 pairs of the four bytes of w
+__device__ __forceinline__ uint4v lookup_word(const uint8_t* table, uint32_t w, uint32_t lane_off) {
+    uint4v r;
+    r.x = lds_word(table, lut_addr<0>(w, lane_off));
+    r.y = lds_word(table, lut_addr<1>(w, lane_off));
+    r.z = lds_word(table, lut_addr<2>(w, lane_off));
+    r.w = lds_word(table, lut_addr<3>(w, lane_off));
+    return r;
+}
+// byte BI of each of four words
+template <int BI>
+__device__ __forceinline__ uint4v lookup_column(const uint8_t* table, const uint32_t (&src)[4], uint32_t lane_off) {
+    uint4v r;
+    r.x = lds_word(table, lut_addr<BI>(src[0], lane_off));
+    r.y = lds_word(table, lut_addr<BI>(src[1], lane_off));
+    r.z = lds_word(table, lut_addr<BI>(src[2], lane_off));
+    r.w = lds_word(table, lut_addr<BI>(src[3], lane_off));
+    return r;
+}
+
+// Fills a 64-copy byte table: entry (byte, copy) = fp16 pair (centroid[byte >> 4],
+// centroid[byte & 15]).  The 16 centroids are fetched once (lane l holds centroid
+// l % 16); a wavefront then writes one byte's 64 copies per step, picking the two
+// values with v_readlane, so the build is a short LDS-write loop with no memory
+// latency inside it.
+__device__ __forceinline__ void fill_byte_table(uint32_t* table, float mine, int wave, int waves, int lane) {
+    for (int byte = wave; byte < 256; byte += waves) {
+        const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), byte >> 4));
+        const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), byte & 15));
+        table[byte * kLutCopies + lane] = pack_h2(_Float16(hi), _Float16(lo));
+    }
+}
+__device__ __forceinline__ void build_byte_table(uint32_t* table, const float* __restrict__ centroids, int wave,
+                                                 int waves, int lane) {
+    fill_byte_table(table, centroids[lane & 15], wave, waves, lane);
+}
+
+// Cross-lane helpers that stay in the VALU (no LDS round trip).
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+// max over lanes l and l ^ 16 (rows of 16 lanes swapped pairwise)
+__device__ __forceinline__ float max_xor16(float v) {
+    const uint32_t u = float_to_bits(v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return __builtin_fmaxf(bits_to_float(r[0]), bits_to_float(r[1]));
+}
+// max over lanes l and l ^ 32
+__device__ __forceinline__ float max_xor32(float v) {
+    const uint32_t u = float_to_bits(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_fmaxf(bits_to_float(r[0]), bits_to_float(r[1]));
+}
+// max over all lanes that share lane % GP
+template <int GP>
+__device__ __forceinline__ float max_same_head(float v) {
+    if (GP <= 4) v = __builtin_fmaxf(v, dpp_mov<0x124>(v));   // row_ror:4
+    if (GP <= 8) v = __builtin_fmaxf(v, dpp_mov<0x128>(v));   // row_ror:8
+    return max_xor32(max_xor16(v));
+}
+
+// ---------------------------------------------------------------------------------------
+// Head rotations: rows of D elements times the D x D rotation, float32 throughout, on the
+// float32 MFMA (v_mfma_f32_16x16x4_f32), so that no splitting of the matrix is needed and
+// the result matches a float32 matmul to rounding.  A workgroup (4 wavefronts) owns 16
+// rows; wavefront w produces the 16-column blocks w, w + 4, ...
+//
+// The contraction index is permuted so that operands load as contiguous runs: MFMA step
+// (j, e) with lane group g uses k = 32 j + 8 g + e, hence lane (m, g) holds the 8-element
+// runs k = 32 j + 8 g .. + 7 of row m (A side) and of the matrix (B side).
+// ---------------------------------------------------------------------------------------
+
+constexpr int kRotRows = 16;
+
+// B operand values of one 16-column block.  TRANSPOSED: out = x @ R.T (B[k][n] = R[col+n][k],
+// contiguous in k); otherwise out = x @ R (B[k][n] = R[k][col+n], 16 lanes contiguous in n).
+template <int D, bool TRANSPOSED>
+__device__ __forceinline__ void load_rotation_block(const float* __restrict__ R, int col, int n, int g,
+                                                    float (&b)[D / 32][8]) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+        if (TRANSPOSED) {
+            const float4v* src = reinterpret_cast<const float4v*>(R + int64_t(col + n) * D + 32 * j + 8 * g);
+            const float4v lo = src[0], hi = src[1];
+            b[j][0] = lo.x; b[j][1] = lo.y; b[j][2] = lo.z; b[j][3] = lo.w;
+            b[j][4] = hi.x; b[j][5] = hi.y; b[j][6] = hi.z; b[j][7] = hi.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) b[j][e] = R[int64_t(32 * j + 8 * g + e) * D + col + n];
+        }
+    }
+}
+
+// Rotation matrix given either row-major (element (i, j) at i*D + j) or column-major
+// (at i + j*D, i.e. the transpose is the contiguous one, which is what a QR factor
+// moved to the GPU looks like).  `x_times_Rt` selects out = x @ R.T, else out = x @ R.
+template <int D>
+__device__ __forceinline__ void load_rotation_any(const float* __restrict__ R, bool col_major, bool x_times_Rt,
+                                                  int col, int n, int g, float (&b)[D / 32][8]) {
+    // x @ R.T on a column-major R reads the same addresses as x @ R on a row-major one
+    if (x_times_Rt != col_major) load_rotation_block<D, true>(R, col, n, g, b);
+    else load_rotation_block<D, false>(R, col, n, g, b);
+}
+
+template <int D>
+__device__ __forceinline__ float4v rotate_block(const float (&a)[D / 32][8], const float (&b)[D / 32][8]) {
+    // four independent partial sums: a single accumulator would chain D/4 dependent MFMAs
+    float4v acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            acc[e & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j][e], b[j][e], acc[e & 3], 0, 0, 0);
+    return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+}
+
+}  // namespace fq

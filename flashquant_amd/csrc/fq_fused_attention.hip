@@ -1,0 +1,429 @@
+// Fused TQ4 FlashAttention (prefill) for gfx950: un-rotated query in, packed TQ4
+// keys and values in, original-space output out.
+//
+// Operator: fused_tq_attention_reference
+// (src/flashquant/kernels/cpu_reference.py:154-227) as dispatched by
+// src/flashquant/kernels/attention.py:85-107:
+//   q_rot = (q @ R^T) rounded to the query dtype
+//   K, V  = centroid[idx] * norm in rotated space
+//   out   = (softmax(q_rot K^T * scale + causal mask) V) @ R, rounded once
+// The causal mask hides key j > query i counted from the top-left corner and is
+// dropped when there is a single query row (cpu_reference.py:97-151).
+//
+// Work split.  A workgroup of 8 wavefronts serves one (batch, KV head) pair and 8
+// "units": a unit is a block of 32 query positions of one query head of the group,
+// so with 4 query heads per KV head a workgroup covers 64 positions of all 4 heads
+// and every dequantised K/V tile is used for 256 query rows.
+//
+// Per 64-token tile all 512 threads dequantise K and V into LDS as fp16 with the
+// norm folded in (one LDS lookup per packed byte in a byte -> (fp16, fp16) table),
+// double buffered, one barrier per tile; then each wavefront runs
+//   S^T (64 tokens x 32 rows)  = K_tile . q_rot^T      16 x v_mfma_f32_32x32x16_f16
+//   O^T (128 coords x 32 rows) += V_tile^T . P^T        16 x v_mfma_f32_32x32x16_f16
+// Both products are transposed so that a lane owns one query row (column l % 32 of
+// every accumulator): the running maximum, the denominator and the rescale of O are
+// per-lane scalars, and P goes from the S accumulator straight into the B operand
+// of the second product.  That works because the contraction index of an MFMA may
+// be permuted freely as long as both operands agree: the accumulator registers
+// r = 8u .. 8u+7 of lane half hf hold rows 16u + 8a + 4hf + c (e = 4a + c), so the
+// V tile stores token 16u + 8a + 4b + c at position 16u + 8b + 4a + c and a lane's
+// 8 consecutive positions are exactly its 8 tokens.  The K tile uses the same
+// permutation on the coordinates, and the query operand is read to match.
+//
+// The two head rotations run on the float32 MFMA inside the kernel (prologue and
+// epilogue), staged through the tile buffers.
+#include "fq_common.hpp"
+#include "fq_device.hpp"
+
+namespace fq {
+
+constexpr int kPfKStride = 272;                       // bytes per token row of the K tile (128 fp16 + pad)
+constexpr int kPfKBytes = 64 * kPfKStride;            // 17408
+constexpr int kPfVBytes = 128 * 128;                  // V^T tile: 128 coordinate rows x 64 tokens fp16
+constexpr int kPfBufBytes = kPfKBytes + kPfVBytes;    // 33792
+constexpr int kPfStageBytes = 8192;                   // per-wavefront staging area for the rotations
+
+struct PrefillParams {
+    const uint16_t* q;          // (B, H_Q, N_Q, 128)
+    const uint8_t* k_packed;    // (B, H_KV, N_KV, 64)
+    const float* k_norms;       // (B, H_KV, N_KV)
+    const uint8_t* v_packed;
+    const float* v_norms;
+    const float* centroids_k;
+    const float* centroids_v;
+    const float* rotation;      // (128, 128)
+    uint16_t* out;              // (B, H_Q, N_Q, 128)
+    int rot_col_major;
+    int H_Q, H_KV, G, N_Q, N_KV;
+    int causal;
+    float scale_log2e;
+};
+
+// Table with the K codebook in the lower 128 bytes of every 256-byte row (32
+// copies, one per bank) and the V codebook in the upper 128 bytes.
+__device__ __forceinline__ void fill_dual_table(uint32_t* table, float mine_k, float mine_v, int wave, int waves,
+                                                int lane) {
+    for (int byte = wave; byte < 256; byte += waves) {
+        const float khi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_k), byte >> 4));
+        const float klo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_k), byte & 15));
+        const float vhi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_v), byte >> 4));
+        const float vlo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_v), byte & 15));
+        table[byte * 64 + lane] = lane < 32 ? pack_h2(_Float16(khi), _Float16(klo)) : pack_h2(_Float16(vhi), _Float16(vlo));
+    }
+}
+
+__device__ __forceinline__ uint32_t scale_pair(uint32_t pair, half2v n2) {
+    const half2v h = __builtin_bit_cast(half2v, pair) * n2;
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+__device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+
+template <int DT>
+__global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillParams p) {
+    constexpr int D = 128;
+    __shared__ __attribute__((aligned(256))) uint32_t lut[256 * 64];
+    extern __shared__ __attribute__((aligned(16))) uint8_t bufs[];   // 2 x (K tile | V^T tile)
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m32 = lane & 31, hf = lane >> 5;     // 32x32 MFMA: column (query row) and lane half
+    const int n16 = lane & 15, g4 = lane >> 4;     // 16x16 MFMA of the rotations
+    const int b = blockIdx.z, hkv = blockIdx.y;
+
+    // ---- units --------------------------------------------------------------------------
+    const int nblk = (p.N_Q + 31) >> 5;
+    const int units = nblk * p.G;
+    const int wg = int(gridDim.x) - 1 - int(blockIdx.x);   // late (long) query blocks start first
+    const int unit_raw = 8 * wg + w;
+    const bool unit_live = unit_raw < units;
+    const int unit = unit_live ? unit_raw : units - 1;
+    const int hq = hkv * p.G + unit % p.G;
+    const int pos0 = 32 * (unit / p.G);
+    const int last_unit = 8 * wg + 7 < units - 1 ? 8 * wg + 7 : units - 1;
+    int wg_maxpos = 32 * (last_unit / p.G) + 31;
+    wg_maxpos = wg_maxpos < p.N_Q - 1 ? wg_maxpos : p.N_Q - 1;
+    int my_maxpos = pos0 + 31 < p.N_Q - 1 ? pos0 + 31 : p.N_Q - 1;
+    const int all_tiles = (p.N_KV + 63) >> 6;
+    int ntiles = all_tiles, my_tiles = all_tiles;
+    if (p.causal) {
+        ntiles = (wg_maxpos >> 6) + 1 < all_tiles ? (wg_maxpos >> 6) + 1 : all_tiles;
+        my_tiles = (my_maxpos >> 6) + 1 < all_tiles ? (my_maxpos >> 6) + 1 : all_tiles;
+    }
+    if (!unit_live) my_tiles = 0;
+
+    // ---- tables -----------------------------------------------------------------------------
+    fill_dual_table(lut, p.centroids_k[lane & 15], p.centroids_v[lane & 15], w, 8, lane);
+    const uint8_t* lutb = reinterpret_cast<const uint8_t*>(lut);
+    const uint32_t lk = 4u * (lane & 31), lv = 128u + lk;
+
+    // ---- dequantisation plan ------------------------------------------------------------------
+    const int64_t kv_row0 = (int64_t(b) * p.H_KV + hkv) * p.N_KV;
+    const uint8_t* kp = p.k_packed + kv_row0 * 64;
+    const uint8_t* vp = p.v_packed + kv_row0 * 64;
+    const float* knp = p.k_norms + kv_row0;
+    const float* vnp = p.v_norms + kv_row0;
+    const int tk = tid >> 3, gqk = tid & 7;        // K: token of the tile, 16-coordinate group
+    const int tp = tid >> 4, jv = tid & 15;        // V: token pair of the tile, dword of the row
+    const int k_wr = tk * kPfKStride + gqk * 32;
+    int v_wr[8];
+    {
+        const int tt = 2 * tp, t16 = tt & 15;
+        const int posv = (tt & ~15) + 8 * ((t16 >> 2) & 1) + 4 * ((t16 >> 3) & 1) + (t16 & 3);
+        const int giv = posv >> 3, within = posv & 7;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int d = 8 * jv + k;
+            const int physg = giv ^ k ^ (jv & 7);
+            v_wr[k] = kPfKBytes + d * 128 + 16 * physg + 2 * within;
+        }
+    }
+    uint2v kraw;
+    uint32_t vra, vrb;
+    float nk, nv0, nv1;
+    auto issue_loads = [&](int tile) {
+        const int t0 = tile * 64;
+        const int last = p.N_KV - 1;
+        const int tkk = t0 + tk < last ? t0 + tk : last;
+        const int ta = t0 + 2 * tp < last ? t0 + 2 * tp : last;
+        const int tb = t0 + 2 * tp + 1 < last ? t0 + 2 * tp + 1 : last;
+        kraw = *reinterpret_cast<const uint2v*>(kp + int64_t(tkk) * 64 + 8 * gqk);
+        nk = knp[tkk];
+        vra = *reinterpret_cast<const uint32_t*>(vp + int64_t(ta) * 64 + 4 * jv);
+        vrb = *reinterpret_cast<const uint32_t*>(vp + int64_t(tb) * 64 + 4 * jv);
+        nv0 = vnp[ta];
+        nv1 = vnp[tb];
+    };
+    auto dequant = [&](int buf) {
+        uint8_t* dst = bufs + buf * kPfBufBytes;
+        const _Float16 hk = _Float16(nk);
+        const half2v nk2 = {hk, hk};
+        const uint4v a0 = lookup_word(lutb, kraw.x, lk);   // coordinates 0..7 of the group
+        const uint4v a1 = lookup_word(lutb, kraw.y, lk);   // coordinates 8..15
+        // positions 0..7 = coordinates (0..3, 8..11), positions 8..15 = (4..7, 12..15)
+        const uint4v w0 = {scale_pair(a0.x, nk2), scale_pair(a0.y, nk2), scale_pair(a1.x, nk2), scale_pair(a1.y, nk2)};
+        const uint4v w1 = {scale_pair(a0.z, nk2), scale_pair(a0.w, nk2), scale_pair(a1.z, nk2), scale_pair(a1.w, nk2)};
+        *reinterpret_cast<uint4v*>(dst + k_wr) = w0;
+        *reinterpret_cast<uint4v*>(dst + k_wr + 16) = w1;
+        // V: 2x2 nibble transpose, so that a byte holds one coordinate of the two tokens
+        const uint32_t X = (vra & 0xF0F0F0F0u) | ((vrb >> 4) & 0x0F0F0F0Fu);   // even coordinates
+        const uint32_t Y = ((vra << 4) & 0xF0F0F0F0u) | (vrb & 0x0F0F0F0Fu);   // odd coordinates
+        const half2v nv2 = {_Float16(nv0), _Float16(nv1)};
+        const uint4v xe = lookup_word(lutb, X, lv);
+        const uint4v yo = lookup_word(lutb, Y, lv);
+        const uint32_t xs[4] = {xe.x, xe.y, xe.z, xe.w}, ys[4] = {yo.x, yo.y, yo.z, yo.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            *reinterpret_cast<uint32_t*>(dst + v_wr[2 * c]) = scale_pair(xs[c], nv2);
+            *reinterpret_cast<uint32_t*>(dst + v_wr[2 * c + 1]) = scale_pair(ys[c], nv2);
+        }
+    };
+
+    issue_loads(0);
+
+    // ---- query: rotate this wavefront's 32 rows, round to the query dtype, scale to fp16 ----------
+    half8 qb[8];
+    float krow;
+    {
+        const uint16_t* qbase = p.q + ((int64_t(b) * p.H_Q + hq) * p.N_Q) * D;
+        uint16_t* st = reinterpret_cast<uint16_t*>(bufs + w * kPfStageBytes);   // (32 rows, 128) raw 16-bit
+        float a[2][4][8];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+            int pos = pos0 + 16 * rb + n16;
+            pos = pos < p.N_Q ? pos : p.N_Q - 1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint4v raw = *reinterpret_cast<const uint4v*>(qbase + int64_t(pos) * D + 32 * j + 8 * g4);
+                const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    a[rb][j][2 * i] = load_elem<DT>(uint16_t(wds[i] & 0xffffu));
+                    a[rb][j][2 * i + 1] = load_elem<DT>(uint16_t(wds[i] >> 16));
+                }
+            }
+        }
+        for (int cb = 0; cb < 8; ++cb) {
+            float rbv[4][8];
+            load_rotation_any<D>(p.rotation, p.rot_col_major != 0, true, 16 * cb, n16, g4, rbv);
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+                const float4v acc = rotate_block<D>(a[rb], rbv);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) st[(16 * rb + 4 * g4 + i) * D + 16 * cb + n16] = store_elem<DT>(acc[i]);
+            }
+        }
+        __syncthreads();
+        float qf[8][8];
+        float mx = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const uint2v lo = *reinterpret_cast<const uint2v*>(st + m32 * D + 16 * ks + 4 * hf);
+            const uint2v hi = *reinterpret_cast<const uint2v*>(st + m32 * D + 16 * ks + 8 + 4 * hf);
+            const uint32_t wds[4] = {lo.x, lo.y, hi.x, hi.y};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                qf[ks][2 * i] = load_elem<DT>(uint16_t(wds[i] & 0xffffu));
+                qf[ks][2 * i + 1] = load_elem<DT>(uint16_t(wds[i] >> 16));
+                mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(qf[ks][2 * i]), __builtin_fabsf(qf[ks][2 * i + 1])));
+            }
+        }
+        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 32));
+        int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+        if (ex < -100 || ex > 100) ex = 0;
+        const float down = bits_to_float(uint32_t(127 - ex) << 23);
+        krow = p.scale_log2e * bits_to_float(uint32_t(127 + ex) << 23);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qb[ks][e] = _Float16(qf[ks][e] * down);
+        __syncthreads();   // the staging area becomes tile buffers
+    }
+
+    // ---- lane-constant LDS read offsets ----------------------------------------------------------
+    const int k_rd = m32 * kPfKStride + 16 * hf;
+    int v_rd[8];
+    {
+        const int lanex = hf ^ (m32 & 7) ^ (m32 >> 3);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) v_rd[c] = kPfKBytes + m32 * 128 + 16 * (lanex ^ c);
+    }
+
+    // ---- running state -----------------------------------------------------------------------------
+    float16v O[4];
+#pragma unroll
+    for (int ob = 0; ob < 4; ++ob)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) O[ob][r] = 0.0f;
+    float m_run = -__builtin_inff();
+    float l_run = 0.0f;
+    const int qpos = pos0 + m32;
+
+    auto compute = [&](int tile, int buf) {
+        const uint8_t* kt = bufs + buf * kPfBufBytes;
+        float16v S[2];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) S[tb][r] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                const half8 a = *reinterpret_cast<const half8*>(kt + k_rd + 32 * tb * kPfKStride + 32 * ks);
+                S[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qb[ks], S[tb], 0, 0, 0);
+            }
+        }
+        const int t0 = tile * 64;
+        const bool need_mask = (t0 + 63 >= p.N_KV) || (p.causal && t0 + 63 > pos0);   // wavefront-uniform
+        if (need_mask) {
+            int lim = p.N_KV - 1;
+            if (p.causal && qpos < lim) lim = qpos;
+            lim -= t0;                         // token offsets <= lim are visible
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int off = 32 * tb + 8 * (r >> 2) + 4 * hf + (r & 3);
+                    if (off > lim) S[tb][r] = -__builtin_inff();
+                }
+        }
+        float mx = S[0][0];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, S[tb][r]);
+        mx = max_xor32(mx);
+        const float mnew = __builtin_fmaxf(m_run, mx * krow);
+        const float ms = mnew == -__builtin_inff() ? 0.0f : mnew;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - ms);
+        m_run = mnew;
+        uint4v pbv[4];
+        float ps = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            float pe[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                pe[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[s >> 1][8 * (s & 1) + e], krow, -ms));
+                ps += pe[e];
+            }
+            pbv[s] = uint4v{pack_rtz(pe[0], pe[1]), pack_rtz(pe[2], pe[3]), pack_rtz(pe[4], pe[5]), pack_rtz(pe[6], pe[7])};
+        }
+        l_run = __builtin_fmaf(l_run, alpha, ps);
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int ob = 0; ob < 4; ++ob)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) O[ob][r] *= alpha;
+        }
+#pragma unroll
+        for (int ob = 0; ob < 4; ++ob)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int c = (2 * s) ^ (4 * (ob & 1));
+                const half8 a = *reinterpret_cast<const half8*>(kt + v_rd[c] + ob * 4096);
+                O[ob] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, __builtin_bit_cast(half8, pbv[s]), O[ob], 0, 0, 0);
+            }
+    };
+
+    // ---- tiles ----------------------------------------------------------------------------------------
+    dequant(0);
+    if (ntiles > 1) issue_loads(1);
+    for (int i = 0; i < ntiles; ++i) {
+        __syncthreads();                       // tile i is complete; the other buffer is free
+        if (i + 1 < ntiles) {
+            dequant((i + 1) & 1);
+            if (i + 2 < ntiles) issue_loads(i + 2);
+        }
+        if (i < my_tiles) compute(i, i & 1);
+    }
+
+    // ---- normalise, rotate back, store -------------------------------------------------------------------
+    const float l_tot = l_run + xor_shuffle(l_run, 32);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    float* stf = reinterpret_cast<float*>(bufs + w * kPfStageBytes);   // (16 rows, 128) float32
+    uint16_t* obase = p.out + ((int64_t(b) * p.H_Q + hq) * p.N_Q) * D;
+    for (int half_rows = 0; half_rows < 2; ++half_rows) {
+        __syncthreads();
+        if ((m32 >> 4) == half_rows) {
+#pragma unroll
+            for (int ob = 0; ob < 4; ++ob)
+#pragma unroll
+                for (int rq = 0; rq < 4; ++rq) {
+                    const float4v v = {O[ob][4 * rq] * inv, O[ob][4 * rq + 1] * inv, O[ob][4 * rq + 2] * inv, O[ob][4 * rq + 3] * inv};
+                    *reinterpret_cast<float4v*>(stf + (m32 & 15) * D + 32 * ob + 8 * rq + 4 * hf) = v;
+                }
+        }
+        __syncthreads();
+        float a[4][8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4v lo = *reinterpret_cast<const float4v*>(stf + n16 * D + 32 * j + 8 * g4);
+            const float4v hi = *reinterpret_cast<const float4v*>(stf + n16 * D + 32 * j + 8 * g4 + 4);
+            a[j][0] = lo.x; a[j][1] = lo.y; a[j][2] = lo.z; a[j][3] = lo.w;
+            a[j][4] = hi.x; a[j][5] = hi.y; a[j][6] = hi.z; a[j][7] = hi.w;
+        }
+        for (int cb = 0; cb < 8; ++cb) {
+            float rbv[4][8];
+            load_rotation_any<D>(p.rotation, p.rot_col_major != 0, false, 16 * cb, n16, g4, rbv);
+            const float4v acc = rotate_block<D>(a, rbv);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int pos = pos0 + 16 * half_rows + 4 * g4 + i;
+                if (unit_live && pos < p.N_Q) obase[int64_t(pos) * D + 16 * cb + n16] = store_elem<DT>(acc[i]);
+            }
+        }
+    }
+}
+
+}  // namespace fq
+
+extern "C" int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, const float* k_norms,
+                                     const uint8_t* v_packed, const float* v_norms,
+                                     const float* centroids_k, const float* centroids_v,
+                                     const float* rotation, int rotation_col_major, void* out,
+                                     int B, int H_Q, int H_KV, int N_Q, int N_KV, int D,
+                                     float sm_scale, int is_causal, int dtype, void* stream) {
+    using namespace fq;
+    if (B < 0 || H_Q <= 0 || H_KV <= 0 || N_Q < 0 || N_KV < 0 || H_Q % H_KV != 0) return FQ_ERR_BAD_SHAPE;
+    if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
+    if (D != 128) return FQ_ERR_UNSUPPORTED_DIM;   // the tile layout is written for 128 coordinates
+    if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
+    if (B == 0 || N_Q == 0) return FQ_OK;
+    if (N_KV == 0) return FQ_ERR_BAD_SHAPE;          // softmax over no keys is undefined
+    if (!q || !k_packed || !k_norms || !v_packed || !v_norms || !centroids_k || !centroids_v || !rotation || !out)
+        return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(q, 16) || !fq_host::aligned(k_packed, 8) || !fq_host::aligned(v_packed, 4) ||
+        !fq_host::aligned(rotation, 16) || !fq_host::aligned(out, 2))
+        return FQ_ERR_MISALIGNED;
+    if (B > 65535 || H_KV > 65535) return FQ_ERR_BAD_SHAPE;
+
+    PrefillParams p;
+    p.q = static_cast<const uint16_t*>(q);
+    p.k_packed = k_packed; p.k_norms = k_norms; p.v_packed = v_packed; p.v_norms = v_norms;
+    p.centroids_k = centroids_k; p.centroids_v = centroids_v;
+    p.rotation = rotation; p.rot_col_major = rotation_col_major;
+    p.out = static_cast<uint16_t*>(out);
+    p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.N_Q = N_Q; p.N_KV = N_KV;
+    p.causal = (is_causal && N_Q > 1) ? 1 : 0;
+    p.scale_log2e = sm_scale * kLog2e;
+
+    const int64_t units = int64_t((N_Q + 31) / 32) * p.G;
+    const int64_t wgs = (units + 7) / 8;
+    if (wgs > 0x7fffffffLL) return FQ_ERR_BAD_SHAPE;
+    const dim3 grid(static_cast<unsigned>(wgs), H_KV, B), block(512);
+    const size_t lds = 2 * size_t(kPfBufBytes);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == FQ_F16) {
+        auto kern = fused_tq_attention_kernel<FQ_F16>;
+        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
+    } else {
+        auto kern = fused_tq_attention_kernel<FQ_BF16>;
+        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
+    }
+    return fq_host::check_launch();
+}

@@ -86,6 +86,32 @@ int fq_tq4_decompress(const uint8_t* packed, const float* norms,
                       int64_t M, int D, void* stream);
 
 /*
+ * Fused TQ4 attention (prefill): un-rotated query, packed keys and values,
+ * original-space output.  Takes the role of the reference's fused launcher
+ * (csrc/cuda/fused_tq_attention.cu:468-479); operator defined by
+ * fused_tq_attention_reference (src/flashquant/kernels/cpu_reference.py:154-227)
+ * with the query pre-rotation of src/flashquant/kernels/attention.py:85-107.
+ *
+ *   q          (B, H_Q, N_Q, D) fp16/bf16, contiguous, 16-byte aligned
+ *   k_packed   (B, H_KV, N_KV, D/2) uint8, contiguous; v_packed the same
+ *   k_norms    (B, H_KV, N_KV) float32; v_norms the same
+ *   centroids_k, centroids_v  (16,) float32
+ *   rotation   (D, D) float32, layout as in fq_split_k_paged_decode
+ *   out        (B, H_Q, N_Q, D) same dtype as q
+ *   is_causal  key j > query i (counted from the top-left corner) is hidden;
+ *              ignored when N_Q == 1, as in the reference
+ * D == 128 (FQ_ERR_UNSUPPORTED_DIM otherwise); H_Q a multiple of H_KV; N_KV >= 1.
+ * K and V are dequantised to fp16 with the norm folded in, so a row norm times a
+ * centroid must stay below 65504.
+ */
+int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, const float* k_norms,
+                          const uint8_t* v_packed, const float* v_norms,
+                          const float* centroids_k, const float* centroids_v,
+                          const float* rotation, int rotation_col_major, void* out,
+                          int B, int H_Q, int H_KV, int N_Q, int N_KV, int D,
+                          float sm_scale, int is_causal, int dtype, void* stream);
+
+/*
  * Split-K paged decode from the packed TQ4 cache, un-rotated query in,
  * original-space output out.  Takes the roles of paged_tq4_decode_cuda
  * (csrc/cuda/paged_decode.cu:346-368) and split_k_reduce_cuda

@@ -228,3 +228,85 @@ def test_paged_decode_distinct_value_codebook():
     got = K.split_k_paged_decode(q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), c.to(DEV), cv.to(DEV),
                                  r.to(DEV), 2, 128, 16)
     assert (got.cpu().float() - want.float()).abs().max() <= 2e-2
+
+
+# ---- fused TQ4 attention (prefill) ------------------------------------------------
+
+def _prefill_case(b, hq, hkv, nq, nkv, dtype, seed, kv_scale=1.0, v_seed_rot=None):
+    c, bnd, r = book(128)
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b, hq, nq, 128, generator=g).to(dtype)
+    k = outlier_rows(b * hkv * nkv, 1, 128, seed + 1).reshape(b, hkv, nkv, 128) * kv_scale
+    v = outlier_rows(b * hkv * nkv, 1, 128, seed + 2).reshape(b, hkv, nkv, 128) * kv_scale
+    kp, kn = O.compress(k.reshape(-1, 1, 128), r, bnd)
+    vp, vn = O.compress(v.reshape(-1, 1, 128), r, bnd)
+    shape_p, shape_n = (b, hkv, nkv, 64), (b, hkv, nkv, 1)
+    return q, kp.reshape(shape_p), kn.reshape(shape_n), vp.reshape(shape_p), vn.reshape(shape_n), c, r
+
+
+def _check_prefill(b, hq, hkv, nq, nkv, dtype, causal, seed=11, kv_scale=1.0, scale=None, cv=None):
+    q, kp, kn, vp, vn, c, r = _prefill_case(b, hq, hkv, nq, nkv, dtype, seed, kv_scale)
+    cv = c if cv is None else cv
+    want = O.fused_tq_attention(q, kp, kn, vp, vn, c, cv, r, sm_scale=scale, is_causal=causal)
+    got = K.fused_tq_attention(q.to(DEV), kp.to(DEV), kn.to(DEV), vp.to(DEV), vn.to(DEV), c.to(DEV), cv.to(DEV),
+                               r.to(DEV), sm_scale=scale, is_causal=causal)
+    torch.cuda.synchronize()
+    assert got.shape == q.shape and got.dtype == q.dtype
+    err = (got.cpu().float() - want.float()).abs().max().item()
+    tol = 2e-2 * max(1.0, want.float().abs().max().item())
+    assert err <= tol, f"max abs error {err} (tolerance {tol})"
+    return err
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_attention_llama_heads(causal, dtype):
+    # 32 query heads over 8 KV heads, several 64-token tiles, a ragged tail
+    _check_prefill(1, 32, 8, 200, 200, dtype, causal)
+
+
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 4), (6, 2), (16, 2), (16, 1), (5, 1)])
+def test_fused_attention_group_sizes(hq, hkv):
+    _check_prefill(2, hq, hkv, 97, 97, torch.bfloat16, True, seed=21)
+
+
+@pytest.mark.parametrize("nq,nkv,causal", [(1, 130, True), (1, 64, False), (33, 257, False), (64, 64, True),
+                                           (65, 300, True), (300, 65, True), (31, 31, True), (128, 128, True)])
+def test_fused_attention_lengths(nq, nkv, causal):
+    _check_prefill(1, 8, 2, nq, nkv, torch.bfloat16, causal, seed=31)
+
+
+def test_fused_attention_scaled_inputs_and_custom_scale():
+    _check_prefill(1, 8, 2, 96, 96, torch.float16, True, seed=41, kv_scale=30.0, scale=0.02)
+
+
+def test_fused_attention_distinct_value_codebook():
+    c, _, _ = book(128)
+    cv = (c * 1.25 + 0.01).contiguous()
+    _check_prefill(1, 8, 2, 80, 80, torch.bfloat16, True, seed=51, cv=cv)
+
+
+def test_fused_attention_matches_dequantize_then_sdpa():
+    # the same result from decompressing with the HIP kernel and running torch's SDPA in rotated space
+    q, kp, kn, vp, vn, c, r = _prefill_case(1, 8, 2, 256, 256, torch.bfloat16, 61)
+    dev = [t.to(DEV) for t in (q, kp, kn, vp, vn, c, r)]
+    got = K.fused_tq_attention(*dev[:5], dev[5], dev[5], dev[6], is_causal=True)
+    kd = K.tq4_decompress(dev[1].reshape(-1, 1, 64), dev[2].reshape(-1, 1, 1), dev[5], dtype=torch.float32).reshape(1, 2, 256, 128)
+    vd = K.tq4_decompress(dev[3].reshape(-1, 1, 64), dev[4].reshape(-1, 1, 1), dev[5], dtype=torch.float32).reshape(1, 2, 256, 128)
+    q_rot = (dev[0].float() @ dev[6].T).to(torch.bfloat16).float()
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q_rot, kd.repeat_interleave(4, 1), vd.repeat_interleave(4, 1), is_causal=True)
+    ref = (ref @ dev[6]).to(torch.bfloat16)
+    # outlier channels reach |value| ~ 10, where one bfloat16 step is 0.06: scale the bound like _check_prefill
+    assert (got.float() - ref.float()).abs().max().item() <= 2e-2 * max(1.0, ref.float().abs().max().item())
+
+
+def test_fused_attention_rejects_bad_arguments():
+    q, kp, kn, vp, vn, c, r = _prefill_case(1, 8, 2, 16, 16, torch.bfloat16, 71)
+    dev = [t.to(DEV) for t in (q, kp, kn, vp, vn, c, r)]
+    with pytest.raises(ValueError):
+        K.fused_tq_attention(dev[0][:, :7], *dev[1:5], dev[5], dev[5], dev[6])      # 7 heads over 2
+    with pytest.raises(ValueError):
+        K.fused_tq_attention(dev[0].float(), *dev[1:5], dev[5], dev[5], dev[6])     # float32 query
+    with pytest.raises(RuntimeError):
+        K.fused_tq_attention(q, *dev[1:5], dev[5], dev[5], dev[6])                  # CPU query
