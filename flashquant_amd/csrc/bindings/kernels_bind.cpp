@@ -89,6 +89,41 @@ std::tuple<at::Tensor, at::Tensor> tq4_compress(const at::Tensor& x, const at::T
     return {packed, norms};
 }
 
+void tq4_compress_store(const at::Tensor& key, const at::Tensor& value, const at::Tensor& rot_T_even,
+                        const at::Tensor& rot_T_odd, const at::Tensor& boundaries, at::Tensor kv_cache,
+                        const at::Tensor& slot_mapping) {
+    fqbind::require_gpu(key, "key");
+    fqbind::require_gpu(value, "value");
+    fqbind::require_gpu(kv_cache, "kv_cache");
+    require(key.dim() == 3 && value.sizes() == key.sizes() && value.scalar_type() == key.scalar_type(),
+            "key and value must both have shape (N, H, D) and one dtype");
+    require(key.scalar_type() == at::kHalf || key.scalar_type() == at::kBFloat16, "key/value must be float16 or bfloat16");
+    const int64_t N = key.size(0), H = key.size(1), D = key.size(2);
+    require(rot_T_even.scalar_type() == at::kFloat && rot_T_odd.scalar_type() == at::kFloat &&
+                boundaries.scalar_type() == at::kFloat,
+            "rotation halves and boundaries must be float32");
+    require(rot_T_even.dim() == 2 && rot_T_even.size(0) == D && rot_T_even.size(1) == D / 2 &&
+                rot_T_odd.sizes() == rot_T_even.sizes(),
+            "rotation halves must have shape (D, D/2)");
+    require(boundaries.numel() == 15, "boundaries must hold 15 values (4-bit codebook)");
+    require(kv_cache.scalar_type() == at::kByte && kv_cache.is_contiguous() && kv_cache.dim() >= 2 &&
+                kv_cache.size(-1) == H * (D + 8),
+            "kv_cache must be a contiguous uint8 tensor whose last dimension is H * (D + 8)");
+    require(slot_mapping.dim() == 1 && slot_mapping.size(0) <= N, "slot_mapping must be 1-D with at most N entries");
+    c10::DeviceGuard guard(key.device());
+    const at::Tensor kc = key.contiguous(), vc = value.contiguous();
+    const at::Tensor re = rot_T_even.to(key.device()).contiguous();
+    const at::Tensor ro = rot_T_odd.to(key.device()).contiguous();
+    const at::Tensor bd = boundaries.to(key.device()).contiguous();
+    const at::Tensor sm = slot_mapping.to(key.device(), at::kLong).contiguous();
+    const int64_t num_slots = kv_cache.numel() / (H * (D + 8));
+    const int st = fq_tq4_compress_store(kc.data_ptr(), vc.data_ptr(), fqbind::dtype_code(key.scalar_type(), "tq4_compress_store"),
+                                         re.data_ptr<float>(), ro.data_ptr<float>(), bd.data_ptr<float>(),
+                                         kv_cache.data_ptr<uint8_t>(), sm.data_ptr<int64_t>(), N, sm.size(0), int(H),
+                                         int(D), num_slots, fqbind::current_stream(key));
+    fqbind::raise_on_error(st, "tq4_compress_store");
+}
+
 at::Tensor tq4_decompress(const at::Tensor& packed, const at::Tensor& norms, const at::Tensor& centroids,
                           at::ScalarType dtype, const std::optional<at::Tensor>& out) {
     fqbind::require_gpu(packed, "packed");
@@ -304,6 +339,9 @@ void bind_kernels(py::module_& m) {
     m.def("tq4_compress", &tq4_compress, py::arg("x"), py::arg("rotation_T_even"), py::arg("rotation_T_odd"),
           py::arg("boundaries"), py::arg("out") = py::none(),
           "TQ4 compress of (N, H, D) fp16/bf16 rows -> (packed (N, H, D/2) uint8, norms (N, H, 1) float32).");
+    m.def("tq4_compress_store", &tq4_compress_store, py::arg("key"), py::arg("value"), py::arg("rotation_T_even"),
+          py::arg("rotation_T_odd"), py::arg("boundaries"), py::arg("kv_cache"), py::arg("slot_mapping"),
+          "Compress key and value (N, H, D) and write them into the packed paged cache at slot_mapping");
     m.def("tq4_decompress", &tq4_decompress, py::arg("packed"), py::arg("norms"), py::arg("centroids"),
           py::arg("dtype"), py::arg("out") = py::none(),
           "TQ4 decompress to (N, H, D) in dtype, rotated space.");

@@ -113,12 +113,39 @@ __device__ __forceinline__ int mfma_row_to_coord(int r) {
     return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
 }
 
-template <int D, int DT>
+// Destination of the fused compress-and-store (the work of _compress_and_store,
+// src/flashquant/vllm/impl.py:220-263, in one launch): rows [0, rows_k) come from the key
+// tensor and rows [rows_k, 2 rows_k) from the value tensor, row = token * H + head, and each
+// lands in the paged cache row of slot_mapping[token]:
+// [K idx H*D/2 | K norm H*4 | V idx H*D/2 | V norm H*4] (src/flashquant/vllm/impl.py:132-138).
+struct PagedDest {
+    const uint4v* x_value;      // (tokens, H, D) values
+    uint8_t* cache;             // (num_slots, H*(D+8))
+    const int64_t* slots;       // (mapped,) flat slot of each token; negative: not stored
+    int64_t rows_k;             // tokens * H
+    int64_t num_slots;
+    int mapped;                 // tokens with a slot
+    int H;
+    int wide;                   // 16-byte stores are aligned
+};
+
+template <int D, int DT, bool PAGED>
 __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     const uint4v* __restrict__ x, const float* __restrict__ rot_T_even,
     const float* __restrict__ rot_T_odd, const float* __restrict__ boundaries,
-    uint8_t* __restrict__ packed, float* __restrict__ norms, int64_t M, int64_t num_tiles) {
+    uint8_t* __restrict__ packed, float* __restrict__ norms, int64_t M, int64_t num_tiles, const PagedDest pd) {
     using C = CompressCfg<D>;
+    // paged mode: cache row of a (tensor, token, head) row, or nullptr when the token has no slot
+    auto paged_row = [&](int64_t row, int& head, int& is_v) -> uint8_t* {
+        is_v = row >= pd.rows_k ? 1 : 0;
+        const int64_t r = row - (is_v ? pd.rows_k : 0);
+        const int64_t tok = r / pd.H;
+        head = int(r - tok * pd.H);
+        if (tok >= pd.mapped) return nullptr;
+        const int64_t slot = pd.slots[tok];
+        if (slot < 0 || slot >= pd.num_slots) return nullptr;
+        return pd.cache + slot * (int64_t(pd.H) * (D + 8)) + (is_v ? int64_t(pd.H) * (D / 2 + 4) : 0);
+    };
     __shared__ __attribute__((aligned(16))) uint8_t xs[2][C::TT * C::XS_STRIDE];
     __shared__ __attribute__((aligned(16))) uint8_t outs[C::TT * C::OUT_STRIDE];
     __shared__ float inv_s[2][C::TT];
@@ -163,7 +190,13 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
 #pragma unroll
         for (int p = 0; p < C::PASSES; ++p) {
             const int64_t row = tile * C::TT + p * C::ROWS_PER_PASS + row_in_pass;
-            pre[p] = row < M ? __builtin_nontemporal_load(x + row * C::CPR + chunk) : uint4v{0, 0, 0, 0};
+            if (PAGED) {
+                const bool second = row >= pd.rows_k;
+                const uint4v* src = second ? pd.x_value + (row - pd.rows_k) * C::CPR : x + row * C::CPR;
+                pre[p] = row < M ? __builtin_nontemporal_load(src + chunk) : uint4v{0, 0, 0, 0};
+            } else {
+                pre[p] = row < M ? __builtin_nontemporal_load(x + row * C::CPR + chunk) : uint4v{0, 0, 0, 0};
+            }
         }
     };
     auto stage = [&](int64_t tile, int buf) {
@@ -202,7 +235,15 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             *reinterpret_cast<uint4v*>(&xs[buf][r * C::XS_STRIDE + chunk * 16]) = h;
             if (chunk == 0) {
                 inv_s[buf][r] = up / (nrm + 1e-10f);
-                if (row < M) norms[row] = nrm;
+                if (row < M) {
+                    if (PAGED) {
+                        int head, is_v;
+                        uint8_t* dst = paged_row(row, head, is_v);
+                        if (dst) *reinterpret_cast<float*>(dst + pd.H * (D / 2) + 4 * head) = nrm;
+                    } else {
+                        norms[row] = nrm;
+                    }
+                }
             }
         }
     };
@@ -258,7 +299,21 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                 const uint2v lo = *reinterpret_cast<const uint2v*>(&outs[r * C::OUT_STRIDE + q * 16]);
                 const uint2v hi = *reinterpret_cast<const uint2v*>(&outs[r * C::OUT_STRIDE + q * 16 + 8]);
                 uint4v v = {lo.x, lo.y, hi.x, hi.y};
-                __builtin_nontemporal_store(v, reinterpret_cast<uint4v*>(packed + row * (D / 2)) + q);
+                if (PAGED) {
+                    int head, is_v;
+                    uint8_t* dst = paged_row(row, head, is_v);
+                    if (dst) {
+                        dst += head * (D / 2) + 16 * q;
+                        if (pd.wide) {
+                            *reinterpret_cast<uint4v*>(dst) = v;
+                        } else {
+                            uint32_t* d4 = reinterpret_cast<uint32_t*>(dst);
+                            d4[0] = v.x; d4[1] = v.y; d4[2] = v.z; d4[3] = v.w;
+                        }
+                    }
+                } else {
+                    __builtin_nontemporal_store(v, reinterpret_cast<uint4v*>(packed + row * (D / 2)) + q);
+                }
             }
         }
         if (next < num_tiles) stage(next, cur ^ 1);
@@ -273,8 +328,22 @@ int launch_compress(const void* x, const float* re, const float* ro, const float
     const int64_t tiles = (M + C::TT - 1) / C::TT;
     const int64_t cap = int64_t(num_cus) * 2;
     const unsigned grid = unsigned(tiles < cap ? tiles : cap);
-    hipLaunchKernelGGL((tq4_compress_kernel<D, DT>), dim3(grid), dim3(C::THREADS), 0, s,
-                       reinterpret_cast<const uint4v*>(x), re, ro, bnd, packed, norms, M, tiles);
+    hipLaunchKernelGGL((tq4_compress_kernel<D, DT, false>), dim3(grid), dim3(C::THREADS), 0, s,
+                       reinterpret_cast<const uint4v*>(x), re, ro, bnd, packed, norms, M, tiles, PagedDest{});
+    return fq_host::check_launch();
+}
+
+template <int D, int DT>
+int launch_compress_store(const void* key, const float* re, const float* ro, const float* bnd, const PagedDest& pd,
+                          int num_cus, hipStream_t s) {
+    using C = CompressCfg<D>;
+    const int64_t M = 2 * pd.rows_k;
+    const int64_t tiles = (M + C::TT - 1) / C::TT;
+    const int64_t cap = int64_t(num_cus) * 2;
+    const unsigned grid = unsigned(tiles < cap ? tiles : cap);
+    hipLaunchKernelGGL((tq4_compress_kernel<D, DT, true>), dim3(grid), dim3(C::THREADS), 0, s,
+                       reinterpret_cast<const uint4v*>(key), re, ro, bnd, static_cast<uint8_t*>(nullptr),
+                       static_cast<float*>(nullptr), M, tiles, pd);
     return fq_host::check_launch();
 }
 
@@ -322,4 +391,44 @@ extern "C" int fq_tq4_compress(const void* x, int x_dtype, const float* rot_T_ev
         default: return FQ_ERR_UNSUPPORTED_DIM;
     }
 #undef FQ_COMPRESS_CASE
+}
+
+extern "C" int fq_tq4_compress_store(const void* key, const void* value, int x_dtype,
+                                     const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
+                                     uint8_t* kv_cache, const int64_t* slot_mapping,
+                                     int64_t num_tokens, int64_t num_mapped, int H_KV, int D,
+                                     int64_t num_slots, void* stream) {
+    using namespace fq;
+    if (num_tokens < 0 || num_mapped < 0 || num_mapped > num_tokens || H_KV <= 0 || num_slots < 0) return FQ_ERR_BAD_SHAPE;
+    if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
+    if (x_dtype != FQ_F16 && x_dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
+    if (num_tokens == 0 || num_mapped == 0) return FQ_OK;
+    if (!key || !value || !rot_T_even || !rot_T_odd || !boundaries || !kv_cache || !slot_mapping) return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(key, 16) || !fq_host::aligned(value, 16) || !fq_host::aligned(kv_cache, 16) ||
+        !fq_host::aligned(slot_mapping, 8))
+        return FQ_ERR_MISALIGNED;
+    if (num_tokens > 0x7fffffffLL || num_tokens * H_KV > (int64_t(1) << 40)) return FQ_ERR_BAD_SHAPE;
+    PagedDest pd;
+    pd.x_value = static_cast<const uint4v*>(value);
+    pd.cache = kv_cache;
+    pd.slots = slot_mapping;
+    pd.rows_k = num_tokens * H_KV;
+    pd.num_slots = num_slots;
+    pd.mapped = int(num_mapped);
+    pd.H = H_KV;
+    pd.wide = ((int64_t(H_KV) * (D + 8)) % 16 == 0 && (int64_t(H_KV) * (D / 2 + 4)) % 16 == 0 && (D / 2) % 16 == 0) ? 1 : 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int cus = fq_host::device_cu_count();
+#define FQ_STORE_CASE(DD)                                                                            \
+    case DD:                                                                                         \
+        return x_dtype == FQ_F16                                                                     \
+                   ? launch_compress_store<DD, FQ_F16>(key, rot_T_even, rot_T_odd, boundaries, pd, cus, s)  \
+                   : launch_compress_store<DD, FQ_BF16>(key, rot_T_even, rot_T_odd, boundaries, pd, cus, s);
+    switch (D) {
+        FQ_STORE_CASE(64)
+        FQ_STORE_CASE(128)
+        FQ_STORE_CASE(256)
+        default: return FQ_ERR_UNSUPPORTED_DIM;
+    }
+#undef FQ_STORE_CASE
 }

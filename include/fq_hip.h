@@ -69,6 +69,26 @@ int fq_tq4_compress(const void* x, int x_dtype,
                     int64_t M, int D, void* stream);
 
 /*
+ * Fused compress-and-store: compresses key and value rows and writes them straight
+ * into the packed paged cache, one launch.  Takes the place of the two tq4_compress
+ * calls, the row assembly and the advanced-index scatter of _compress_and_store
+ * (src/flashquant/vllm/impl.py:220-263); cache row layout of
+ * src/flashquant/vllm/impl.py:132-138.
+ *
+ *   key, value    (num_tokens, H_KV, D) fp16 or bf16, contiguous, 16-byte aligned
+ *   kv_cache      (num_slots, H_KV*(D+8)) uint8 viewed flat over (block, position), 16-byte aligned
+ *   slot_mapping  (num_mapped,) int64: flat slot of token i; tokens i >= num_mapped are
+ *                 not stored (impl.py:259-261).  A negative or out-of-range slot is
+ *                 skipped (the reference's index assignment would wrap a negative one).
+ * Tokens that map to the same slot race, as they do in the reference.
+ */
+int fq_tq4_compress_store(const void* key, const void* value, int x_dtype,
+                          const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
+                          uint8_t* kv_cache, const int64_t* slot_mapping,
+                          int64_t num_tokens, int64_t num_mapped, int H_KV, int D,
+                          int64_t num_slots, void* stream);
+
+/*
  * TQ4 decompress.  Takes the role of tq4_decompress_cuda
  * (csrc/cuda/decompress.cuh:40-48); operator defined by decompress_reference
  * (src/flashquant/kernels/cpu_reference.py:64-94) followed by the cast of

@@ -310,3 +310,68 @@ def test_fused_attention_rejects_bad_arguments():
         K.fused_tq_attention(dev[0].float(), *dev[1:5], dev[5], dev[5], dev[6])     # float32 query
     with pytest.raises(RuntimeError):
         K.fused_tq_attention(q, *dev[1:5], dev[5], dev[5], dev[6])                  # CPU query
+
+
+# ---- fused compress-and-store into the paged cache -----------------------------------
+
+@pytest.mark.parametrize("h,d,dtype", [(8, 128, torch.bfloat16), (8, 128, torch.float16), (1, 64, torch.bfloat16),
+                                       (3, 256, torch.float16), (2, 128, torch.bfloat16)])
+def test_compress_and_store_matches_compress_then_scatter(h, d, dtype):
+    c, bnd, r = book(d)
+    n, bs, nb = 203, 16, 20
+    key = outlier_rows(n, h, d, 81, dtype=dtype)
+    value = outlier_rows(n, h, d, 82, dtype=dtype)
+    g = torch.Generator().manual_seed(83)
+    slots = torch.randperm(nb * bs, generator=g)[:n].long()
+    slots[5] = -1                      # padding token: not stored
+    slots[77] = -1
+    mapped = n - 9                     # the last 9 tokens have no slot at all
+    cache0 = torch.randint(0, 256, (nb, bs, h * (d + 8)), dtype=torch.uint8, generator=g)
+    cache = cache0.clone().to(DEV)
+    K.tq4_compress_and_store(key.to(DEV), value.to(DEV), r.to(DEV), bnd.to(DEV), cache, slots[:mapped].to(DEV))
+    kp, kn = K.tq4_compress(key.to(DEV), r.to(DEV), bnd.to(DEV))
+    vp, vn = K.tq4_compress(value.to(DEV), r.to(DEV), bnd.to(DEV))
+    torch.cuda.synchronize()
+    want = cache0.clone()
+    keep = (slots[:mapped] >= 0).nonzero().flatten()
+    O.store_rows(want, slots[:mapped][keep], kp.cpu()[keep], kn.cpu()[keep], vp.cpu()[keep], vn.cpu()[keep])
+    assert torch.equal(cache.cpu(), want)
+
+
+def test_compress_and_store_then_decode_matches_oracle():
+    # the write path and the read path agree on the page layout: store with the HIP kernel,
+    # decode with the HIP kernel, compare with the oracle working from the original K/V
+    c, bnd, r = book(128)
+    hq, hkv, bs, L = 32, 8, 16, 300
+    g = torch.Generator().manual_seed(91)
+    k = torch.randn(L, hkv, 128, generator=g).to(torch.bfloat16)
+    v = torch.randn(L, hkv, 128, generator=g).to(torch.bfloat16)
+    q = torch.randn(1, hq, 128, generator=g).to(torch.bfloat16)
+    nb = (L + bs - 1) // bs + 2
+    table = torch.randperm(nb, generator=g)[: (L + bs - 1) // bs].reshape(1, -1).int()
+    t = torch.arange(L)
+    slots = table[0].long()[t // bs] * bs + t % bs
+    cache = torch.zeros(nb, bs, hkv * 136, dtype=torch.uint8, device=DEV)
+    K.tq4_compress_and_store(k.to(DEV), v.to(DEV), r.to(DEV), bnd.to(DEV), cache, slots.to(DEV))
+    lens = torch.tensor([L], dtype=torch.int32)
+    got = K.split_k_paged_decode(q.to(DEV), cache, table.to(DEV), lens.to(DEV), c.to(DEV), c.to(DEV), r.to(DEV),
+                                 hkv, 128, bs)
+    cache_ref = torch.zeros(nb, bs, hkv * 136, dtype=torch.uint8)
+    kp, kn = O.compress(k, r, bnd)
+    vp, vn = O.compress(v, r, bnd)
+    O.store_rows(cache_ref, slots, kp, kn, vp, vn)
+    want = O.split_k_paged_decode(q, cache_ref, table, lens, c, c, r, hkv, 128, bs)
+    assert (got.cpu().float() - want.float()).abs().max().item() <= 2e-2
+
+
+def test_compress_and_store_rejects_bad_arguments():
+    c, bnd, r = book(128)
+    key = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device=DEV)
+    cache = torch.zeros(2, 16, 2 * 136, dtype=torch.uint8, device=DEV)
+    slots = torch.arange(4, device=DEV)
+    with pytest.raises(ValueError):
+        K.tq4_compress_and_store(key, key[:, :1], r.to(DEV), bnd.to(DEV), cache, slots)        # shapes differ
+    with pytest.raises(ValueError):
+        K.tq4_compress_and_store(key, key, r.to(DEV), bnd.to(DEV), cache[..., :100], slots)    # wrong row size
+    with pytest.raises(ValueError):
+        K.tq4_compress_and_store(key, key, r.to(DEV), bnd.to(DEV), cache, torch.arange(5, device=DEV))  # too many slots
