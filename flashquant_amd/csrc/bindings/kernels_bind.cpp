@@ -248,6 +248,88 @@ at::Tensor fused_tq_attention(const at::Tensor& q, const at::Tensor& k_packed, c
     return result;
 }
 
+std::tuple<at::Tensor, at::Tensor, at::Tensor> prod_compress(const at::Tensor& x, const at::Tensor& rotation,
+                                                             const at::Tensor& sketch_rot, const at::Tensor& boundaries,
+                                                             const at::Tensor& centroids) {
+    fqbind::require_gpu(x, "x");
+    require(x.dim() == 3, "x must have shape (N, H, D)");
+    require(x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16, "x must be float16 or bfloat16");
+    const int64_t N = x.size(0), H = x.size(1), D = x.size(2);
+    require(boundaries.numel() == 7 && centroids.numel() == 8 && boundaries.scalar_type() == at::kFloat &&
+                centroids.scalar_type() == at::kFloat,
+            "the 3-bit codebook has 7 float32 boundaries and 8 float32 centroids");
+    require(sketch_rot.dim() == 2 && sketch_rot.size(0) == D && sketch_rot.size(1) == D &&
+                sketch_rot.scalar_type() == at::kFloat,
+            "sketch_rot must be float32 of shape (D, D)");
+    c10::DeviceGuard guard(x.device());
+    const at::Tensor xc = x.contiguous();
+    const RotationArg rot = rotation_arg(rotation, x.device(), D);
+    const at::Tensor w = sketch_rot.to(x.device()).contiguous();
+    const at::Tensor bd = boundaries.to(x.device()).contiguous(), ce = centroids.to(x.device()).contiguous();
+    at::Tensor packed = at::empty({N, H, D / 2}, x.options().dtype(at::kByte));
+    at::Tensor norms = at::empty({N, H, 1}, x.options().dtype(at::kFloat));
+    at::Tensor gam = at::empty({N, H, 1}, x.options().dtype(at::kFloat));
+    const int st = fq_prod_compress(xc.data_ptr(), fqbind::dtype_code(x.scalar_type(), "prod_compress"), rot.ptr,
+                                    rot.col_major, w.data_ptr<float>(), bd.data_ptr<float>(), ce.data_ptr<float>(),
+                                    packed.data_ptr<uint8_t>(), norms.data_ptr<float>(), gam.data_ptr<float>(), N * H,
+                                    int(D), fqbind::current_stream(x));
+    fqbind::raise_on_error(st, "prod_compress");
+    return {packed, norms, gam};
+}
+
+at::Tensor prod_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache, const at::Tensor& block_table,
+                             const at::Tensor& seq_lens, const at::Tensor& centroids_k3, const at::Tensor& centroids_v,
+                             const at::Tensor& rotation, const at::Tensor& sketch, int64_t num_kv_heads,
+                             int64_t head_dim, int64_t block_size, std::optional<double> sm_scale,
+                             const std::optional<at::Tensor>& out, int64_t num_splits) {
+    fqbind::require_gpu(q, "q");
+    fqbind::require_gpu(kv_cache, "kv_cache");
+    require(q.dim() == 3 && q.size(2) == head_dim, "q must have shape (num_seqs, H_Q, D)");
+    require(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, "q must be float16 or bfloat16");
+    require(kv_cache.dim() == 3 && kv_cache.scalar_type() == at::kByte && kv_cache.is_contiguous() &&
+                kv_cache.size(1) == block_size && kv_cache.size(2) == num_kv_heads * (head_dim + 12),
+            "kv_cache must be contiguous uint8 of shape (num_blocks, block_size, num_kv_heads * (head_dim + 12))");
+    require(block_table.dim() == 2 && block_table.scalar_type() == at::kInt && block_table.size(0) == q.size(0),
+            "block_table must be int32 of shape (num_seqs, max_blocks)");
+    require(seq_lens.scalar_type() == at::kInt && seq_lens.numel() == q.size(0), "seq_lens must be int32 (num_seqs,)");
+    require(centroids_k3.numel() == 8 && centroids_v.numel() == 16 && centroids_k3.scalar_type() == at::kFloat &&
+                centroids_v.scalar_type() == at::kFloat,
+            "centroids_k3 must hold 8 and centroids_v 16 float32 values");
+    require(sketch.dim() == 2 && sketch.size(0) == head_dim && sketch.size(1) == head_dim &&
+                sketch.scalar_type() == at::kFloat,
+            "sketch must be float32 of shape (D, D)");
+    require(num_splits >= 0, "num_splits must be >= 0");
+    c10::DeviceGuard guard(q.device());
+    const int S = int(q.size(0)), HQ = int(q.size(1)), D = int(head_dim);
+    const double scale = sm_scale.has_value() ? *sm_scale : 1.0 / std::sqrt(double(head_dim));
+    const at::Tensor qc = q.contiguous();
+    const at::Tensor bt = block_table.to(q.device()).contiguous();
+    const at::Tensor sl = seq_lens.to(q.device()).contiguous();
+    const at::Tensor ck = centroids_k3.to(q.device()).contiguous(), cv = centroids_v.to(q.device()).contiguous();
+    const RotationArg rot = rotation_arg(rotation, q.device(), D);
+    const at::Tensor sk = sketch.to(q.device()).contiguous();
+    at::Tensor result;
+    if (out.has_value()) {
+        result = *out;
+        require(result.is_cuda() && result.is_contiguous() && result.scalar_type() == q.scalar_type() &&
+                    result.sizes() == q.sizes(),
+                "out must be a contiguous GPU tensor with the shape and dtype of q");
+    } else {
+        result = at::empty_like(qc);
+    }
+    const int max_blocks = int(bt.size(1));
+    const size_t ws_bytes = fq_paged_decode_workspace_bytes(S, HQ, int(num_kv_heads), D, int(block_size), max_blocks,
+                                                            int(num_splits));
+    at::Tensor ws = at::empty({int64_t(ws_bytes)}, q.options().dtype(at::kByte));
+    const int st = fq_prod_paged_decode(
+        qc.data_ptr(), kv_cache.data_ptr<uint8_t>(), bt.data_ptr<int32_t>(), sl.data_ptr<int32_t>(), ck.data_ptr<float>(),
+        cv.data_ptr<float>(), rot.ptr, rot.col_major, sk.data_ptr<float>(), result.data_ptr(), S, HQ, int(num_kv_heads), D,
+        int(block_size), max_blocks, kv_cache.size(0), float(scale), fqbind::dtype_code(q.scalar_type(), "prod_paged_decode"),
+        int(num_splits), ws.data_ptr(), ws_bytes, fqbind::current_stream(q));
+    fqbind::raise_on_error(st, "prod_paged_decode");
+    return result;
+}
+
 at::Tensor rotate_query(const at::Tensor& q, const at::Tensor& rotation) {
     fqbind::require_gpu(q, "q");
     require(q.dim() == 3 && (q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16),
@@ -361,6 +443,14 @@ void bind_kernels(py::module_& m) {
           py::arg("v_packed"), py::arg("v_norms"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),
           py::arg("sm_scale") = py::none(), py::arg("is_causal") = false,
           "Fused TQ4 attention: un-rotated q (B, H_Q, N_Q, D) over packed K/V, original-space output");
+    m.def("prod_compress", &prod_compress, py::arg("x"), py::arg("rotation"), py::arg("sketch_rot"),
+          py::arg("boundaries"), py::arg("centroids"),
+          "TurboQuantProd key compress: (packed nibbles sign<<3|idx (N,H,D/2), norms (N,H,1), residual norms (N,H,1))");
+    m.def("prod_paged_decode", &prod_paged_decode, py::arg("q"), py::arg("kv_cache"), py::arg("block_table"),
+          py::arg("seq_lens"), py::arg("centroids_k3"), py::arg("centroids_v"), py::arg("rotation"), py::arg("sketch"),
+          py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),
+          py::arg("out") = py::none(), py::arg("num_splits") = 0,
+          "Split-K paged decode over TurboQuantProd key / TQ4 value pages");
     m.def("rotate_query", &rotate_query, py::arg("q"), py::arg("rotation"),
           "q_rot = (q @ rotation.T) rounded to q's dtype.");
     m.def("paged_tq4_decode_partials", &paged_tq4_decode_partials, py::arg("q_rot"), py::arg("kv_cache"),

@@ -56,6 +56,21 @@ __device__ __forceinline__ void fill_byte_table(uint32_t* table, float mine, int
         table[byte * kLutCopies + lane] = pack_h2(_Float16(hi), _Float16(lo));
     }
 }
+// Two tables in one 64 KB array of 256-byte rows: the K table in the lower 128 bytes of
+// every row (lanes 0..31 write it, 32 copies, one per LDS bank of a half-wave) and the V
+// table in the upper 128 bytes.  A K nibble is looked up as `nibble & k_mask` (15 for TQ4,
+// 7 when bit 3 of the nibble is a sign bit), a V nibble as it is.  Lane l holds
+// k_centroids[l & k_mask] and v_centroids[l & 15].
+__device__ __forceinline__ void fill_pair_tables(uint32_t* table, float mine_k, float mine_v, int k_mask, int wave,
+                                                 int waves, int lane) {
+    for (int byte = wave; byte < 256; byte += waves) {
+        const float khi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_k), (byte >> 4) & k_mask));
+        const float klo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_k), byte & k_mask));
+        const float vhi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_v), byte >> 4));
+        const float vlo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_v), byte & 15));
+        table[byte * 64 + lane] = lane < 32 ? pack_h2(_Float16(khi), _Float16(klo)) : pack_h2(_Float16(vhi), _Float16(vlo));
+    }
+}
 __device__ __forceinline__ void build_byte_table(uint32_t* table, const float* __restrict__ centroids, int wave,
                                                  int waves, int lane) {
     fill_byte_table(table, centroids[lane & 15], wave, waves, lane);

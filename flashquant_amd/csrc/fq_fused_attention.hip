@@ -59,19 +59,6 @@ struct PrefillParams {
     float scale_log2e;
 };
 
-// Table with the K codebook in the lower 128 bytes of every 256-byte row (32
-// copies, one per bank) and the V codebook in the upper 128 bytes.
-__device__ __forceinline__ void fill_dual_table(uint32_t* table, float mine_k, float mine_v, int wave, int waves,
-                                                int lane) {
-    for (int byte = wave; byte < 256; byte += waves) {
-        const float khi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_k), byte >> 4));
-        const float klo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_k), byte & 15));
-        const float vhi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_v), byte >> 4));
-        const float vlo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_v), byte & 15));
-        table[byte * 64 + lane] = lane < 32 ? pack_h2(_Float16(khi), _Float16(klo)) : pack_h2(_Float16(vhi), _Float16(vlo));
-    }
-}
-
 __device__ __forceinline__ uint32_t scale_pair(uint32_t pair, half2v n2) {
     const half2v h = __builtin_bit_cast(half2v, pair) * n2;
     return __builtin_bit_cast(uint32_t, h);
@@ -116,7 +103,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     if (!unit_live) my_tiles = 0;
 
     // ---- tables -----------------------------------------------------------------------------
-    fill_dual_table(lut, p.centroids_k[lane & 15], p.centroids_v[lane & 15], w, 8, lane);
+    fill_pair_tables(lut, p.centroids_k[lane & 15], p.centroids_v[lane & 15], 15, w, 8, lane);
     const uint8_t* lutb = reinterpret_cast<const uint8_t*>(lut);
     const uint32_t lk = 4u * (lane & 31), lv = 128u + lk;
 

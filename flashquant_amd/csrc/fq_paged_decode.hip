@@ -74,6 +74,7 @@ struct DecodeParams {
     const void* q_rot;          // (S, H_Q, D) query dtype: rotated, or un-rotated when `rotation` is set
     int rot_col_major;          // layout of `rotation` / of the matrix given to the side kernels
     const float* rotation;      // staged kernel only: rotate the query in the prologue (NULL: already rotated)
+    const float* sketch;        // TurboQuantProd pages only: the (D, D) sign-sketch matrix S
     const uint8_t* cache;       // (num_blocks, BS, H_KV*(D+8))
     const int32_t* block_table; // (S, max_blocks)
     const int32_t* seq_lens;    // (S,)
@@ -527,12 +528,21 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 // (head, token) scores.
 // ---------------------------------------------------------------------------------------
 
-constexpr int kStageBytes = 17408;            // 16 rows x 8 heads x 136 bytes
-constexpr int kTileBytes = 2 * kStageBytes;   // 32 tokens
+// TurboQuantProd pages (PROD): the key nibble is (sign bit << 3 | 3-bit index) and a key
+// carries a second float32, the residual norm, so a token row is
+// [K nibbles H*64 | K norm H*4 | K residual norm H*4 | V idx H*64 | V norm H*4] = H*140 bytes
+// and a stage grows by 512 bytes of residual norms.
+template <bool PROD>
+struct StagedCfg {
+    static constexpr int CHUNKS_PER_ROW = PROD ? 70 : 68;          // 16-byte chunks of a token row, 8 heads
+    static constexpr int ROWB = 16 * CHUNKS_PER_ROW;               // 1088 / 1120
+    static constexpr int STAGE_BYTES = 16 * ROWB;                  // 17408 / 17920
+    static constexpr int TILE_BYTES = 2 * STAGE_BYTES;             // 32 tokens
+    static constexpr int CHUNKS_PER_TILE = 32 * CHUNKS_PER_ROW;    // 2176 / 2240
+};
 constexpr int kStageKnOff = 16384;
 constexpr int kStageVnOff = 16896;
-constexpr int kChunksPerRow = 68;
-constexpr int kChunksPerTile = 32 * kChunksPerRow;   // 2176
+constexpr int kStageKgOff = 17408;
 
 __host__ __device__ constexpr int staged_slot(int h, int r, int q) {
     const int pp = (r ^ ((r >> 2) & 1) ^ (h & 1)) & 15;
@@ -540,6 +550,7 @@ __host__ __device__ constexpr int staged_slot(int h, int r, int q) {
 }
 
 // LDS byte offset (inside a tile slot) of the 16-byte chunk `ci` of tile row `row` (0..31).
+template <bool PROD>
 __device__ __forceinline__ int staged_chunk_dst(int row, int ci) {
     const int stage = row >> 4, r = row & 15;
     int off;
@@ -547,23 +558,46 @@ __device__ __forceinline__ int staged_chunk_dst(int row, int ci) {
         off = 16 * staged_slot(ci >> 2, r, ci & 3);
     } else if (ci < 34) {
         off = kStageKnOff + 32 * r + 16 * (ci - 32);
-    } else if (ci < 66) {
-        off = 8192 + 16 * staged_slot((ci - 34) >> 2, r, (ci - 34) & 3);
+    } else if (PROD && ci < 36) {
+        off = kStageKgOff + 32 * r + 16 * (ci - 34);
     } else {
-        off = kStageVnOff + 32 * r + 16 * (ci - 66);
+        const int cv = ci - (PROD ? 36 : 34);
+        if (cv < 32) off = 8192 + 16 * staged_slot(cv >> 2, r, cv & 3);
+        else off = kStageVnOff + 32 * r + 16 * (cv - 32);
     }
-    return stage * kStageBytes + off;
+    return stage * StagedCfg<PROD>::STAGE_BYTES + off;
 }
 
-template <int BSL, int GP, int DT, int PVR>
+// TurboQuantProd sign operand: the fp16 pairs (+-1, +-1) of the eight sign bits (bit 3 of
+// every nibble) of one key dword.  Element e of the result belongs to the coordinate
+// kSignOrder[e] of the dword's eight: the query-side operand is permuted to match.
+__device__ __forceinline__ uint4v sign_operand(uint32_t w, uint32_t ones) {
+    uint4v r;
+    r.x = (w & 0x80008000u) | ones;
+    r.y = ((w << 4) & 0x80008000u) | ones;
+    r.z = ((w << 8) & 0x80008000u) | ones;
+    r.w = ((w << 12) & 0x80008000u) | ones;
+    return r;
+}
+__device__ __forceinline__ constexpr int sign_order(int e) {
+    constexpr int order[8] = {2, 6, 3, 7, 0, 4, 1, 5};
+    return order[e];
+}
+
+template <int BSL, int GP, int DT, int PVR, bool PROD>
 __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodeParams p) {
+    using Cfg = StagedCfg<PROD>;
+    constexpr int kStageBytes = Cfg::STAGE_BYTES;
+    constexpr int kTileBytes = Cfg::TILE_BYTES;
+    constexpr int kChunksPerRow = Cfg::CHUNKS_PER_ROW;
+    constexpr int kChunksPerTile = Cfg::CHUNKS_PER_TILE;
     constexpr int D = 128;
     constexpr int BS = 1 << BSL;
     constexpr int KS = 4;                 // k-steps of the score product
     constexpr int DPL = 8;                // V coordinates per lane
     constexpr int NSC = GP / 2;           // scores per lane per tile
     constexpr int H = 8;
-    constexpr int ROWB = H * (D + 8);     // 1088
+    constexpr int ROWB = Cfg::ROWB;       // 1088, or 1120 with residual norms
     constexpr int PPT = BS >= 32 ? 1 : 32 / BS;   // pages per tile
 
     // The table is a static array so that its LDS address is a compile-time constant
@@ -588,15 +622,21 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     // Every load that depends on nothing is asked for first, so that the memory
     // latencies of the prologue overlap instead of adding up: the centroids, the
     // rotation columns of this wavefront and the first 32 query heads.
-    const float cent_mine = p.centroids_k[lane & 15];
+    // K table in the lower 128 bytes of every 256-byte table row (32 copies, one per bank),
+    // V table in the upper 128 bytes
+    const float cent_k_mine = p.centroids_k[lane & (PROD ? 7 : 15)];
+    const float cent_v_mine = p.centroids_v[lane & 15];
     const uint8_t* lut_k = reinterpret_cast<const uint8_t*>(lut);
-    const uint8_t* lut_v = lut_k;          // this kernel is used when K and V share the codebook
-    const uint32_t lane_off = 4u * lane;
+    const uint8_t* lut_v = lut_k;
+    const uint32_t lane_off = 4u * (lane & 31);
+    const uint32_t lane_off_v = 128u + lane_off;
     const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + int64_t(seq) * p.H_Q * 128;
     float rot_b[4][8];
+    float rot_s[4][8];
     uint4v q_pre[2][4];
     if (p.rotation != nullptr) {
         load_rotation_any<128>(p.rotation, p.rot_col_major != 0, true, 16 * h, n, g, rot_b);
+        if constexpr (PROD) load_rotation_any<128>(p.sketch, false, true, 16 * h, n, g, rot_s);
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
@@ -648,7 +688,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         return v;
     };
     // the table is filled while the page ids are on their way
-    fill_byte_table(lut, cent_mine, h, 8, lane);
+    fill_pair_tables(lut, cent_k_mine, cent_v_mine, PROD ? 7 : 15, h, 8, lane);
 
     // ---- copy plan: chunk c = tid + 512 k of the tile, k = 0..4 (the last round only
     // for the first 128 threads) -----------------------------------------------------------
@@ -663,7 +703,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         const int row = c / kChunksPerRow, ci = c % kChunksPerRow;
         src_page[k] = BS >= 32 ? 0 : row >> BSL;
         src_off[k] = uint32_t((row & (BS - 1)) * ROWB + ci * 16);
-        dst_off[k] = staged_chunk_dst(row, ci);
+        dst_off[k] = staged_chunk_dst<PROD>(row, ci);
     }
     const bool has_round4 = tid < kChunksPerTile - 4 * 512;   // 128 threads, whole wavefronts
 
@@ -700,13 +740,16 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     // rounded to the query dtype as the reference rounds it, and the heads are exchanged
     // through LDS (the tile slots are not in use yet).
     half8 qh[KS];
+    half8 qsh[KS];              // PROD: sketched query S q (times sqrt(pi/2) / D), elements in sign order
     float qscale;
+    float qscale_s = 0.0f;
     {
         float qf[KS][8];
         float mx = 0.0f;
         const bool live = hd < p.G;
         if (p.rotation != nullptr) {
-            float* qs = reinterpret_cast<float*>(slots);   // (H_Q, D) float32, H_Q <= 128
+            float* qs = reinterpret_cast<float*>(slots);   // (H_Q, D) float32, H_Q <= 128 (64 with a sketch)
+            float* qs2 = qs + 64 * D;                      // PROD: (H_Q, D) float32 sketched query
             for (int rb = 0; 16 * rb < p.H_Q; ++rb) {
                 const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
                 float a[KS][8];
@@ -731,6 +774,14 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                     const int head = 16 * rb + 4 * g + i;
                     if (head < p.H_Q) qs[head * D + 16 * h + n] = load_elem<DT>(store_elem<DT>(acc[i]));
                 }
+                if constexpr (PROD) {
+                    const float4v acc2 = rotate_block<D>(a, rot_s);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int head = 16 * rb + 4 * g + i;
+                        if (head < p.H_Q) qs2[head * D + 16 * h + n] = acc2[i];
+                    }
+                }
             }
             FQ_MARK(4);
             __syncthreads();
@@ -743,6 +794,29 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                     qf[ks][e] = live ? src[8 * ks + e] : 0.0f;
                     mx = __builtin_fmaxf(mx, __builtin_fabsf(qf[ks][e]));
                 }
+            if constexpr (PROD) {
+                // <S q, signs> * sqrt(pi/2) / D: the constant rides on the query side
+                const float* src2 = qs2 + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
+                float qf2[KS][8];
+                float mx2 = 0.0f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        qf2[ks][e] = live ? src2[8 * ks + sign_order(e)] * (1.2533141373155003f / float(D)) : 0.0f;
+                        mx2 = __builtin_fmaxf(mx2, __builtin_fabsf(qf2[ks][e]));
+                    }
+                mx2 = __builtin_fmaxf(mx2, xor_shuffle(mx2, 16));
+                mx2 = __builtin_fmaxf(mx2, xor_shuffle(mx2, 32));
+                int ex2 = int((float_to_bits(mx2) >> 23) & 0xffu) - 127;
+                if (ex2 < -100 || ex2 > 100) ex2 = 0;
+                const float down2 = bits_to_float(uint32_t(127 - ex2) << 23);
+                qscale_s = p.scale_log2e * bits_to_float(uint32_t(127 + ex2) << 23);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) qsh[ks][e] = _Float16(qf2[ks][e] * down2);
+            }
             FQ_MARK(6);
             __syncthreads();   // the slots are about to receive tiles
         } else {
@@ -806,7 +880,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         // operands of this lane, raw
         uint4v kraw[2];
         uint32_t vraw[2][4];
-        float kn[NSC], vn[NSC];
+        float kn[NSC], vn[NSC], kg[NSC];
 #pragma unroll
         for (int b = 0; b < 2; ++b) kraw[b] = *reinterpret_cast<const uint4v*>(tile + k_rd[b]);
 #pragma unroll
@@ -817,6 +891,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         for (int e = 0; e < NSC; ++e) {
             kn[e] = *reinterpret_cast<const float*>(tile + n_rd[e]);
             vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageVnOff - kStageKnOff));
+            kg[e] = PROD ? *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageKgOff - kStageKnOff)) : 0.0f;
         }
 
         // ---- scores: lookups of block 1 in flight during the MFMAs of block 0 ----------------
@@ -840,20 +915,29 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             for (int e = 0; e < 4; ++e) {
                 const int db = 4 * grp + e, bi = db / 2;
                 const uint32_t (&src)[4] = (db & 1) ? Y : X;
-                dst[e] = (bi == 0) ? lookup_column<0>(lut_v, src, lane_off)
-                       : (bi == 1) ? lookup_column<1>(lut_v, src, lane_off)
-                       : (bi == 2) ? lookup_column<2>(lut_v, src, lane_off)
-                                   : lookup_column<3>(lut_v, src, lane_off);
+                dst[e] = (bi == 0) ? lookup_column<0>(lut_v, src, lane_off_v)
+                       : (bi == 1) ? lookup_column<1>(lut_v, src, lane_off_v)
+                       : (bi == 2) ? lookup_column<2>(lut_v, src, lane_off_v)
+                                   : lookup_column<3>(lut_v, src, lane_off_v);
             }
         };
         __builtin_amdgcn_sched_barrier(0);
         float4v acc[2];
+        float4v acc_s[2];
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             acc[b] = float4v{0.f, 0.f, 0.f, 0.f};
+            acc_s[b] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
                 acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ka[b][ks]), qh[ks], acc[b], 0, 0, 0);
+            if constexpr (PROD) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const uint4v sg = sign_operand(kw[b][ks], 0x3C003C00u);
+                    acc_s[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, sg), qsh[ks], acc_s[b], 0, 0, 0);
+                }
+            }
             if (b == 0) v_group(0, vb[0]);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -863,19 +947,28 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         float tmax = -__builtin_inff();
 #pragma unroll
         for (int e = 0; e < NSC; ++e) {
-            float s;
+            float s, s2 = 0.0f;
             if (GP == 4) {
                 const float s0 = (cls & 1) ? acc[0][2 + e] : acc[0][e];
                 const float s1 = (cls & 1) ? acc[1][2 + e] : acc[1][e];
                 s = (cls >> 1) ? s1 : s0;
+                if (PROD) {
+                    const float u0 = (cls & 1) ? acc_s[0][2 + e] : acc_s[0][e];
+                    const float u1 = (cls & 1) ? acc_s[1][2 + e] : acc_s[1][e];
+                    s2 = (cls >> 1) ? u1 : u0;
+                }
             } else if (GP == 8) {
                 s = cls ? acc[1][e] : acc[0][e];
+                if (PROD) s2 = cls ? acc_s[1][e] : acc_s[0][e];
             } else {
                 s = acc[e >> 2][e & 3];
+                if (PROD) s2 = acc_s[e >> 2][e & 3];
             }
             const bool live = t0 + sc_tok[e] < end;
             rv[e] = live ? vn[e] : 0.0f;
-            a_[e] = live ? s * kn[e] * qscale : -__builtin_inff();
+            float sc = s * kn[e] * qscale;
+            if (PROD) sc = __builtin_fmaf(s2 * kg[e], qscale_s, sc);
+            a_[e] = live ? sc : -__builtin_inff();
             tmax = __builtin_fmaxf(tmax, a_[e]);
         }
         tmax = max_same_head<GP>(tmax);
@@ -1141,16 +1234,38 @@ int launch_with_lds(K kernel, const DecodeParams& p, dim3 grid, dim3 block, size
     return fq_host::check_launch();
 }
 
-// The staged kernel covers 8 KV heads of dimension 128 sharing one codebook.
-inline bool staged_applies(int D, int H_KV, bool two_tables) {
-    return D == 128 && H_KV == 8 && !two_tables && !fq_host::force_direct_decode();
+// The staged kernel covers 8 KV heads of dimension 128.
+inline bool staged_applies(int D, int H_KV) {
+    return D == 128 && H_KV == 8 && !fq_host::force_direct_decode();
 }
 
-template <typename K>
+template <bool PROD, typename K>
 int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream) {
     // dynamic part only; the 64 KB table is static
-    const size_t lds = 2 * size_t(kTileBytes);
+    const size_t lds = 2 * size_t(StagedCfg<PROD>::TILE_BYTES);
     return launch_with_lds(kernel, p, dim3(p.num_splits, S, 1), dim3(512), lds, stream);
+}
+
+// Staged kernel for every page size and group size; PROD selects the TurboQuantProd page format.
+template <int DT, bool PROD>
+int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream_t stream) {
+#define FQ_STAGED_GP(BSL, GPV)                                                                                  \
+    return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD>, p, S, stream)        \
+                : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD>, p, S, stream)
+#define FQ_STAGED_BS(BSL)                         \
+    do {                                          \
+        if (p.G <= 4) { FQ_STAGED_GP(BSL, 4); }   \
+        else if (p.G <= 8) { FQ_STAGED_GP(BSL, 8); } \
+        else { FQ_STAGED_GP(BSL, 16); }           \
+    } while (0)
+    switch (BS) {
+        case 8: FQ_STAGED_BS(3); break;
+        case 16: FQ_STAGED_BS(4); break;
+        default: FQ_STAGED_BS(5); break;
+    }
+#undef FQ_STAGED_BS
+#undef FQ_STAGED_GP
+    return FQ_ERR_UNSUPPORTED_BLOCK;
 }
 
 template <int D, int DT>
@@ -1160,24 +1275,7 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
     const int64_t chunk = (((max_ctx + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
     const bool wide = chunk / BS > 64;   // begin is a multiple of 64 tokens, hence page aligned
 
-    if (staged_applies(D, p.H_KV, p.two_tables != 0)) {
-#define FQ_STAGED_GP(BSL, GPV)                                                                      \
-    return wide ? launch_staged(paged_decode_staged_kernel<BSL, GPV, DT, 4>, p, S, stream)         \
-                : launch_staged(paged_decode_staged_kernel<BSL, GPV, DT, 1>, p, S, stream)
-#define FQ_STAGED_BS(BSL)                         \
-    do {                                          \
-        if (p.G <= 4) { FQ_STAGED_GP(BSL, 4); }   \
-        else if (p.G <= 8) { FQ_STAGED_GP(BSL, 8); } \
-        else { FQ_STAGED_GP(BSL, 16); }           \
-    } while (0)
-        switch (BS) {
-            case 8: FQ_STAGED_BS(3); break;
-            case 16: FQ_STAGED_BS(4); break;
-            default: FQ_STAGED_BS(5); break;
-        }
-#undef FQ_STAGED_BS
-#undef FQ_STAGED_GP
-    }
+    if (staged_applies(D, p.H_KV)) return launch_staged_any<DT, false>(p, S, BS, wide, stream);
 
     const int waves = p.H_KV < 8 ? p.H_KV : 8;
     const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
@@ -1342,7 +1440,7 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
         (rotation && !fq_host::aligned(rotation, 16)))
         return FQ_ERR_MISALIGNED;
     DecodeParams p;
-    p.q_rot = q; p.rotation = rotation; p.rot_col_major = rotation_col_major; p.cache = kv_cache; p.block_table = block_table; p.seq_lens = seq_lens;
+    p.q_rot = q; p.rotation = rotation; p.sketch = nullptr; p.rot_col_major = rotation_col_major; p.cache = kv_cache; p.block_table = block_table; p.seq_lens = seq_lens;
     p.centroids_k = centroids_k; p.centroids_v = centroids_v;
     p.part_acc = partial_acc; p.part_m = partial_m; p.part_l = partial_l;
     p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.max_blocks = max_blocks_per_seq;
@@ -1365,7 +1463,8 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
 }  // namespace fq
 
 extern "C" int fq_paged_decode_fuses_rotation(int D, int H_KV, int shared_codebook) {
-    return fq::staged_applies(D, H_KV, shared_codebook == 0) ? 1 : 0;
+    (void)shared_codebook;   // both codebooks fit the kernel's table
+    return fq::staged_applies(D, H_KV) ? 1 : 0;
 }
 
 extern "C" int fq_paged_tq4_decode(const void* q, const float* rotation, int rotation_col_major,
@@ -1374,7 +1473,7 @@ extern "C" int fq_paged_tq4_decode(const void* q, const float* rotation, int rot
                                    float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D,
                                    int block_size, int max_blocks_per_seq, int64_t num_blocks, float sm_scale,
                                    int dtype, int num_splits, void* stream) {
-    if (rotation && !fq::staged_applies(D, H_KV, centroids_k != centroids_v)) return FQ_ERR_BAD_SHAPE;
+    if (rotation && !fq::staged_applies(D, H_KV)) return FQ_ERR_BAD_SHAPE;
     return fq::decode_partials(q, rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k,
                                centroids_v, partial_acc, partial_m, partial_l, num_seqs, H_Q, H_KV, D, block_size,
                                max_blocks_per_seq, num_blocks, sm_scale, dtype, num_splits, stream);
@@ -1419,7 +1518,7 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     const void* q_in = q;
     const float* fused_rotation = nullptr;
     if (rotation) {
-        if (centroids_k && staged_applies(D, H_KV, centroids_k != centroids_v)) {
+        if (centroids_k && staged_applies(D, H_KV)) {
             fused_rotation = rotation;       // the staged kernel rotates the query in its prologue
         } else {
             const int st = fq_rotate_query(q, rotation, rotation_col_major, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
@@ -1430,6 +1529,54 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     int st = decode_partials(q_in, fused_rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m,
                              l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
                              num_splits, stream);
+    if (st != FQ_OK) return st;
+    return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_splits, stream);
+}
+
+// TurboQuantProd pages: 3-bit keys with a sign-sketch correction of the scores, TQ4 values.
+extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
+                                    const int32_t* seq_lens, const float* centroids_k3,
+                                    const float* centroids_v, const float* rotation, int rotation_col_major,
+                                    const float* sketch, void* out, int num_seqs, int H_Q, int H_KV, int D,
+                                    int block_size, int max_blocks_per_seq, int64_t num_blocks, float sm_scale,
+                                    int dtype, int num_splits, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
+    using namespace fq;
+    const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
+                                       num_splits);
+    if (bad != FQ_OK) return bad;
+    if (D != 128) return FQ_ERR_UNSUPPORTED_DIM;
+    if (H_KV != 8 || H_Q > 64) return FQ_ERR_BAD_SHAPE;   // the kernel stages 8 KV heads per token row
+    if (num_seqs == 0) return FQ_OK;
+    if (!q || !out || !kv_cache || !block_table || !seq_lens || !centroids_k3 || !centroids_v || !rotation || !sketch)
+        return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16) || !fq_host::aligned(kv_cache, 16) ||
+        !fq_host::aligned(rotation, 16) || !fq_host::aligned(sketch, 16))
+        return FQ_ERR_MISALIGNED;
+    num_splits = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
+    const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_splits);
+    if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
+    if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    float* acc = reinterpret_cast<float*>(ws + w.acc);
+    float* m = reinterpret_cast<float*>(ws + w.m);
+    float* l = reinterpret_cast<float*>(ws + w.l);
+
+    DecodeParams p;
+    p.q_rot = q; p.rotation = rotation; p.sketch = sketch; p.rot_col_major = rotation_col_major;
+    p.cache = kv_cache; p.block_table = block_table; p.seq_lens = seq_lens;
+    p.centroids_k = centroids_k3; p.centroids_v = centroids_v;
+    p.part_acc = acc; p.part_m = m; p.part_l = l;
+    p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.max_blocks = max_blocks_per_seq;
+    p.num_blocks = int(num_blocks); p.num_splits = num_splits;
+    p.two_tables = 1;
+    p.scale_log2e = sm_scale * kLog2e;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t max_ctx = int64_t(max_blocks_per_seq) * block_size;
+    const int64_t chunk = (((max_ctx + num_splits - 1) / num_splits) + 63) & ~int64_t(63);
+    const bool wide = chunk / block_size > 64;
+    const int st = dtype == FQ_F16 ? launch_staged_any<FQ_F16, true>(p, num_seqs, block_size, wide, s)
+                                   : launch_staged_any<FQ_BF16, true>(p, num_seqs, block_size, wide, s);
     if (st != FQ_OK) return st;
     return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_splits, stream);
 }

@@ -177,7 +177,7 @@ int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
  * fq_paged_tq4_decode: q pre-rotated and rotation NULL, or q un-rotated with the rotation,
  *                      which the kernel then applies itself: allowed only where
  *                      fq_paged_decode_fuses_rotation() returns 1 (8 KV heads of dimension
- *                      128 sharing one codebook), FQ_ERR_BAD_SHAPE elsewhere.
+ *                      128), FQ_ERR_BAD_SHAPE elsewhere.
  *                      Writes un-normalised float32 partials
  *                      partial_acc (num_seqs, H_Q, num_splits, D) and the base-2 running
  *                      maximum / denominator partial_m, partial_l (num_seqs, H_Q, num_splits);
@@ -205,6 +205,38 @@ int fq_split_k_reduce(const float* partial_acc, const float* partial_m,
                       int rotation_col_major, void* out,
                       int num_seqs, int H_Q, int D, int dtype, int num_splits,
                       void* stream);
+
+/*
+ * TurboQuantProd keys (3-bit Lloyd-Max index + 1-bit sign sketch of the residual) with
+ * TQ4 values, as pages.  The reference defines the quantizer
+ * (TurboQuantProd.quantize / estimate_inner_product, src/flashquant/core/quantizer.py:285-370;
+ * C++ twin csrc/core/quantizer.cpp:76-184) but has no paged or fused path for it, so the
+ * packed record is this library's own:
+ *
+ *   key nibble   = sign_bit << 3 | index (sign_bit 1 where resid . S_j < 0), two per byte,
+ *                  even coordinate in the high nibble
+ *   token row    = [K nibbles H*D/2 | K norm H*4 | K residual norm H*4 | V idx H*D/2 | V norm H*4],
+ *                  H*(D+12) bytes, norms little-endian float32
+ *
+ * fq_prod_compress: x (M, D) fp16/bf16 -> packed (M, D/2) uint8, norms (M,), residual_norms (M,).
+ *   rotation    (D, D) float32 R, layout flag as in fq_split_k_paged_decode
+ *   sketch_rot  (D, D) float32 row-major, S @ R.T for the (D, D) sketch S (computed once by the caller)
+ *   boundaries  (7,), centroids (8,) float32: the 3-bit codebook
+ * fq_prod_paged_decode: split-K decode over such pages, un-rotated query in, original-space
+ *   output out: score = <q, k_mse> + gamma sqrt(pi/2)/D <S q, signs> (quantizer.py:355-370),
+ *   softmax, TQ4 values.  sketch is S itself, (D, D) row-major.  Workspace and num_splits as in
+ *   fq_split_k_paged_decode.  D == 128, H_KV == 8, H_Q <= 64.
+ */
+int fq_prod_compress(const void* x, int x_dtype, const float* rotation, int rotation_col_major,
+                     const float* sketch_rot, const float* boundaries, const float* centroids,
+                     uint8_t* packed, float* norms, float* residual_norms, int64_t M, int D, void* stream);
+
+int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
+                         const int32_t* seq_lens, const float* centroids_k3, const float* centroids_v,
+                         const float* rotation, int rotation_col_major, const float* sketch, void* out,
+                         int num_seqs, int H_Q, int H_KV, int D, int block_size, int max_blocks_per_seq,
+                         int64_t num_blocks, float sm_scale, int dtype, int num_splits,
+                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* Number of splits fq_split_k_paged_decode uses when num_splits == 0
  * (counterpart of paged_tq4_decode_num_splits, csrc/cuda/paged_decode.cu:424-426,

@@ -549,3 +549,98 @@ def prod_inner_product(
     q_proj = (query.float().reshape(-1, d) @ sketch.T).reshape(*query.shape[:-1], m)
     corr = (q_proj * signs).sum(dim=-1, keepdim=True)
     return first + residual_norms * math.sqrt(math.pi / 2.0) / m * corr
+
+
+# ---------------------------------------------------------------------------
+# TurboQuantProd keys + TQ4 values as pages (a composition: the reference has
+# the quantizer, src/flashquant/core/quantizer.py:270-370, but no paged path)
+# ---------------------------------------------------------------------------
+
+
+def prod_pack_keys(indices: torch.Tensor, signs: torch.Tensor) -> torch.Tensor:
+    """Key nibble = sign_bit << 3 | 3-bit index (sign_bit 1 for a -1 sign),
+    packed two per byte like nibble_pack (even coordinate in the high nibble)."""
+    nib = indices.long() | ((signs < 0).long() << 3)
+    return nibble_pack(nib)
+
+
+def prod_page_layout(num_kv_heads: int, head_dim: int) -> Tuple[int, int, int, int, int]:
+    """Offsets (k_norm, k_gamma, v_idx, v_norm, row_bytes) of the token row
+    [K nibbles | K norms | K residual norms | V idx | V norms]."""
+    k_norm = num_kv_heads * (head_dim // 2)
+    k_gamma = k_norm + NORM_BYTES * num_kv_heads
+    v_idx = k_gamma + NORM_BYTES * num_kv_heads
+    v_norm = v_idx + num_kv_heads * (head_dim // 2)
+    return k_norm, k_gamma, v_idx, v_norm, v_norm + NORM_BYTES * num_kv_heads
+
+
+def prod_store_rows(kv_cache, slot_mapping, k_packed, k_norms, k_gamma, v_packed, v_norms) -> None:
+    n, h, half = k_packed.shape
+    k_norm, k_gam, v_idx, v_norm, row_bytes = prod_page_layout(h, 2 * half)
+    row = torch.empty(n, row_bytes, dtype=torch.uint8)
+    row[:, :k_norm] = k_packed.reshape(n, -1)
+    row[:, k_norm:k_gam] = k_norms.reshape(n, h).contiguous().view(torch.uint8)
+    row[:, k_gam:v_idx] = k_gamma.reshape(n, h).contiguous().view(torch.uint8)
+    row[:, v_idx:v_norm] = v_packed.reshape(n, -1)
+    row[:, v_norm:] = v_norms.reshape(n, h).contiguous().view(torch.uint8)
+    kv_cache.view(-1, row_bytes)[slot_mapping.long()] = row
+
+
+def prod_paged_decode(
+    q: torch.Tensor,
+    kv_cache: torch.Tensor,
+    block_table: torch.Tensor,
+    seq_lens: torch.Tensor,
+    centroids_k3: torch.Tensor,
+    centroids_v: torch.Tensor,
+    rotation: torch.Tensor,
+    sketch: torch.Tensor,
+    num_kv_heads: int,
+    head_dim: int,
+    block_size: int,
+    sm_scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Decode over TurboQuantProd key / TQ4 value pages.
+
+    Score of a key = TurboQuantProd.estimate_inner_product
+    (src/flashquant/core/quantizer.py:355-370): <q, k_mse> + gamma sqrt(pi/2)/m
+    <S q, signs>, with <q, k_mse> evaluated in rotated space as norm * <q_rot,
+    centroids[idx]> and q_rot = (q @ R.T) rounded to q.dtype as the TQ4 decode
+    dispatcher rounds it (src/flashquant/kernels/paged_decode.py:113).  Values are
+    TQ4 in rotated space; the result is rounded to q.dtype, multiplied by R and
+    rounded again (paged_decode.py:123).  A sequence of length 0 gives zeros.
+    """
+    s_count, hq, d = q.shape
+    m = sketch.shape[0]
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(head_dim)
+    half = head_dim // 2
+    k_norm, k_gam, v_idx, v_norm, row_bytes = prod_page_layout(num_kv_heads, head_dim)
+    rep = hq // num_kv_heads
+    q_rot = torch.matmul(q.float(), rotation.T).to(q.dtype).float()
+    q_s = torch.matmul(q.float(), sketch.T)
+    out_rot = torch.zeros(s_count, hq, d, dtype=q.dtype)
+    for s in range(s_count):
+        length = int(seq_lens[s])
+        if length == 0:
+            continue
+        t = torch.arange(length)
+        pages = block_table[s].long()[t // block_size]
+        rows = kv_cache.view(-1, row_bytes)[pages * block_size + (t % block_size)]
+        nib = nibble_unpack(rows[:, :k_norm].reshape(length, num_kv_heads, half))
+        idx, sign = nib & 7, 1.0 - 2.0 * (nib >> 3).float()
+        kn = rows[:, k_norm:k_gam].contiguous().view(torch.float32).reshape(length, num_kv_heads, 1)
+        kg = rows[:, k_gam:v_idx].contiguous().view(torch.float32).reshape(length, num_kv_heads, 1)
+        vb = rows[:, v_idx:v_norm].reshape(length, num_kv_heads, half)
+        vn = rows[:, v_norm:].contiguous().view(torch.float32).reshape(length, num_kv_heads, 1)
+        k_mse = (centroids_k3[idx] * kn).permute(1, 0, 2)                 # (H, L, D), rotated space
+        sg = (sign * kg * (math.sqrt(math.pi / 2.0) / m)).permute(1, 0, 2)   # (H, L, m)
+        v = decompress(vb, vn, centroids_v).permute(1, 0, 2)
+        if rep > 1:
+            k_mse = k_mse.repeat_interleave(rep, dim=0)
+            sg = sg.repeat_interleave(rep, dim=0)
+            v = v.repeat_interleave(rep, dim=0)
+        sc = torch.bmm(q_rot[s].unsqueeze(1), k_mse.transpose(-2, -1)) + torch.bmm(q_s[s].unsqueeze(1), sg.transpose(-2, -1))
+        w = torch.softmax(sc * sm_scale, dim=-1)
+        out_rot[s] = torch.bmm(w, v).squeeze(1).to(q.dtype)
+    return torch.matmul(out_rot.float(), rotation).to(q.dtype)

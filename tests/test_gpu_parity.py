@@ -375,3 +375,114 @@ def test_compress_and_store_rejects_bad_arguments():
         K.tq4_compress_and_store(key, key, r.to(DEV), bnd.to(DEV), cache[..., :100], slots)    # wrong row size
     with pytest.raises(ValueError):
         K.tq4_compress_and_store(key, key, r.to(DEV), bnd.to(DEV), cache, torch.arange(5, device=DEV))  # too many slots
+
+
+# ---- TurboQuantProd keys (3-bit + sign sketch) with TQ4 values --------------------------------
+
+def _prod_books():
+    c3, b3 = O.lloyd_max_gaussian(128, 3)
+    c4, b4 = O.lloyd_max_gaussian(128, 4)
+    return c3, b3, c4, b4, O.haar_orthogonal(128, 42), O.qjl_matrix(128, 42)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_prod_compress_parity(dtype):
+    c3, b3, c4, b4, r, s = _prod_books()
+    x = outlier_rows(1500, 8, 128, 101, dtype=dtype)
+    x[7] = 0                                     # zero rows: index of 0, all signs +
+    idx, kn, sg, gam = O.prod_quantize(x, r, b3, c3, s)
+    want = O.prod_pack_keys(idx, sg)
+    packed, norms, gamma = K.prod_compress(x.to(DEV), r.to(DEV), s.to(DEV), b3.to(DEV), c3.to(DEV))
+    torch.cuda.synchronize()
+    nib_g, nib_w = O.nibble_unpack(packed.cpu()), O.nibble_unpack(want)
+    idx_bad = ((nib_g & 7) != (nib_w & 7)).float().mean().item()
+    sign_bad = ((nib_g >> 3) != (nib_w >> 3)).float().mean().item()
+    assert idx_bad <= 1e-4, f"index mismatch rate {idx_bad}"
+    assert sign_bad <= 1e-4, f"sign mismatch rate {sign_bad}"
+    assert torch.allclose(norms.cpu(), kn, rtol=1e-5, atol=1e-30)
+    assert torch.allclose(gamma.cpu(), gam, rtol=2e-4, atol=1e-6)
+    assert torch.equal(nib_g[7], torch.full_like(nib_g[7], int((b3 < 0).sum())))
+
+
+def _prod_case(lens, hq, bs=16, seed=7, dtype=torch.bfloat16, extra_blocks=2):
+    c3, b3, c4, b4, r, s = _prod_books()
+    hkv, d = 8, 128
+    g = torch.Generator().manual_seed(seed)
+    S = len(lens)
+    max_blocks = max(1, (max(lens) + bs - 1) // bs)
+    nb = S * max_blocks + extra_blocks
+    row_bytes = O.prod_page_layout(hkv, d)[4]
+    cache = torch.randint(0, 256, (nb, bs, row_bytes), dtype=torch.uint8, generator=g)
+    table = torch.randperm(nb, generator=g)[: S * max_blocks].reshape(S, max_blocks).int()
+    for i, L in enumerate(lens):
+        if L == 0:
+            continue
+        k = torch.randn(L, hkv, d, generator=g)
+        v = torch.randn(L, hkv, d, generator=g)
+        idx, kn, sg, gam = O.prod_quantize(k, r, b3, c3, s)
+        vp, vn = O.compress(v, r, b4)
+        t = torch.arange(L)
+        O.prod_store_rows(cache, table[i].long()[t // bs] * bs + t % bs, O.prod_pack_keys(idx, sg), kn, gam, vp, vn)
+    q = torch.randn(S, hq, d, generator=g).to(dtype)
+    return q, cache, table, torch.tensor(lens, dtype=torch.int32)
+
+
+def _check_prod_decode(lens, hq, bs=16, num_splits=0, dtype=torch.bfloat16, seed=7):
+    c3, b3, c4, b4, r, s = _prod_books()
+    q, cache, table, sl = _prod_case(lens, hq, bs, seed, dtype)
+    want = O.prod_paged_decode(q, cache, table, sl, c3, c4, r, s, 8, 128, bs)
+    got = K.prod_paged_decode(q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), c3.to(DEV), c4.to(DEV), r.to(DEV),
+                              s.to(DEV), 8, 128, bs, num_splits=num_splits)
+    torch.cuda.synchronize()
+    err = (got.cpu().float() - want.float()).abs().max().item()
+    assert err <= 2e-2, f"max abs error {err}"
+
+
+@pytest.mark.parametrize("hq", [8, 32, 64])
+@pytest.mark.parametrize("num_splits", [0, 1, 5])
+def test_prod_paged_decode_group_sizes_and_splits(hq, num_splits):
+    _check_prod_decode([300, 1, 77, 0, 129], hq, num_splits=num_splits)
+
+
+@pytest.mark.parametrize("bs", [8, 16, 32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_prod_paged_decode_page_sizes(bs, dtype):
+    _check_prod_decode([200, 33], 64, bs=bs, dtype=dtype, seed=9)
+
+
+def test_prod_compress_store_decode_end_to_end():
+    c3, b3, c4, b4, r, s = _prod_books()
+    hkv, hq, d, bs, L = 8, 64, 128, 16, 500
+    g = torch.Generator().manual_seed(13)
+    k = torch.randn(L, hkv, d, generator=g).to(torch.bfloat16)
+    v = torch.randn(L, hkv, d, generator=g).to(torch.bfloat16)
+    q = torch.randn(1, hq, d, generator=g).to(torch.bfloat16)
+    nb = (L + bs - 1) // bs + 1
+    table = torch.randperm(nb, generator=g)[: (L + bs - 1) // bs].reshape(1, -1).int()
+    t = torch.arange(L)
+    slots = table[0].long()[t // bs] * bs + t % bs
+    kp, kn, kg = K.prod_compress(k.to(DEV), r.to(DEV), s.to(DEV), b3.to(DEV), c3.to(DEV))
+    vp, vn = K.tq4_compress(v.to(DEV), r.to(DEV), b4.to(DEV))
+    cache = torch.zeros(nb, bs, K.prod_page_layout(hkv, d)[4], dtype=torch.uint8, device=DEV)
+    K.prod_store_rows(cache, slots.to(DEV), kp, kn, kg, vp, vn)
+    sl = torch.tensor([L], dtype=torch.int32)
+    got = K.prod_paged_decode(q.to(DEV), cache, table.to(DEV), sl.to(DEV), c3.to(DEV), c4.to(DEV), r.to(DEV), s.to(DEV),
+                              hkv, d, bs)
+    idx, on, sg, gam = O.prod_quantize(k, r, b3, c3, s)
+    ovp, ovn = O.compress(v, r, b4)
+    cache_ref = torch.zeros(nb, bs, O.prod_page_layout(hkv, d)[4], dtype=torch.uint8)
+    O.prod_store_rows(cache_ref, slots, O.prod_pack_keys(idx, sg), on, gam, ovp, ovn)
+    want = O.prod_paged_decode(q, cache_ref, table, sl, c3, c4, r, s, hkv, d, bs)
+    assert (got.cpu().float() - want.float()).abs().max().item() <= 2e-2
+
+
+def test_prod_entry_points_reject_unsupported_shapes():
+    c3, b3, c4, b4, r, s = _prod_books()
+    q = torch.zeros(1, 8, 128, dtype=torch.bfloat16, device=DEV)
+    cache = torch.zeros(2, 16, 4 * 140, dtype=torch.uint8, device=DEV)
+    table = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
+    sl = torch.ones(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError):          # 4 KV heads: the kernel stages rows of 8
+        K.prod_paged_decode(q, cache, table, sl, c3.to(DEV), c4.to(DEV), r.to(DEV), s.to(DEV), 4, 128, 16)
+    with pytest.raises(ValueError):          # 4-bit codebook where the 3-bit one is expected
+        K.prod_compress(torch.zeros(4, 8, 128, dtype=torch.bfloat16, device=DEV), r.to(DEV), s.to(DEV), b4.to(DEV), c4.to(DEV))

@@ -251,3 +251,40 @@ def test_prod_estimator_unbiased():
     assert abs((est - true).mean().item()) / true.abs().mean().item() < 0.05
     mse_only = (q * O.mse_dequantize(idx, norms, r, c3)).sum(-1)
     assert abs((est - true).mean()) < abs((mse_only - true).mean()) + 0.05
+
+
+# ---- TurboQuantProd pages (composition) ---------------------------------------------
+
+def test_prod_page_scores_equal_the_estimator_formula():
+    """prod_paged_decode's scores are prod_inner_product's, through the packed page."""
+    import math
+    d, h, L, bs = 128, 2, 37, 16
+    c3, b3 = O.lloyd_max_gaussian(d, 3)
+    c4, b4 = O.lloyd_max_gaussian(d, 4)
+    r = O.haar_orthogonal(d, 42)
+    s = O.qjl_matrix(d, 42)
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn(L, h, d, generator=g)
+    v = torch.randn(L, h, d, generator=g)
+    q = torch.randn(1, h, d, generator=g)          # one query head per KV head, float32: no rounding of q_rot
+    idx, kn, sg, gam = O.prod_quantize(k, r, b3, c3, s)
+    assert int(idx.max()) <= 7 and set(sg.unique().tolist()) <= {-1.0, 1.0}
+    kp = O.prod_pack_keys(idx, sg)
+    # the nibble carries both fields
+    nib = O.nibble_unpack(kp)
+    assert torch.equal(nib & 7, idx) and torch.equal(1.0 - 2.0 * (nib >> 3).float(), sg)
+    vp, vn = O.compress(v, r, b4)
+    nb = (L + bs - 1) // bs
+    cache = torch.zeros(nb, bs, O.prod_page_layout(h, d)[4], dtype=torch.uint8)
+    table = torch.arange(nb).flip(0).reshape(1, nb).int()
+    t = torch.arange(L)
+    O.prod_store_rows(cache, table[0].long()[t // bs] * bs + t % bs, kp, kn, gam, vp, vn)
+    got = O.prod_paged_decode(q, cache, table, torch.tensor([L], dtype=torch.int32), c3, c4, r, s, h, d, bs)
+    # explicit: estimator scores -> softmax -> original-space TQ4 values
+    want = torch.zeros(1, h, d)
+    for head in range(h):
+        sc = O.prod_inner_product(q[0, head].expand(L, d), idx[:, head], kn[:, head], sg[:, head], gam[:, head], r, c3, s)
+        w = torch.softmax(sc.reshape(L) / math.sqrt(d), dim=0)
+        vv = O.mse_dequantize(O.nibble_unpack(vp[:, head]), vn[:, head], r, c4)
+        want[0, head] = w @ vv
+    assert (got - want).abs().max().item() < 2e-5
