@@ -117,6 +117,6 @@ def test_split_count_rules(lib):
 
 def test_rotation_fusion_rule(lib):
     assert lib.fq_paged_decode_fuses_rotation(128, 8, 1) == 1
-    assert lib.fq_paged_decode_fuses_rotation(128, 8, 0) == 0
+    assert lib.fq_paged_decode_fuses_rotation(128, 8, 0) == 1    # distinct K and V codebooks share the table
     assert lib.fq_paged_decode_fuses_rotation(64, 8, 1) == 0
     assert lib.fq_paged_decode_fuses_rotation(128, 4, 1) == 0
