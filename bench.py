@@ -273,6 +273,61 @@ def main():
             "prefill_tokens_per_s": pb * pn / (p_ms * 1e-3),
         })
         del q3, kp3, kn3, vp3, vn3
+        torch.cuda.empty_cache()
+
+        # ---- long-context decode over TurboQuantProd key / TQ4 value pages (configs[4]) ----------
+        # batch 8, 64 query heads over 8, ragged contexts U{16K..128K} (seed 1004), 16-token pages
+        hq4, b4 = 64, 8
+        c3, b3 = O.lloyd_max_gaussian(D, 3)
+        sk = O.qjl_matrix(D, 42)
+        c3_d, b3_d, sk_d = c3.to(dev), b3.to(dev), sk.to(dev)
+        g4 = torch.Generator(device="cpu").manual_seed(1004)
+        lens4 = torch.randint(16384, 131072 + 1, (b4,), generator=g4)
+        pages4 = (lens4 + BS - 1) // BS
+        max_pages = int(pages4.max())
+        total_pages = int(pages4.sum())
+        row4 = K.prod_page_layout(H_KV, D)[4]
+        cache4 = torch.zeros(total_pages, BS, row4, dtype=torch.uint8, device=dev)
+        perm = torch.randperm(total_pages, generator=g4)
+        table4 = torch.zeros(b4, max_pages, dtype=torch.int32)
+        w_rot = None
+        first = 0
+        for s_i in range(b4):
+            L = int(lens4[s_i])
+            npg = int(pages4[s_i])
+            table4[s_i, :npg] = perm[first:first + npg].to(torch.int32)
+            first += npg
+            t = torch.arange(L)
+            slots = (table4[s_i].long()[t // BS] * BS + t % BS).to(dev)
+            kx = outlier_rows(L, H_KV, D, 1400 + s_i, dev)
+            vx = outlier_rows(L, H_KV, D, 1500 + s_i, dev)
+            kp4, kn4, kg4 = K.prod_compress(kx, rot_d, sk_d, b3_d, c3_d)
+            vp4, vn4 = K.tq4_compress(vx, rot_d, bnd_d)
+            K.prod_store_rows(cache4, slots, kp4, kn4, kg4, vp4, vn4)
+            del kx, vx, kp4, kn4, kg4, vp4, vn4
+        table4 = table4.to(dev)
+        lens4_d = lens4.to(torch.int32).to(dev)
+        q4 = torch.randn(b4, hq4, D, generator=torch.Generator(device="cpu").manual_seed(1044)).to(torch.bfloat16).to(dev)
+        out4 = torch.empty_like(q4)
+
+        def prod_step(i):
+            K.prod_paged_decode(q4, cache4, table4, lens4_d, c3_d, cent_d, rot_d, sk_d, H_KV, D, BS,
+                                sm_scale=scale, out=out4)
+
+        for i in range(3):
+            prod_step(i)
+        pd_ms = time_events(prod_step, 10)
+        prod_bytes = int(lens4.sum()) * row4
+        extra.update({
+            "prod_decode_ms": pd_ms,
+            "prod_decode_gbps": prod_bytes / (pd_ms * 1e-3) / 1e9,
+            "prod_decode_pct_hbm_peak": 100.0 * prod_bytes / (pd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "prod_decode_tokens_per_s": b4 / (pd_ms * 1e-3),
+            "prod_context_tokens": int(lens4.sum()),
+            "prod_bytes_per_token_per_kv_head": row4 // H_KV,
+            "prod_cache_bytes": prod_bytes,
+        })
+        del cache4
 
     value = kv_bytes / (step_ms * 1e-3) / 1e9
     line = {
