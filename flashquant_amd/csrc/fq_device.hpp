@@ -61,14 +61,22 @@ __device__ __forceinline__ void fill_byte_table(uint32_t* table, float mine, int
 // table in the upper 128 bytes.  A K nibble is looked up as `nibble & k_mask` (15 for TQ4,
 // 7 when bit 3 of the nibble is a sign bit), a V nibble as it is.  Lane l holds
 // k_centroids[l & k_mask] and v_centroids[l & 15].
+template <int WAVES>
 __device__ __forceinline__ void fill_pair_tables(uint32_t* table, float mine_k, float mine_v, int k_mask, int wave,
-                                                 int waves, int lane) {
-    for (int byte = wave; byte < 256; byte += waves) {
-        const float khi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_k), (byte >> 4) & k_mask));
-        const float klo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_k), byte & k_mask));
-        const float vhi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_v), byte >> 4));
-        const float vlo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_v), byte & 15));
-        table[byte * 64 + lane] = lane < 32 ? pack_h2(_Float16(khi), _Float16(klo)) : pack_h2(_Float16(vhi), _Float16(vlo));
+                                                 int lane) {
+    // the fp16 centroid of this lane; entries are then assembled on the scalar unit
+    const int hk = int(__builtin_bit_cast(uint16_t, _Float16(mine_k)));
+    const int hv = int(__builtin_bit_cast(uint16_t, _Float16(mine_v)));
+    uint32_t* mine = table + lane;
+#pragma unroll
+    for (int i = 0; i < 256 / WAVES; ++i) {
+        const int byte = wave + WAVES * i;
+        const uint32_t khi = uint32_t(__builtin_amdgcn_readlane(hk, (byte >> 4) & k_mask));
+        const uint32_t klo = uint32_t(__builtin_amdgcn_readlane(hk, byte & k_mask));
+        const uint32_t vhi = uint32_t(__builtin_amdgcn_readlane(hv, byte >> 4));
+        const uint32_t vlo = uint32_t(__builtin_amdgcn_readlane(hv, byte & 15));
+        const uint32_t ke = khi | (klo << 16), ve = vhi | (vlo << 16);
+        mine[wave * 64 + WAVES * 64 * i] = lane < 32 ? ke : ve;
     }
 }
 __device__ __forceinline__ void build_byte_table(uint32_t* table, const float* __restrict__ centroids, int wave,
@@ -156,6 +164,79 @@ __device__ __forceinline__ float4v rotate_block(const float (&a)[D / 32][8], con
         for (int e = 0; e < 8; ++e)
             acc[e & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j][e], b[j][e], acc[e & 3], 0, 0, 0);
     return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+}
+
+// ---------------------------------------------------------------------------------------
+// The same rotations on the fp16 MFMA (v_mfma_f32_16x16x32_f16), 8 times the rate of the
+// float32 one.  The matrix block is split once into two fp16 terms, b = hi + lo / 4096
+// (22 significant bits); a row operand that is exact in fp16 after scaling by a power of
+// two (fp16 / bf16 data) needs no split, so a block costs 2 MFMAs per 32 contraction
+// indices and the products are exact.  Operand layout as rotate_block: lane (m, g) holds
+// k = 32 j + 8 g + e.
+// ---------------------------------------------------------------------------------------
+template <int D>
+__device__ __forceinline__ void split_rotation_block(const float (&b)[D / 32][8], half8 (&hi)[D / 32],
+                                                     half8 (&lo)[D / 32]) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            // any rounding of the high term will do: the low term takes up the remainder
+            const auto h2 = __builtin_amdgcn_cvt_pkrtz(b[j][e], b[j][e + 1]);
+            const auto l2 = __builtin_amdgcn_cvt_pkrtz((b[j][e] - float(h2[0])) * 4096.0f, (b[j][e + 1] - float(h2[1])) * 4096.0f);
+            hi[j][e] = h2[0]; hi[j][e + 1] = h2[1];
+            lo[j][e] = l2[0]; lo[j][e + 1] = l2[1];
+        }
+}
+
+template <int D>
+__device__ __forceinline__ float4v rotate_block_f16(const half8 (&a)[D / 32], const half8 (&bhi)[D / 32],
+                                                    const half8 (&blo)[D / 32]) {
+    float4v acc_hi = {0.f, 0.f, 0.f, 0.f}, acc_lo = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+        acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], bhi[j], acc_hi, 0, 0, 0);
+        acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], blo[j], acc_lo, 0, 0, 0);
+    }
+    return acc_hi + acc_lo * (1.0f / 4096.0f);
+}
+
+// Wavefront-wide maximum (all 64 lanes receive it), in the VALU: rotations inside the rows
+// of 16 lanes, then the row swaps.
+__device__ __forceinline__ float wave_max(float v) {
+    v = __builtin_fmaxf(v, dpp_mov<0x121>(v));   // row_ror:1
+    v = __builtin_fmaxf(v, dpp_mov<0x122>(v));   // row_ror:2
+    v = __builtin_fmaxf(v, dpp_mov<0x124>(v));   // row_ror:4
+    v = __builtin_fmaxf(v, dpp_mov<0x128>(v));   // row_ror:8
+    return max_xor32(max_xor16(v));
+}
+
+// 16-bit rows (fp16 / bf16 raw words, lane (m, g) holding k = 32 j + 8 g + e) as the fp16 A
+// operand, scaled by one power of two for the whole 16-row block so that the largest
+// element lies in [1, 2); `up` undoes the scaling on the result.
+template <int D, int DT>
+__device__ __forceinline__ void rows_as_f16(const uint4v (&raw)[D / 32], half8 (&a)[D / 32], float& up) {
+    float v[D / 32][8];
+    float mx = 0.0f;
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+        const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[j][2 * i] = load_elem<DT>(uint16_t(w[i] & 0xffffu));
+            v[j][2 * i + 1] = load_elem<DT>(uint16_t(w[i] >> 16));
+            mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(v[j][2 * i]), __builtin_fabsf(v[j][2 * i + 1])));
+        }
+    }
+    mx = wave_max(mx);
+    int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+    if (ex < -100 || ex > 100) ex = 0;
+    const float down = bits_to_float(uint32_t(127 - ex) << 23);
+    up = bits_to_float(uint32_t(127 + ex) << 23);
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[j][e] = _Float16(v[j][e] * down);
 }
 
 }  // namespace fq

@@ -103,7 +103,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     if (!unit_live) my_tiles = 0;
 
     // ---- tables -----------------------------------------------------------------------------
-    fill_pair_tables(lut, p.centroids_k[lane & 15], p.centroids_v[lane & 15], 15, w, 8, lane);
+    fill_pair_tables<8>(lut, p.centroids_k[lane & 15], p.centroids_v[lane & 15], 15, w, lane);
     const uint8_t* lutb = reinterpret_cast<const uint8_t*>(lut);
     const uint32_t lk = 4u * (lane & 31), lv = 128u + lk;
 

@@ -56,7 +56,7 @@
 #endif
 
 #ifdef FQ_DBG_TIMING
-#define FQ_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x == 3 && blockIdx.y == 5) tmark[i] = wall_clock64(); } while (0)
+#define FQ_MARK(i) do { if ((threadIdx.x & 63) == 0 && blockIdx.x == 3 && blockIdx.y == 5) tmark[i] = wall_clock64(); } while (0)
 #else
 #define FQ_MARK(i)
 #endif
@@ -171,8 +171,7 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
                 mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(qf[ks][2 * i]), __builtin_fabsf(qf[ks][2 * i + 1])));
             }
         }
-        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 16));
-        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 32));
+        mx = max_xor32(max_xor16(mx));
         int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
         if (ex < -100 || ex > 100) ex = 0;
         const float down = bits_to_float(uint32_t(127 - ex) << 23);
@@ -551,9 +550,9 @@ __host__ __device__ constexpr int staged_slot(int h, int r, int q) {
 
 // LDS byte offset (inside a tile slot) of the 16-byte chunk `ci` of tile row `row` (0..31).
 template <bool PROD>
-__device__ __forceinline__ int staged_chunk_dst(int row, int ci) {
+__host__ __device__ constexpr int staged_chunk_dst(int row, int ci) {
     const int stage = row >> 4, r = row & 15;
-    int off;
+    int off = 0;
     if (ci < 32) {
         off = 16 * staged_slot(ci >> 2, r, ci & 3);
     } else if (ci < 34) {
@@ -567,6 +566,19 @@ __device__ __forceinline__ int staged_chunk_dst(int row, int ci) {
     }
     return stage * StagedCfg<PROD>::STAGE_BYTES + off;
 }
+
+// The same offsets for every chunk of a tile, worked out at compile time: a thread reads its
+// five entries instead of dividing by the row length and walking the layout.
+template <bool PROD>
+struct ChunkDstTable {
+    uint16_t off[StagedCfg<PROD>::CHUNKS_PER_TILE];
+    constexpr ChunkDstTable() : off() {
+        for (int c = 0; c < StagedCfg<PROD>::CHUNKS_PER_TILE; ++c)
+            off[c] = uint16_t(staged_chunk_dst<PROD>(c / StagedCfg<PROD>::CHUNKS_PER_ROW, c % StagedCfg<PROD>::CHUNKS_PER_ROW));
+    }
+};
+template <bool PROD>
+__device__ const ChunkDstTable<PROD> kChunkDst{};
 
 // TurboQuantProd sign operand: the fp16 pairs (+-1, +-1) of the eight sign bits (bit 3 of
 // every nibble) of one key dword.  Element e of the result belongs to the coordinate
@@ -644,6 +656,19 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             for (int j = 0; j < 4; ++j) q_pre[rb][j] = *reinterpret_cast<const uint4v*>(qseq + row * 128 + 32 * j + 8 * g);
         }
     }
+    // Page ids.  When the whole block-table row fits the registers (64 * PVR pages) it is
+    // fetched now, before the sequence length is known, so that the two loads overlap;
+    // otherwise the registers hold the pages of this split, which depend on the length.
+    const int32_t* bt = p.block_table + int64_t(seq) * p.max_blocks;
+    const bool rowwide = p.max_blocks <= 64 * PVR;
+    int pv[PVR];
+    if (rowwide) {
+#pragma unroll
+        for (int r = 0; r < PVR; ++r) {
+            const int idx = 64 * r + lane < p.max_blocks ? 64 * r + lane : p.max_blocks - 1;
+            pv[r] = bt[idx];
+        }
+    }
     FQ_MARK(1);
 
     int L = p.seq_lens[seq];
@@ -662,21 +687,20 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         }
         return;
     }
-    const int32_t* bt = p.block_table + int64_t(seq) * p.max_blocks;
     const int last_page_idx = (L - 1) >> BSL;
     const int max_page = p.num_blocks - 1;
     const uint8_t* cache = p.cache;
     constexpr int64_t page_bytes = int64_t(BS) * ROWB;
 
     // ---- page ids of the split in registers (see the direct kernel) ---------------------
-    int pv[PVR];
-    const int split_p0 = begin >> BSL;
+    const int split_p0 = rowwide ? 0 : begin >> BSL;   // page index held by lane 0 of pv[0]
+    if (!rowwide) {
 #pragma unroll
-    for (int r = 0; r < PVR; ++r) {
-        int idx = split_p0 + 64 * r + lane;
-        idx = idx > last_page_idx ? last_page_idx : idx;
-        int pg = bt[idx];
-        pv[r] = pg < 0 ? 0 : (pg > max_page ? max_page : pg);
+        for (int r = 0; r < PVR; ++r) {
+            int idx = split_p0 + 64 * r + lane;
+            idx = idx > last_page_idx ? last_page_idx : idx;
+            pv[r] = bt[idx];
+        }
     }
     auto page_id = [&](int rel) -> int {
         int v = __builtin_amdgcn_readlane(pv[0], rel & 63);
@@ -688,7 +712,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         return v;
     };
     // the table is filled while the page ids are on their way
-    fill_pair_tables(lut, cent_k_mine, cent_v_mine, PROD ? 7 : 15, h, 8, lane);
+    fill_pair_tables<8>(lut, cent_k_mine, cent_v_mine, PROD ? 7 : 15, h, lane);
 
     // ---- copy plan: chunk c = tid + 512 k of the tile, k = 0..4 (the last round only
     // for the first 128 threads) -----------------------------------------------------------
@@ -700,10 +724,14 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     for (int k = 0; k < ROUNDS; ++k) {
         int c = tid + 512 * k;
         c = c < kChunksPerTile ? c : kChunksPerTile - 1;
-        const int row = c / kChunksPerRow, ci = c % kChunksPerRow;
-        src_page[k] = BS >= 32 ? 0 : row >> BSL;
-        src_off[k] = uint32_t((row & (BS - 1)) * ROWB + ci * 16);
-        dst_off[k] = staged_chunk_dst<PROD>(row, ci);
+        // rows of a page are contiguous: chunk c of the tile is chunk c - page * (chunks per page) of its page
+        constexpr int PC = BS * kChunksPerRow;
+        int pg = 0;
+#pragma unroll
+        for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
+        src_page[k] = pg;
+        src_off[k] = uint32_t(16 * (c - pg * PC));
+        dst_off[k] = kChunkDst<PROD>.off[c];
     }
     const bool has_round4 = tid < kChunksPerTile - 4 * 512;   // 128 threads, whole wavefronts
 
@@ -730,6 +758,8 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     };
 
     FQ_MARK(2);
+#pragma unroll
+    for (int r = 0; r < PVR; ++r) pv[r] = pv[r] < 0 ? 0 : (pv[r] > max_page ? max_page : pv[r]);
     // the loads of the first tile fly while the query is prepared
     issue_loads(begin);
     FQ_MARK(3);
@@ -748,52 +778,57 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         float mx = 0.0f;
         const bool live = hd < p.G;
         if (p.rotation != nullptr) {
-            float* qs = reinterpret_cast<float*>(slots);   // (H_Q, D) float32, H_Q <= 128 (64 with a sketch)
-            float* qs2 = qs + 64 * D;                      // PROD: (H_Q, D) float32 sketched query
+            // The rotated heads are exchanged through the second tile slot as 16-bit words of the
+            // query dtype (32 KB for 128 heads): the first tile goes to the first slot, and the
+            // second slot is not written before the barrier of the first loop iteration, which
+            // every wavefront reaches after it has read its heads back.  With a sketch the
+            // float32 sketched query (H_Q <= 64) takes the first slot and a barrier of its own.
+            uint16_t* qs = reinterpret_cast<uint16_t*>(slots + kTileBytes);
+            float* qs2 = reinterpret_cast<float*>(slots);
+            // this wavefront's 16 matrix columns as two fp16 terms each
+            half8 rot_hi[KS], rot_lo[KS], sk_hi[KS], sk_lo[KS];
+            split_rotation_block<D>(rot_b, rot_hi, rot_lo);
+            if constexpr (PROD) split_rotation_block<D>(rot_s, sk_hi, sk_lo);
             for (int rb = 0; 16 * rb < p.H_Q; ++rb) {
                 const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
-                float a[KS][8];
+                uint4v raw[KS];
 #pragma unroll
-                for (int j = 0; j < KS; ++j) {
-                    const uint4v raw = rb < 2 ? q_pre[rb & 1][j]
-                                              : *reinterpret_cast<const uint4v*>(qseq + row * D + 32 * j + 8 * g);
-                    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        a[j][2 * i] = load_elem<DT>(uint16_t(w[i] & 0xffffu));
-                        a[j][2 * i + 1] = load_elem<DT>(uint16_t(w[i] >> 16));
-                    }
-                }
-#ifdef FQ_DBG_NO_ROT_MFMA
-                const float4v acc = {a[0][0] + rot_b[0][0], a[1][1] + rot_b[1][1], a[2][2], a[3][3]};
-#else
-                const float4v acc = rotate_block<D>(a, rot_b);
-#endif
+                for (int j = 0; j < KS; ++j)
+                    raw[j] = rb < 2 ? q_pre[rb & 1][j]
+                                    : *reinterpret_cast<const uint4v*>(qseq + row * D + 32 * j + 8 * g);
+                half8 a[KS];
+                float up;
+                rows_as_f16<D, DT>(raw, a, up);
+                const float4v acc = rotate_block_f16<D>(a, rot_hi, rot_lo);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int head = 16 * rb + 4 * g + i;
-                    if (head < p.H_Q) qs[head * D + 16 * h + n] = load_elem<DT>(store_elem<DT>(acc[i]));
+                    if (head < p.H_Q) qs[head * D + 16 * h + n] = store_elem<DT>(acc[i] * up);
                 }
                 if constexpr (PROD) {
-                    const float4v acc2 = rotate_block<D>(a, rot_s);
+                    const float4v acc2 = rotate_block_f16<D>(a, sk_hi, sk_lo);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int head = 16 * rb + 4 * g + i;
-                        if (head < p.H_Q) qs2[head * D + 16 * h + n] = acc2[i];
+                        if (head < p.H_Q) qs2[head * D + 16 * h + n] = acc2[i] * up;
                     }
                 }
             }
             FQ_MARK(4);
             __syncthreads();
             FQ_MARK(5);
-            const float* src = qs + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
+            const uint16_t* src = qs + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
+            for (int ks = 0; ks < KS; ++ks) {
+                const uint4v raw = *reinterpret_cast<const uint4v*>(src + 8 * ks);
+                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    qf[ks][e] = live ? src[8 * ks + e] : 0.0f;
-                    mx = __builtin_fmaxf(mx, __builtin_fabsf(qf[ks][e]));
+                for (int i = 0; i < 4; ++i) {
+                    qf[ks][2 * i] = live ? load_elem<DT>(uint16_t(w[i] & 0xffffu)) : 0.0f;
+                    qf[ks][2 * i + 1] = live ? load_elem<DT>(uint16_t(w[i] >> 16)) : 0.0f;
+                    mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(qf[ks][2 * i]), __builtin_fabsf(qf[ks][2 * i + 1])));
                 }
+            }
             if constexpr (PROD) {
                 // <S q, signs> * sqrt(pi/2) / D: the constant rides on the query side
                 const float* src2 = qs2 + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
@@ -806,8 +841,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                         qf2[ks][e] = live ? src2[8 * ks + sign_order(e)] * (1.2533141373155003f / float(D)) : 0.0f;
                         mx2 = __builtin_fmaxf(mx2, __builtin_fabsf(qf2[ks][e]));
                     }
-                mx2 = __builtin_fmaxf(mx2, xor_shuffle(mx2, 16));
-                mx2 = __builtin_fmaxf(mx2, xor_shuffle(mx2, 32));
+                mx2 = max_xor32(max_xor16(mx2));
                 int ex2 = int((float_to_bits(mx2) >> 23) & 0xffu) - 127;
                 if (ex2 < -100 || ex2 > 100) ex2 = 0;
                 const float down2 = bits_to_float(uint32_t(127 - ex2) << 23);
@@ -818,7 +852,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                     for (int e = 0; e < 8; ++e) qsh[ks][e] = _Float16(qf2[ks][e] * down2);
             }
             FQ_MARK(6);
-            __syncthreads();   // the slots are about to receive tiles
+            if constexpr (PROD) __syncthreads();   // the first slot is about to receive a tile
         } else {
             const uint16_t* qsrc = qseq + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
@@ -833,8 +867,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                 }
             }
         }
-        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 16));
-        mx = __builtin_fmaxf(mx, xor_shuffle(mx, 32));
+        mx = max_xor32(max_xor16(mx));
         int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
         if (ex < -100 || ex > 100) ex = 0;
         const float down = bits_to_float(uint32_t(127 - ex) << 23);
@@ -1082,9 +1115,9 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     }
 #ifdef FQ_DBG_TIMING
     FQ_MARK(9);
-    if (threadIdx.x == 0 && blockIdx.x == 3 && blockIdx.y == 5)
-        printf("marks(100MHz ticks): start->lut %llu ->split %llu ->issue0 %llu ->rot %llu ->bar %llu ->qf %llu ->loop %llu ->tiles %llu ->end %llu\n",
-               tmark[1]-tmark[0], tmark[2]-tmark[1], tmark[3]-tmark[2], tmark[4]-tmark[3], tmark[5]-tmark[4], tmark[6]-tmark[5], tmark[7]-tmark[6], tmark[8]-tmark[7], tmark[9]-tmark[8]);
+    if ((threadIdx.x & 63) == 0 && (threadIdx.x == 0 || threadIdx.x == 256 || threadIdx.x == 448) && blockIdx.x == 3 && blockIdx.y == 5)
+        printf("w%d t0 %llu marks(100MHz ticks): start->lut %llu ->split %llu ->issue0 %llu ->rot %llu ->bar %llu ->qf %llu ->loop %llu ->tiles %llu ->end %llu\n",
+               int(threadIdx.x >> 6), tmark[0] % 100000ull, tmark[1]-tmark[0], tmark[2]-tmark[1], tmark[3]-tmark[2], tmark[4]-tmark[3], tmark[5]-tmark[4], tmark[6]-tmark[5], tmark[7]-tmark[6], tmark[8]-tmark[7], tmark[9]-tmark[8]);
 #endif
 }
 
@@ -1275,7 +1308,9 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
     const int64_t chunk = (((max_ctx + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
     const bool wide = chunk / BS > 64;   // begin is a multiple of 64 tokens, hence page aligned
 
-    if (staged_applies(D, p.H_KV)) return launch_staged_any<DT, false>(p, S, BS, wide, stream);
+    // four page-id registers also when they can hold the whole block-table row
+    if (staged_applies(D, p.H_KV))
+        return launch_staged_any<DT, false>(p, S, BS, wide || (p.max_blocks > 64 && p.max_blocks <= 256), stream);
 
     const int waves = p.H_KV < 8 ? p.H_KV : 8;
     const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
@@ -1574,7 +1609,7 @@ extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, cons
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t max_ctx = int64_t(max_blocks_per_seq) * block_size;
     const int64_t chunk = (((max_ctx + num_splits - 1) / num_splits) + 63) & ~int64_t(63);
-    const bool wide = chunk / block_size > 64;
+    const bool wide = chunk / block_size > 64 || (max_blocks_per_seq > 64 && max_blocks_per_seq <= 256);
     const int st = dtype == FQ_F16 ? launch_staged_any<FQ_F16, true>(p, num_seqs, block_size, wide, s)
                                    : launch_staged_any<FQ_BF16, true>(p, num_seqs, block_size, wide, s);
     if (st != FQ_OK) return st;
