@@ -1164,23 +1164,35 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
                                                             const float* __restrict__ part_l,
                                                             const float* __restrict__ R, uint16_t* __restrict__ out,
                                                             int64_t rows, int NS, int col_major) {
-    __shared__ float os[kRotRows][D + 4];
+    constexpr int CBW = D / 64;            // 16-column blocks per wavefront
+    constexpr int OSTRIDE = D + 8;         // 16-bit words per staged row (padded: conflict-free operand reads)
+    __shared__ __attribute__((aligned(16))) uint16_t os[kRotRows * OSTRIDE];   // combined rows, query dtype
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int64_t row0 = int64_t(blockIdx.x) * kRotRows;
-    // ---- combine: thread t handles 8 consecutive coordinates of row t / 16; splits are taken
-    // eight at a time so that their loads are all in flight together ------------------------------
+
+    // the matrix columns of this wavefront are asked for first: they arrive during the combine
+    float rbv[CBW][D / 32][8];
+    if (R != nullptr) {
+#pragma unroll
+        for (int i = 0; i < CBW; ++i) load_rotation_any<D>(R, col_major != 0, false, 16 * (wave + 4 * i), n, g, rbv[i]);
+    }
+
+    // ---- combine: thread t handles 8 consecutive coordinates of row t / 16; the loads of up to
+    // eight splits (maximum, denominator, accumulator) are all in flight together -------------------
     {
         const int r = threadIdx.x >> 4;
         const int64_t row = row0 + r < rows ? row0 + r : rows - 1;
         const int64_t base = row * NS;
         float mstar = -__builtin_inff();
-        for (int s0 = 0; s0 < NS; s0 += 8) {
-            float mv[8];
+        if (NS > 8) {
+            for (int s0 = 0; s0 < NS; s0 += 8) {
+                float mv[8];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) mv[k] = part_m[base + (s0 + k < NS ? s0 + k : NS - 1)];
+                for (int k = 0; k < 8; ++k) mv[k] = part_m[base + (s0 + k < NS ? s0 + k : NS - 1)];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) mstar = __builtin_fmaxf(mstar, mv[k]);
+                for (int k = 0; k < 8; ++k) mstar = __builtin_fmaxf(mstar, mv[k]);
+            }
         }
         for (int c0 = 8 * (threadIdx.x & 15); c0 < D; c0 += 128) {
             float num[8];
@@ -1195,49 +1207,64 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
                     const int sidx = s0 + k < NS ? s0 + k : NS - 1;
                     mv[k] = part_m[base + sidx];
                     lv[k] = part_l[base + sidx];
-                    // an empty split (m = -inf) never wrote its accumulator: do not read it
-                    const bool use = s0 + k < NS && mv[k] != -__builtin_inff();
+                    // an empty split (m = -inf) never wrote its accumulator: whatever is read there gets weight 0
                     const float4v* src = reinterpret_cast<const float4v*>(part_acc + (base + sidx) * D + c0);
-                    lo[k] = use ? src[0] : float4v{0.f, 0.f, 0.f, 0.f};
-                    hi[k] = use ? src[1] : float4v{0.f, 0.f, 0.f, 0.f};
-                    mv[k] = use ? mv[k] : -__builtin_inff();
+                    lo[k] = src[0];
+                    hi[k] = src[1];
+                }
+                if (NS <= 8) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) mstar = __builtin_fmaxf(mstar, mv[k]);
                 }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    const float w = mv[k] == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(mv[k] - mstar);
+                    const bool use = s0 + k < NS && mv[k] != -__builtin_inff();
+                    const float w = use ? __builtin_amdgcn_exp2f(mv[k] - mstar) : 0.0f;
                     den = __builtin_fmaf(lv[k], w, den);
-                    num[0] = __builtin_fmaf(lo[k].x, w, num[0]); num[1] = __builtin_fmaf(lo[k].y, w, num[1]);
-                    num[2] = __builtin_fmaf(lo[k].z, w, num[2]); num[3] = __builtin_fmaf(lo[k].w, w, num[3]);
-                    num[4] = __builtin_fmaf(hi[k].x, w, num[4]); num[5] = __builtin_fmaf(hi[k].y, w, num[5]);
-                    num[6] = __builtin_fmaf(hi[k].z, w, num[6]); num[7] = __builtin_fmaf(hi[k].w, w, num[7]);
+                    // a weight of 0 must also silence a NaN or Inf in memory that no split wrote
+                    num[0] = use ? __builtin_fmaf(lo[k].x, w, num[0]) : num[0]; num[1] = use ? __builtin_fmaf(lo[k].y, w, num[1]) : num[1];
+                    num[2] = use ? __builtin_fmaf(lo[k].z, w, num[2]) : num[2]; num[3] = use ? __builtin_fmaf(lo[k].w, w, num[3]) : num[3];
+                    num[4] = use ? __builtin_fmaf(hi[k].x, w, num[4]) : num[4]; num[5] = use ? __builtin_fmaf(hi[k].y, w, num[5]) : num[5];
+                    num[6] = use ? __builtin_fmaf(hi[k].z, w, num[6]) : num[6]; num[7] = use ? __builtin_fmaf(hi[k].w, w, num[7]) : num[7];
                 }
             }
             const bool live = row0 + r < rows && den > 0.0f;
+            uint32_t wds[4];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) os[r][c0 + e] = live ? load_elem<DT>(store_elem<DT>(num[e] / den)) : 0.0f;
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t a0 = live ? store_elem<DT>(num[2 * e] / den) : 0u;
+                const uint32_t a1 = live ? store_elem<DT>(num[2 * e + 1] / den) : 0u;
+                wds[e] = a0 | (a1 << 16);
+            }
+            *reinterpret_cast<uint4v*>(&os[r * OSTRIDE + c0]) = uint4v{wds[0], wds[1], wds[2], wds[3]};
         }
     }
     __syncthreads();
     if (R == nullptr) {
-        for (int i = threadIdx.x; i < kRotRows * D; i += 256) {
-            const int64_t row = row0 + i / D;
-            if (row < rows) out[row * D + i % D] = store_elem<DT>(os[i / D][i % D]);
+        for (int c = threadIdx.x; c < kRotRows * (D / 8); c += 256) {
+            const int r = c / (D / 8), q = c % (D / 8);
+            const int64_t row = row0 + r;
+            if (row < rows) reinterpret_cast<uint4v*>(out + row * D)[q] = *reinterpret_cast<const uint4v*>(&os[r * OSTRIDE + 8 * q]);
         }
         return;
     }
-    float a[D / 32][8];
+    // ---- rotate back on the fp16 MFMA: the rows are exact in fp16 up to a power of two ----------------
+    uint4v raw[D / 32];
 #pragma unroll
-    for (int j = 0; j < D / 32; ++j)
+    for (int j = 0; j < D / 32; ++j) raw[j] = *reinterpret_cast<const uint4v*>(&os[n * OSTRIDE + 32 * j + 8 * g]);
+    half8 a[D / 32];
+    float up;
+    rows_as_f16<D, DT>(raw, a, up);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) a[j][e] = os[n][32 * j + 8 * g + e];
-    for (int cb = wave; cb < D / 16; cb += 4) {
-        float b[D / 32][8];
-        load_rotation_any<D>(R, col_major != 0, false, 16 * cb, n, g, b);
-        const float4v acc = rotate_block<D>(a, b);
+    for (int i = 0; i < CBW; ++i) {
+        half8 rhi[D / 32], rlo[D / 32];
+        split_rotation_block<D>(rbv[i], rhi, rlo);
+        const float4v acc = rotate_block_f16<D>(a, rhi, rlo);
+        const int cb = wave + 4 * i;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int64_t row = row0 + 4 * g + i;
-            if (row < rows) out[row * D + 16 * cb + n] = store_elem<DT>(acc[i]);
+        for (int k = 0; k < 4; ++k) {
+            const int64_t row = row0 + 4 * g + k;
+            if (row < rows) out[row * D + 16 * cb + n] = store_elem<DT>(acc[k] * up);
         }
     }
 }
