@@ -46,6 +46,7 @@
 #include <cstdlib>
 #include <map>
 #include <mutex>
+#include <type_traits>
 #include <utility>
 
 #include "fq_common.hpp"
@@ -744,9 +745,13 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         const uint32_t in_page = BS >= 32 ? uint32_t((t0 & (BS - 1)) * ROWB) : 0u;
 #pragma unroll
         for (int k = 0; k < ROUNDS; ++k) {
+            // where a page is a whole number of wavefront rounds (16 rows of 68 chunks = 17 x 64), a
+            // wavefront's 64 chunks lie in one page and the page base stays in scalar registers
+            constexpr bool kUniformPage = (BS * kChunksPerRow) % 64 == 0;
+            const int pg_k = kUniformPage ? __builtin_amdgcn_readfirstlane(src_page[k]) : src_page[k];
             const uint8_t* b = base[0];
 #pragma unroll
-            for (int i = 1; i < PPT; ++i) b = src_page[k] == i ? base[i] : b;
+            for (int i = 1; i < PPT; ++i) b = pg_k == i ? base[i] : b;
             if (k < 4 || has_round4) stage_reg[k] = *reinterpret_cast<const uint4v*>(b + in_page + src_off[k]);
         }
     };
@@ -901,6 +906,17 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         n_rd[e] = blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
     }
 
+    // dword d of the P operand holds slots 2d, 2d + 1: it is this lane's when its class owns them
+    uint32_t pa_mask[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        bool mine;
+        if (GP == 4) mine = d == cls;                 // class = 2 * block + half, one dword each
+        else if (GP == 8) mine = (d >> 1) == cls;     // class = block, two dwords each
+        else mine = true;
+        pa_mask[d] = mine ? 0xffffffffu : 0u;
+    }
+
     // ---- running state ---------------------------------------------------------------------
     float4v O[DPL];
 #pragma unroll
@@ -908,7 +924,8 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     float M = -__builtin_inff();
     float lsum = 0.0f;
 
-    auto compute_tile = [&](int t0, int slot) {
+    auto compute_tile = [&](int t0, int slot, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;   // the tile may reach past the end of the split
         const uint8_t* tile = slots + slot * kTileBytes;
         // operands of this lane, raw
         uint4v kraw[2];
@@ -997,7 +1014,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                 s = acc[e >> 2][e & 3];
                 if (PROD) s2 = acc_s[e >> 2][e & 3];
             }
-            const bool live = t0 + sc_tok[e] < end;
+            const bool live = !MASKED || t0 + sc_tok[e] < end;
             rv[e] = live ? vn[e] : 0.0f;
             float sc = s * kn[e] * qscale;
             if (PROD) sc = __builtin_fmaf(s2 * kg[e], qscale_s, sc);
@@ -1005,17 +1022,20 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             tmax = __builtin_fmaxf(tmax, a_[e]);
         }
         tmax = max_same_head<GP>(tmax);
-        const float Mnew = __builtin_fmaxf(M, tmax);
+        // The running maximum moves only when it would grow by more than 2^4: weights then stay
+        // below 16 (fine in fp16 next to value norms up to 4000), and the rescale of the
+        // accumulators, 32 multiplies, becomes rare.
+        const float Mnew = tmax > M + 4.0f ? tmax : M;
         const float Ms = Mnew == -__builtin_inff() ? 0.0f : Mnew;
         const float alpha = __builtin_amdgcn_exp2f(M - Ms);
         M = Mnew;
-        _Float16 wh[NSC];
+        float wv[NSC];
         float psum = 0.0f;
 #pragma unroll
         for (int e = 0; e < NSC; ++e) {
             const float w = __builtin_amdgcn_exp2f(a_[e] - Ms);
             psum += w;
-            wh[e] = _Float16(__builtin_fminf(w * rv[e], kHalfMax));
+            wv[e] = __builtin_fminf(w * rv[e], kHalfMax);
         }
         lsum = __builtin_fmaf(lsum, alpha, psum);
 
@@ -1037,14 +1057,20 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         }
 
         // ---- weights as the A operand: slot j <-> (block j / 4, row 4g + j % 4) -------------------
-        half8 pa;
+        // (the weights of this lane are packed once and placed with lane-constant masks)
+        uint32_t pk[NSC / 2];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            constexpr _Float16 zero = _Float16(0.0f);
-            if (GP == 4) pa[j] = ((j >> 2) == (cls >> 1) && ((j >> 1) & 1) == (cls & 1)) ? wh[j & 1] : zero;
-            else if (GP == 8) pa[j] = ((j >> 2) == cls) ? wh[(j & 3) % NSC] : zero;
-            else pa[j] = wh[j % NSC];
+        for (int e = 0; e < NSC / 2; ++e) {
+            const half2v h2 = {_Float16(wv[2 * e]), _Float16(wv[2 * e + 1])};
+            pk[e] = __builtin_bit_cast(uint32_t, h2);
         }
+        uint4v pa_w;
+        if (GP == 16) {
+            pa_w = uint4v{pk[0], pk[1 % (NSC / 2)], pk[2 % (NSC / 2)], pk[3 % (NSC / 2)]};
+        } else {
+            pa_w = uint4v{pk[0] & pa_mask[0], pk[1 % (NSC / 2)] & pa_mask[1], pk[0] & pa_mask[2], pk[1 % (NSC / 2)] & pa_mask[3]};
+        }
+        const half8 pa = __builtin_bit_cast(half8, pa_w);
 
         // ---- O += P . V ------------------------------------------------------------------------------
         __builtin_amdgcn_sched_barrier(0);
@@ -1076,7 +1102,8 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             issue_loads(clamp_t0(t0 + 64));       // tile i + 2
 #endif
 #if FQ_STAGED_DEBUG_MODE != 1
-            compute_tile(t0, i & 1);
+            if (t0 + 32 <= end) compute_tile(t0, i & 1, std::false_type{});
+            else compute_tile(t0, i & 1, std::true_type{});
 #endif
         }
     }
