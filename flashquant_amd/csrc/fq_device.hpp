@@ -239,4 +239,45 @@ __device__ __forceinline__ void rows_as_f16(const uint4v (&raw)[D / 32], half8 (
         for (int e = 0; e < 8; ++e) a[j][e] = _Float16(v[j][e] * down);
 }
 
+// float32 rows (lane (m, g) holding k = 32 j + 8 g + e) as two fp16 terms, v = (hi + lo / 4096) * up,
+// scaled by one power of two per 16-row block; with a split matrix block the product is
+// hi.hi + (hi.lo + lo.hi) / 4096, accurate to about 2^-22 of the block's largest element.
+template <int D>
+__device__ __forceinline__ void rows_split_f16(const float (&v)[D / 32][8], half8 (&hi)[D / 32], half8 (&lo)[D / 32],
+                                               float& up) {
+    float mx = 0.0f;
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mx = __builtin_fmaxf(mx, __builtin_fabsf(v[j][e]));
+    mx = wave_max(mx);
+    int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+    if (ex < -100 || ex > 100) ex = 0;
+    const float down = bits_to_float(uint32_t(127 - ex) << 23);
+    up = bits_to_float(uint32_t(127 + ex) << 23);
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            const float a0 = v[j][e] * down, a1 = v[j][e + 1] * down;
+            const auto h2 = __builtin_amdgcn_cvt_pkrtz(a0, a1);
+            const auto l2 = __builtin_amdgcn_cvt_pkrtz((a0 - float(h2[0])) * 4096.0f, (a1 - float(h2[1])) * 4096.0f);
+            hi[j][e] = h2[0]; hi[j][e + 1] = h2[1];
+            lo[j][e] = l2[0]; lo[j][e + 1] = l2[1];
+        }
+}
+
+template <int D>
+__device__ __forceinline__ float4v rotate_block_f16x3(const half8 (&ahi)[D / 32], const half8 (&alo)[D / 32],
+                                                      const half8 (&bhi)[D / 32], const half8 (&blo)[D / 32]) {
+    float4v acc_hi = {0.f, 0.f, 0.f, 0.f}, acc_lo = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+        acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi[j], bhi[j], acc_hi, 0, 0, 0);
+        acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi[j], blo[j], acc_lo, 0, 0, 0);
+        acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo[j], bhi[j], acc_lo, 0, 0, 0);
+    }
+    return acc_hi + acc_lo * (1.0f / 4096.0f);
+}
+
 }  // namespace fq

@@ -30,8 +30,8 @@
 // 8 consecutive positions are exactly its 8 tokens.  The K tile uses the same
 // permutation on the coordinates, and the query operand is read to match.
 //
-// The two head rotations run on the float32 MFMA inside the kernel (prologue and
-// epilogue), staged through the tile buffers.
+// The two head rotations run inside the kernel (prologue and epilogue) on the fp16 MFMA
+// with operands split into two fp16 terms, staged through the tile buffers.
 #include "fq_common.hpp"
 #include "fq_device.hpp"
 
@@ -177,30 +177,28 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     {
         const uint16_t* qbase = p.q + ((int64_t(b) * p.H_Q + hq) * p.N_Q) * D;
         uint16_t* st = reinterpret_cast<uint16_t*>(bufs + w * kPfStageBytes);   // (32 rows, 128) raw 16-bit
-        float a[2][4][8];
+        // the rows are exact in fp16 up to a power of two: fp16-split MFMA, two terms
+        half8 a[2][4];
+        float up[2];
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             int pos = pos0 + 16 * rb + n16;
             pos = pos < p.N_Q ? pos : p.N_Q - 1;
+            uint4v raw[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint4v raw = *reinterpret_cast<const uint4v*>(qbase + int64_t(pos) * D + 32 * j + 8 * g4);
-                const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    a[rb][j][2 * i] = load_elem<DT>(uint16_t(wds[i] & 0xffffu));
-                    a[rb][j][2 * i + 1] = load_elem<DT>(uint16_t(wds[i] >> 16));
-                }
-            }
+            for (int j = 0; j < 4; ++j) raw[j] = *reinterpret_cast<const uint4v*>(qbase + int64_t(pos) * D + 32 * j + 8 * g4);
+            rows_as_f16<D, DT>(raw, a[rb], up[rb]);
         }
         for (int cb = 0; cb < 8; ++cb) {
             float rbv[4][8];
             load_rotation_any<D>(p.rotation, p.rot_col_major != 0, true, 16 * cb, n16, g4, rbv);
+            half8 rhi[4], rlo[4];
+            split_rotation_block<D>(rbv, rhi, rlo);
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb) {
-                const float4v acc = rotate_block<D>(a[rb], rbv);
+                const float4v acc = rotate_block_f16<D>(a[rb], rhi, rlo);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) st[(16 * rb + 4 * g4 + i) * D + 16 * cb + n16] = store_elem<DT>(acc[i]);
+                for (int i = 0; i < 4; ++i) st[(16 * rb + 4 * g4 + i) * D + 16 * cb + n16] = store_elem<DT>(acc[i] * up[rb]);
             }
         }
         __syncthreads();
@@ -352,14 +350,20 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             a[j][0] = lo.x; a[j][1] = lo.y; a[j][2] = lo.z; a[j][3] = lo.w;
             a[j][4] = hi.x; a[j][5] = hi.y; a[j][6] = hi.z; a[j][7] = hi.w;
         }
+        // float32 rows: both operands as two fp16 terms, three MFMA terms
+        half8 ahi[4], alo[4];
+        float up;
+        rows_split_f16<D>(a, ahi, alo, up);
         for (int cb = 0; cb < 8; ++cb) {
             float rbv[4][8];
             load_rotation_any<D>(p.rotation, p.rot_col_major != 0, false, 16 * cb, n16, g4, rbv);
-            const float4v acc = rotate_block<D>(a, rbv);
+            half8 rhi[4], rlo[4];
+            split_rotation_block<D>(rbv, rhi, rlo);
+            const float4v acc = rotate_block_f16x3<D>(ahi, alo, rhi, rlo);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int pos = pos0 + 16 * half_rows + 4 * g4 + i;
-                if (unit_live && pos < p.N_Q) obase[int64_t(pos) * D + 16 * cb + n16] = store_elem<DT>(acc[i]);
+                if (unit_live && pos < p.N_Q) obase[int64_t(pos) * D + 16 * cb + n16] = store_elem<DT>(acc[i] * up);
             }
         }
     }
