@@ -131,7 +131,8 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     uint2v kraw;
     uint32_t vra, vrb;
     float nk, nv0, nv1;
-    auto issue_loads = [&](int tile) {
+    auto issue_loads = [&](int tile_raw) {
+        const int tile = tile_raw < ntiles ? tile_raw : ntiles - 1;   // past the end: the last tile again, never used
         const int t0 = tile * 64;
         const int last = p.N_KV - 1;
         const int tkk = t0 + tk < last ? t0 + tk : last;
@@ -280,7 +281,10 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
 #pragma unroll
             for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, S[tb][r]);
         mx = max_xor32(mx);
-        const float mnew = __builtin_fmaxf(m_run, mx * krow);
+        // the running maximum moves only when it would grow by more than 2^4: the weights stay
+        // below 16 and the rescale of the 64 accumulator registers becomes rare
+        const float cand = mx * krow;
+        const float mnew = cand > m_run + 4.0f ? cand : m_run;
         const float ms = mnew == -__builtin_inff() ? 0.0f : mnew;
         const float alpha = __builtin_amdgcn_exp2f(m_run - ms);
         m_run = mnew;
@@ -315,14 +319,21 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
 
     // ---- tiles ----------------------------------------------------------------------------------------
     dequant(0);
-    if (ntiles > 1) issue_loads(1);
-    for (int i = 0; i < ntiles; ++i) {
+    issue_loads(1);
+    // The dequantisation of tile i + 1 and the products of tile i sit in one basic block (no
+    // conditions between them), so that the lookups and LDS writes of the one interleave with
+    // the MFMAs of the other.
+    int i = 0;
+    for (; i < my_tiles; ++i) {
         __syncthreads();                       // tile i is complete; the other buffer is free
-        if (i + 1 < ntiles) {
-            dequant((i + 1) & 1);
-            if (i + 2 < ntiles) issue_loads(i + 2);
-        }
-        if (i < my_tiles) compute(i, i & 1);
+        dequant((i + 1) & 1);
+        issue_loads(i + 2);
+        compute(i, i & 1);
+    }
+    for (; i < ntiles; ++i) {                  // tiles only the other wavefronts of the workgroup need
+        __syncthreads();
+        dequant((i + 1) & 1);
+        issue_loads(i + 2);
     }
 
     // ---- normalise, rotate back, store -------------------------------------------------------------------
