@@ -48,6 +48,13 @@ struct CompressCfg {
 
 constexpr float kLoScale = 1.0f / 4096.0f;
 
+// lane exchange inside the VALU (DPP): CTRL 0xB1 / 0x4E swap lanes inside quads, 0x141 / 0x140
+// mirror the 8- / 16-lane rows
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+
 struct BucketTable {
     uint2v cell[256];   // x = threshold bits, y = base count
     float bnd[16];
@@ -217,10 +224,16 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                 ss = __builtin_fmaf(e[i], e[i], ss);
                 mx = __builtin_fmaxf(mx, __builtin_fabsf(e[i]));
             }
-#pragma unroll
-            for (int m = 1; m < C::CPR; m <<= 1) {
-                ss += xor_shuffle(ss, m);
-                mx = __builtin_fmaxf(mx, xor_shuffle(mx, m));
+            // all-reduce over the CPR lanes of the row, in the VALU (quad swaps, mirrors, row swap)
+            ss += dpp_f32<0xB1>(ss); mx = __builtin_fmaxf(mx, dpp_f32<0xB1>(mx));      // lane ^ 1
+            ss += dpp_f32<0x4E>(ss); mx = __builtin_fmaxf(mx, dpp_f32<0x4E>(mx));      // lane ^ 2
+            ss += dpp_f32<0x141>(ss); mx = __builtin_fmaxf(mx, dpp_f32<0x141>(mx));    // mirror of 8: the other quad
+            if (C::CPR >= 16) { ss += dpp_f32<0x140>(ss); mx = __builtin_fmaxf(mx, dpp_f32<0x140>(mx)); }   // mirror of 16
+            if (C::CPR >= 32) {
+                const auto sw = __builtin_amdgcn_permlane16_swap(float_to_bits(ss), float_to_bits(ss), false, false);
+                ss = bits_to_float(sw[0]) + bits_to_float(sw[1]);
+                const auto mw = __builtin_amdgcn_permlane16_swap(float_to_bits(mx), float_to_bits(mx), false, false);
+                mx = __builtin_fmaxf(bits_to_float(mw[0]), bits_to_float(mw[1]));
             }
             const float nrm = __builtin_sqrtf(ss);
             int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;

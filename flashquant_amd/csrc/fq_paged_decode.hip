@@ -5,43 +5,46 @@
 // src/flashquant/kernels/paged_decode.py:112-128.  Token row of the cache:
 // [K idx H*D/2 | K norm H*4 | V idx H*D/2 | V norm H*4] (src/flashquant/vllm/impl.py:132-138).
 //
-// Three launches on the caller's stream:
-//   1. rotate_q_kernel       q_rot = (q @ R^T) rounded to the query dtype
-//   2. paged_decode_kernel   one workgroup per (split, sequence, group of <= 8 KV
-//                            heads), one wavefront per KV head; writes float32
-//                            partials (m, l, acc[D]) per (sequence, query head, split)
-//   3. reduce_rotate_kernel  log-sum-exp combine of the splits, rounded to the
-//                            query dtype, then (out_rot @ R) rounded again
+// Launches on the caller's stream:
+//   rotate_q_kernel              q_rot = (q @ R^T) rounded to the query dtype; only for
+//                                shapes whose decode kernel does not rotate the query itself
+//   paged_decode_staged_kernel   8 KV heads of 128 coordinates: one workgroup of 8 wavefronts
+//                                per (split, sequence) copies whole token rows to LDS and
+//                                wavefront h works on KV head h; rotates the query in its
+//                                prologue; also serves TurboQuantProd pages
+//   paged_decode_kernel          every other shape: one wavefront per (split, sequence, KV
+//                                head), operands read straight from global memory
+//   reduce_rotate_kernel         log-sum-exp combine of the split partials (m, l, acc[D]),
+//                                rounded to the query dtype, then (out_rot @ R) rounded again
 //
-// The decode kernel is bound by HBM traffic (136 bytes per token per KV head)
-// but only if the per-byte work is small: with 4 query heads per KV head,
-// float32 FMAs alone would cost more than the memory time, so both products
-// run on the 16x16x32 fp16 MFMA and the dequantisation is one LDS lookup per
-// packed byte: a 256-entry table maps a byte to the fp16 pair
-// (centroid[hi nibble], centroid[lo nibble]), replicated 32 times so that lane
-// l always reads bank l % 32 (no bank conflicts whatever the data).
+// The decode kernels are bound by HBM traffic (136 bytes per token per KV head) only
+// if the per-byte work is small: with 4 query heads per KV head, float32 FMAs alone
+// would cost more than the memory time, so both products run on the 16x16x32 fp16
+// MFMA and the dequantisation is one LDS lookup per packed byte: a 256-entry table maps
+// a byte to the fp16 pair (centroid[hi nibble], centroid[lo nibble]), replicated so
+// that the lanes of a half-wave always read different banks whatever the data.
 //
-// Tile = 64 tokens = 4 blocks of 16.
+// Per 16-token block:
 //   scores   S^T_blk = K_blk (16 tokens x D) . Q^T (D x 16 columns).  Column n
 //            carries query head n % GP (GP = group size padded to 4, 8 or 16), so
 //            every block's result holds each head 16/GP times; lane (n, g) keeps
 //            the copy of block class n / GP.  After that selection a lane owns
-//            4 consecutive tokens of one head per kept block, all lanes busy.
+//            consecutive tokens of one head per kept block, all lanes busy.
 //            A lane's K operand is the 16 bytes it loaded (token n, quarter g of
 //            the row): the contraction index is permuted (k-step ks, group g,
 //            element e) <-> d = g*D/4 + 8*ks + e, and Q is loaded the same way.
-//   softmax  the V norm is folded into the exponent: w = 2^(s + log2|v| - M) lies
-//            in (0, 1] and is safe in fp16 whatever the scale of V; the
-//            denominator accumulates w / |v|.
-//   output   O (16 rows x D) += P (16 x 64 tokens) . V (64 tokens x D), where row
-//            n of P holds the weights of head n % GP for the tokens of block class
-//            n / GP only (zero elsewhere), so the lane that computed a weight is
-//            the lane that feeds it to the MFMA: no cross-lane movement.  The
-//            classes are summed once per split.  V's contraction index is the
-//            token, so a lane loads, for its 16 tokens of the tile, the bytes of
-//            D/16 consecutive coordinates (lane n <-> d = n*D/16 ...), and a
-//            2x2 nibble transpose of token pairs makes each byte hold the same
-//            coordinate of two consecutive tokens: again one lookup per byte.
+//   softmax  base 2, float32; the weight handed to the second product is
+//            min(w * |v|, 65504) in fp16 (the V norm rides on the weight), the
+//            denominator accumulates w.
+//   output   O (16 rows x D) += P (16 x tokens) . V (tokens x D), where row n of P
+//            holds the weights of head n % GP for the tokens of block class n / GP
+//            only (zero elsewhere), so the lane that computed a weight is the lane
+//            that feeds it to the MFMA: no cross-lane movement.  The classes are
+//            summed once per split.  V's contraction index is the token, so a lane
+//            loads the bytes of D/16 consecutive coordinates (lane n <-> d = n*D/16
+//            ...) of its tokens, and a 2x2 nibble transpose of token pairs makes
+//            each byte hold the same coordinate of two consecutive tokens: again
+//            one lookup per byte.
 
 #include <cstdlib>
 #include <map>
@@ -51,16 +54,6 @@
 
 #include "fq_common.hpp"
 #include "fq_device.hpp"
-
-#ifndef FQ_STAGED_DEBUG_MODE
-#define FQ_STAGED_DEBUG_MODE 0   // 1: copy only, 2: compute only (timing experiments; never shipped)
-#endif
-
-#ifdef FQ_DBG_TIMING
-#define FQ_MARK(i) do { if ((threadIdx.x & 63) == 0 && blockIdx.x == 3 && blockIdx.y == 5) tmark[i] = wall_clock64(); } while (0)
-#else
-#define FQ_MARK(i)
-#endif
 
 namespace fq_host {
 // FQ_DECODE_DIRECT=1 in the environment routes every shape to the direct kernel
@@ -618,10 +611,6 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     __shared__ __attribute__((aligned(256))) uint32_t lut[kLutWords];
     extern __shared__ __attribute__((aligned(16))) uint8_t slots[];   // two tile slots
 
-#ifdef FQ_DBG_TIMING
-    unsigned long long tmark[12] = {};
-#endif
-    FQ_MARK(0);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int h = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront = KV head
@@ -670,7 +659,6 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             pv[r] = bt[idx];
         }
     }
-    FQ_MARK(1);
 
     int L = p.seq_lens[seq];
     L = L < 0 ? 0 : L;
@@ -762,12 +750,10 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             if (k < 4 || has_round4) *reinterpret_cast<uint4v*>(dst + dst_off[k]) = stage_reg[k];
     };
 
-    FQ_MARK(2);
 #pragma unroll
     for (int r = 0; r < PVR; ++r) pv[r] = pv[r] < 0 ? 0 : (pv[r] > max_page ? max_page : pv[r]);
     // the loads of the first tile fly while the query is prepared
     issue_loads(begin);
-    FQ_MARK(3);
 
     // ---- query operand ------------------------------------------------------------------
     // With a rotation matrix the workgroup first rotates all query heads of its sequence:
@@ -819,9 +805,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                     }
                 }
             }
-            FQ_MARK(4);
             __syncthreads();
-            FQ_MARK(5);
             const uint16_t* src = qs + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -856,7 +840,6 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
 #pragma unroll
                     for (int e = 0; e < 8; ++e) qsh[ks][e] = _Float16(qf2[ks][e] * down2);
             }
-            FQ_MARK(6);
             if constexpr (PROD) __syncthreads();   // the first slot is about to receive a tile
         } else {
             const uint16_t* qsrc = qseq + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
@@ -1089,26 +1072,18 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     {
         const int last_t0 = begin + ((end - begin - 1) & ~31);
         auto clamp_t0 = [&](int t) { return t < last_t0 ? t : last_t0; };
-        FQ_MARK(7);
         write_slot(0);                            // tile 0, loaded before the query was prepared
         issue_loads(clamp_t0(begin + 32));
         int i = 0;
-        for (int t0 = begin; t0 < (FQ_STAGED_DEBUG_MODE == 3 ? begin : end); t0 += 32, ++i) {
-#ifndef FQ_STAGED_NO_BARRIER
+        for (int t0 = begin; t0 < end; t0 += 32, ++i) {
             __syncthreads();                      // tile i is in LDS; slot of tile i - 1 is free
-#endif
-#if FQ_STAGED_DEBUG_MODE != 2
             write_slot((i + 1) & 1);              // tile i + 1 (its loads ran during tile i - 1)
             issue_loads(clamp_t0(t0 + 64));       // tile i + 2
-#endif
-#if FQ_STAGED_DEBUG_MODE != 1
             if (t0 + 32 <= end) compute_tile(t0, i & 1, std::false_type{});
             else compute_tile(t0, i & 1, std::true_type{});
-#endif
         }
     }
 
-    FQ_MARK(8);
     // ---- publish the partial of this split (as in the direct kernel) -----------------------------
 #pragma unroll
     for (int mask = GP; mask < 64; mask <<= 1) lsum += xor_shuffle(lsum, mask);
@@ -1140,12 +1115,6 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             }
         }
     }
-#ifdef FQ_DBG_TIMING
-    FQ_MARK(9);
-    if ((threadIdx.x & 63) == 0 && (threadIdx.x == 0 || threadIdx.x == 256 || threadIdx.x == 448) && blockIdx.x == 3 && blockIdx.y == 5)
-        printf("w%d t0 %llu marks(100MHz ticks): start->lut %llu ->split %llu ->issue0 %llu ->rot %llu ->bar %llu ->qf %llu ->loop %llu ->tiles %llu ->end %llu\n",
-               int(threadIdx.x >> 6), tmark[0] % 100000ull, tmark[1]-tmark[0], tmark[2]-tmark[1], tmark[3]-tmark[2], tmark[4]-tmark[3], tmark[5]-tmark[4], tmark[6]-tmark[5], tmark[7]-tmark[6], tmark[8]-tmark[7], tmark[9]-tmark[8]);
-#endif
 }
 
 // q_rot[row, j] = sum_k q[row, k] * R[j, k], rounded to the query dtype
