@@ -25,7 +25,7 @@ __device__ __forceinline__ float rounded_product(float a, float b) {
 namespace fq {
 
 constexpr int kDecThreads = 256;
-constexpr int kDecUnroll = 4;
+constexpr int kDecUnroll = 8;   // packed dwords per lane: eight loads and eight 16-byte stores in flight
 
 template <int DT>
 __device__ __forceinline__ void store_unit(void* out, int64_t unit, const float (&v)[8]) {
