@@ -49,7 +49,6 @@
 #include <cstdlib>
 #include <map>
 #include <mutex>
-#include <type_traits>
 #include <utility>
 
 #include "fq_common.hpp"
@@ -124,7 +123,10 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
     L = L < 0 ? 0 : L;
     L = L > p.max_blocks * BS ? p.max_blocks * BS : L;
     const int NS = p.num_splits;
-    const int chunk = (((L + NS - 1) / NS) + 63) & ~63;
+    // every sequence is cut into the same token chunks (those of the longest possible context):
+    // the work of a workgroup does not depend on its sequence's length, short sequences just
+    // leave their last splits empty
+    const int chunk = (((p.max_blocks * BS + NS - 1) / NS) + 63) & ~63;
     const int begin = split * chunk;
     const int end = L < begin + chunk ? L : begin + chunk;
 
@@ -664,7 +666,10 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     L = L < 0 ? 0 : L;
     L = L > p.max_blocks * BS ? p.max_blocks * BS : L;
     const int NS = p.num_splits;
-    const int chunk = (((L + NS - 1) / NS) + 63) & ~63;
+    // every sequence is cut into the same token chunks (those of the longest possible context):
+    // the work of a workgroup does not depend on its sequence's length, short sequences just
+    // leave their last splits empty
+    const int chunk = (((p.max_blocks * BS + NS - 1) / NS) + 63) & ~63;
     const int begin = split * chunk;
     const int end = L < begin + chunk ? L : begin + chunk;
     const int hq_lane = h * p.G + n;
@@ -907,8 +912,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     float M = -__builtin_inff();
     float lsum = 0.0f;
 
-    auto compute_tile = [&](int t0, int slot, auto masked_tag) {
-        constexpr bool MASKED = decltype(masked_tag)::value;   // the tile may reach past the end of the split
+    auto compute_tile = [&](int t0, int slot) {
         const uint8_t* tile = slots + slot * kTileBytes;
         // operands of this lane, raw
         uint4v kraw[2];
@@ -997,7 +1001,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                 s = acc[e >> 2][e & 3];
                 if (PROD) s2 = acc_s[e >> 2][e & 3];
             }
-            const bool live = !MASKED || t0 + sc_tok[e] < end;
+            const bool live = t0 + sc_tok[e] < end;
             rv[e] = live ? vn[e] : 0.0f;
             float sc = s * kn[e] * qscale;
             if (PROD) sc = __builtin_fmaf(s2 * kg[e], qscale_s, sc);
@@ -1079,8 +1083,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             __syncthreads();                      // tile i is in LDS; slot of tile i - 1 is free
             write_slot((i + 1) & 1);              // tile i + 1 (its loads ran during tile i - 1)
             issue_loads(clamp_t0(t0 + 64));       // tile i + 2
-            if (t0 + 32 <= end) compute_tile(t0, i & 1, std::false_type{});
-            else compute_tile(t0, i & 1, std::true_type{});
+            compute_tile(t0, i & 1);
         }
     }
 
@@ -1203,7 +1206,8 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
                     const int sidx = s0 + k < NS ? s0 + k : NS - 1;
                     mv[k] = part_m[base + sidx];
                     lv[k] = part_l[base + sidx];
-                    // an empty split (m = -inf) never wrote its accumulator: whatever is read there gets weight 0
+                    // An empty split (m = -inf) never wrote its accumulator; it is read all the same
+                    // (and ignored below), so that no load has to wait for another one.
                     const float4v* src = reinterpret_cast<const float4v*>(part_acc + (base + sidx) * D + c0);
                     lo[k] = src[0];
                     hi[k] = src[1];
@@ -1439,11 +1443,16 @@ extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_siz
     if (num_seqs <= 0 || H_KV <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 1;
     const int64_t max_ctx = int64_t(block_size) * max_blocks_per_seq;
     const int64_t tiles = (max_ctx + 63) / 64;
-    // aim at two wavefronts per SIMD over the whole chip, one wavefront per (sequence, KV head, split)
+    // one round of workgroups over the chip (8 wavefronts per CU, one wavefront per sequence,
+    // KV head and split) ...
     const int64_t target_waves = int64_t(fq_host::device_cu_count()) * 8;
-    int64_t ns = (target_waves + int64_t(num_seqs) * H_KV - 1) / (int64_t(num_seqs) * H_KV);
+    const int64_t one_round = (target_waves + int64_t(num_seqs) * H_KV - 1) / (int64_t(num_seqs) * H_KV);
+    // ... and up to four rounds when the contexts are long enough for splits of 1024 tokens: the
+    // lengths of the sequences are not known here, and ragged batches leave many splits empty
+    int64_t ns = 4 * one_round < max_ctx / 1024 ? 4 * one_round : max_ctx / 1024;
+    if (ns < one_round) ns = one_round;
     if (ns > tiles) ns = tiles;
-    if (ns > 64) ns = 64;
+    if (ns > 256) ns = 256;
     const int64_t floor_ns = fq_paged_decode_min_splits(block_size, max_blocks_per_seq);
     if (ns < floor_ns) ns = floor_ns;
     if (ns < 1) ns = 1;
