@@ -356,8 +356,8 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a plain copy
             # (profiles/paged_decode_hbm_traffic_pmc.txt); a measured constant, not read live
-            "traffic": 150.1e6,
-            "kernel": "paged_decode_staged_kernel<4,4,bf16,1>",
+            "traffic": 150.5e6,
+            "kernel": "paged_decode_staged_kernel<4,4,bf16,4,false>",
         },
         "cpu_baseline": cpu,
         "extra": extra,

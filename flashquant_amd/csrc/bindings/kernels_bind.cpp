@@ -330,6 +330,44 @@ at::Tensor prod_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache, co
     return result;
 }
 
+at::Tensor nibble_pack(const at::Tensor& indices) {
+    fqbind::require_gpu(indices, "indices");
+    require(indices.dim() >= 1 && indices.size(-1) % 2 == 0, "Last dimension must be even for nibble packing");
+    int bytes = 0;
+    switch (indices.scalar_type()) {
+        case at::kByte: bytes = 1; break;
+        case at::kInt: bytes = 4; break;
+        case at::kLong: bytes = 8; break;
+        default: throw std::invalid_argument("nibble_pack: indices must be uint8, int32 or int64");
+    }
+    c10::DeviceGuard guard(indices.device());
+    const at::Tensor ic = indices.contiguous();
+    auto shape = ic.sizes().vec();
+    shape.back() /= 2;
+    at::Tensor packed = at::empty(shape, ic.options().dtype(at::kByte));
+    at::Tensor bad = at::zeros({1}, ic.options().dtype(at::kInt));
+    const int st = fq_nibble_pack(ic.data_ptr(), bytes, packed.data_ptr<uint8_t>(), packed.numel(), bad.data_ptr<int>(),
+                                  fqbind::current_stream(indices));
+    fqbind::raise_on_error(st, "nibble_pack");
+    // the reference validates before it packs (csrc/core/packing.cpp:8-19): same error, after the fact
+    if (bad.item<int>() != 0) throw std::invalid_argument("Indices out of range for 4-bit packing. Expected [0, 15]");
+    return packed;
+}
+
+at::Tensor nibble_unpack(const at::Tensor& packed) {
+    fqbind::require_gpu(packed, "packed");
+    require(packed.scalar_type() == at::kByte, "nibble_unpack: packed must be uint8");
+    c10::DeviceGuard guard(packed.device());
+    const at::Tensor pc = packed.contiguous();
+    auto shape = pc.sizes().vec();
+    shape.back() *= 2;
+    at::Tensor out = at::empty(shape, pc.options().dtype(at::kLong));
+    const int st = fq_nibble_unpack(pc.data_ptr<uint8_t>(), out.data_ptr<int64_t>(), pc.numel(),
+                                    fqbind::current_stream(packed));
+    fqbind::raise_on_error(st, "nibble_unpack");
+    return out;
+}
+
 at::Tensor rotate_query(const at::Tensor& q, const at::Tensor& rotation) {
     fqbind::require_gpu(q, "q");
     require(q.dim() == 3 && (q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16),
@@ -451,6 +489,8 @@ void bind_kernels(py::module_& m) {
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),
           py::arg("out") = py::none(), py::arg("num_splits") = 0,
           "Split-K paged decode over TurboQuantProd key / TQ4 value pages");
+    m.def("nibble_pack", &nibble_pack, py::arg("indices"), "Pack pairs of 4-bit indices (..., D) into bytes (..., D/2)");
+    m.def("nibble_unpack", &nibble_unpack, py::arg("packed"), "Unpack bytes (..., D/2) into int64 indices (..., D)");
     m.def("rotate_query", &rotate_query, py::arg("q"), py::arg("rotation"),
           "q_rot = (q @ rotation.T) rounded to q's dtype.");
     m.def("paged_tq4_decode_partials", &paged_tq4_decode_partials, py::arg("q_rot"), py::arg("kv_cache"),

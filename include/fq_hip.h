@@ -207,6 +207,19 @@ int fq_split_k_reduce(const float* partial_acc, const float* partial_m,
                       void* stream);
 
 /*
+ * Nibble pack / unpack of 4-bit indices (src/flashquant/core/packing.py:54-98; C++ twin
+ * csrc/core/packing.cpp:21-46).
+ *   fq_nibble_pack    indices: 2 * n_packed values of index_bytes (1: uint8, 4: int32, 8: int64)
+ *                     bytes each; packed[j] = idx[2j] << 4 | idx[2j+1].  *bad_count (device int,
+ *                     zeroed by the caller) is raised when an index lies outside [0, 15]: the
+ *                     reference rejects such input (validate_indices, csrc/core/packing.cpp:8-19).
+ *   fq_nibble_unpack  indices (int64, as the Python fallback returns): [high, low] interleaved.
+ */
+int fq_nibble_pack(const void* indices, int index_bytes, uint8_t* packed, int64_t n_packed,
+                   int* bad_count, void* stream);
+int fq_nibble_unpack(const uint8_t* packed, int64_t* indices, int64_t n_packed, void* stream);
+
+/*
  * TurboQuantProd keys (3-bit Lloyd-Max index + 1-bit sign sketch of the residual) with
  * TQ4 values, as pages.  The reference defines the quantizer
  * (TurboQuantProd.quantize / estimate_inner_product, src/flashquant/core/quantizer.py:285-370;

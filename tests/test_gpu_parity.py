@@ -486,3 +486,31 @@ def test_prod_entry_points_reject_unsupported_shapes():
         K.prod_paged_decode(q, cache, table, sl, c3.to(DEV), c4.to(DEV), r.to(DEV), s.to(DEV), 4, 128, 16)
     with pytest.raises(ValueError):          # 4-bit codebook where the 3-bit one is expected
         K.prod_compress(torch.zeros(4, 8, 128, dtype=torch.bfloat16, device=DEV), r.to(DEV), s.to(DEV), b4.to(DEV), c4.to(DEV))
+
+
+# ---- nibble packing on the GPU: bit exact ---------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int32, torch.int64])
+def test_nibble_pack_unpack_bit_exact(dtype):
+    g = torch.Generator().manual_seed(5)
+    idx = torch.randint(0, 16, (7, 3, 130), generator=g).to(dtype)
+    packed = K.nibble_pack(idx.to(DEV))
+    assert packed.dtype == torch.uint8 and packed.shape == (7, 3, 65)
+    assert torch.equal(packed.cpu(), O.nibble_pack(idx))
+    back = K.nibble_unpack(packed)
+    assert back.dtype == torch.int64 and torch.equal(back.cpu(), idx.long())
+    # every byte value, and the known answer of the reference's tests (tests/test_packing.py:46-64)
+    allb = torch.arange(256, dtype=torch.uint8)
+    assert torch.equal(K.nibble_unpack(allb.to(DEV)).cpu(), O.nibble_unpack(allb))
+    known = torch.tensor([0x0, 0xF, 0xA, 0x5], dtype=dtype)
+    assert K.nibble_pack(known.to(DEV)).cpu().tolist() == [0x0F, 0xA5]
+
+
+def test_nibble_pack_rejects_bad_input():
+    with pytest.raises(ValueError):
+        K.nibble_pack(torch.zeros(4, 3, dtype=torch.uint8, device=DEV))          # odd last dimension
+    with pytest.raises(ValueError):
+        K.nibble_pack(torch.tensor([1, 16], dtype=torch.int64, device=DEV))       # 16 does not fit a nibble
+    with pytest.raises(ValueError):
+        K.nibble_pack(torch.tensor([-1, 3], dtype=torch.int32, device=DEV))
+    assert K.nibble_pack(torch.zeros(0, 8, dtype=torch.uint8, device=DEV)).shape == (0, 4)
