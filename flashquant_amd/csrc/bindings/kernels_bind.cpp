@@ -248,6 +248,57 @@ at::Tensor fused_tq_attention(const at::Tensor& q, const at::Tensor& k_packed, c
     return result;
 }
 
+at::Tensor paged_tq4_prefill(const at::Tensor& q, const at::Tensor& cu_seqlens_q, int64_t max_seqlen_q,
+                             const at::Tensor& kv_cache, const at::Tensor& block_table, const at::Tensor& seq_lens,
+                             const at::Tensor& centroids_k, const at::Tensor& centroids_v,
+                             const at::Tensor& rotation, int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                             std::optional<double> sm_scale, bool causal, std::optional<at::Tensor> out) {
+    fqbind::require_gpu(q, "q");
+    fqbind::require_gpu(kv_cache, "kv_cache");
+    fqbind::require_gpu(block_table, "block_table");
+    fqbind::require_gpu(seq_lens, "seq_lens");
+    fqbind::require_gpu(cu_seqlens_q, "cu_seqlens_q");
+    require(q.dim() == 3 && q.size(2) == head_dim, "q must have shape (tokens, H_Q, head_dim)");
+    require(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, "q must be float16 or bfloat16");
+    const int64_t T = q.size(0), HQ = q.size(1);
+    require(num_kv_heads > 0 && HQ % num_kv_heads == 0, "H_Q must be a multiple of num_kv_heads");
+    require(kv_cache.dim() == 3 && kv_cache.scalar_type() == at::kByte && kv_cache.size(1) == block_size &&
+                kv_cache.size(2) == num_kv_heads * (head_dim + 8) && kv_cache.is_contiguous(),
+            "kv_cache must be contiguous uint8 of shape (num_blocks, block_size, H_KV * (head_dim + 8))");
+    require(block_table.dim() == 2 && block_table.scalar_type() == at::kInt, "block_table must be int32 (S, max_blocks)");
+    const int64_t S = block_table.size(0);
+    require(seq_lens.scalar_type() == at::kInt && seq_lens.numel() == S, "seq_lens must be int32 of shape (S,)");
+    require(cu_seqlens_q.scalar_type() == at::kInt && cu_seqlens_q.numel() == S + 1,
+            "cu_seqlens_q must be int32 of shape (S + 1,)");
+    require(max_seqlen_q >= 0 && max_seqlen_q <= T, "max_seqlen_q must lie in [0, tokens]");
+    require(centroids_k.numel() == 16 && centroids_v.numel() == 16 && centroids_k.scalar_type() == at::kFloat &&
+                centroids_v.scalar_type() == at::kFloat,
+            "centroids must be 16 float32 values");
+    c10::DeviceGuard guard(q.device());
+    const double scale = sm_scale.has_value() ? *sm_scale : 1.0 / std::sqrt(double(head_dim));
+    const at::Tensor qc = q.contiguous();
+    const at::Tensor bt = block_table.contiguous(), sl = seq_lens.contiguous(), cu = cu_seqlens_q.contiguous();
+    const at::Tensor ck = centroids_k.to(q.device()).contiguous(), cv = centroids_v.to(q.device()).contiguous();
+    const RotationArg rot = rotation_arg(rotation, q.device(), head_dim);
+    at::Tensor result;
+    if (out.has_value()) {
+        require(out->sizes() == qc.sizes() && out->scalar_type() == q.scalar_type() && out->is_contiguous() &&
+                    out->device() == q.device(),
+                "out must be contiguous with the shape, dtype and device of q");
+        result = *out;
+    } else {
+        result = at::zeros_like(qc);
+    }
+    const int st = fq_paged_tq4_prefill(
+        qc.data_ptr(), cu.data_ptr<int32_t>(), kv_cache.data_ptr<uint8_t>(), bt.data_ptr<int32_t>(),
+        sl.data_ptr<int32_t>(), ck.data_ptr<float>(), cv.data_ptr<float>(), rot.ptr, rot.col_major, result.data_ptr(),
+        int(S), int(max_seqlen_q), int(HQ), int(num_kv_heads), int(head_dim), int(block_size), int(bt.size(1)),
+        kv_cache.size(0), float(scale), causal ? 1 : 0, fqbind::dtype_code(q.scalar_type(), "paged_tq4_prefill"),
+        fqbind::current_stream(q));
+    fqbind::raise_on_error(st, "paged_tq4_prefill");
+    return result;
+}
+
 std::tuple<at::Tensor, at::Tensor, at::Tensor> prod_compress(const at::Tensor& x, const at::Tensor& rotation,
                                                              const at::Tensor& sketch_rot, const at::Tensor& boundaries,
                                                              const at::Tensor& centroids) {
@@ -481,6 +532,12 @@ void bind_kernels(py::module_& m) {
           py::arg("v_packed"), py::arg("v_norms"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),
           py::arg("sm_scale") = py::none(), py::arg("is_causal") = false,
           "Fused TQ4 attention: un-rotated q (B, H_Q, N_Q, D) over packed K/V, original-space output");
+    m.def("paged_tq4_prefill", &paged_tq4_prefill, py::arg("q"), py::arg("cu_seqlens_q"), py::arg("max_seqlen_q"),
+          py::arg("kv_cache"), py::arg("block_table"), py::arg("seq_lens"), py::arg("centroids_k"),
+          py::arg("centroids_v"), py::arg("rotation"), py::arg("num_kv_heads"), py::arg("head_dim"),
+          py::arg("block_size"), py::arg("sm_scale") = py::none(), py::arg("causal") = true,
+          py::arg("out") = py::none(),
+          "Variable-length prefill over the packed paged TQ4 cache: un-rotated q (tokens, H_Q, D), original-space output");
     m.def("prod_compress", &prod_compress, py::arg("x"), py::arg("rotation"), py::arg("sketch_rot"),
           py::arg("boundaries"), py::arg("centroids"),
           "TurboQuantProd key compress: (packed nibbles sign<<3|idx (N,H,D/2), norms (N,H,1), residual norms (N,H,1))");

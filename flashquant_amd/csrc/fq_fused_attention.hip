@@ -57,6 +57,12 @@ struct PrefillParams {
     int H_Q, H_KV, G, N_Q, N_KV;
     int causal;
     float scale_log2e;
+    // paged mode (variable-length queries over the packed paged cache)
+    const int32_t* cu_seqlens_q;   // (S + 1,) first query token of every sequence in q / out (tokens, H_Q, 128)
+    const int32_t* seq_lens;       // (S,) keys of every sequence, the new tokens included
+    const int32_t* block_table;    // (S, max_blocks)
+    const uint8_t* cache;          // (num_blocks, block_size, H_KV * 136)
+    int max_blocks, num_blocks, bs_log2;
 };
 
 __device__ __forceinline__ uint32_t scale_pair(uint32_t pair, half2v n2) {
@@ -68,7 +74,12 @@ __device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
 }
 
-template <int DT>
+// PAGED: the sequences' queries are packed along the token axis of q (tokens, H_Q, 128), the keys
+// and values come from the paged TQ4 cache through the block table, query j of a sequence with
+// n queries and L keys sits at position L - n + j (the new tokens are the last ones), and the
+// attention result is rounded to the query dtype before the rotation back, as the attention
+// library's output is in the path this replaces (src/flashquant/vllm/impl.py:265-336, 470-512).
+template <int DT, bool PAGED>
 __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillParams p) {
     constexpr int D = 128;
     __shared__ __attribute__((aligned(256))) uint32_t lut[256 * 64];
@@ -81,10 +92,26 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const int n16 = lane & 15, g4 = lane >> 4;     // 16x16 MFMA of the rotations
     const int b = blockIdx.z, hkv = blockIdx.y;
 
+    // ---- this sequence -----------------------------------------------------------------------
+    int NQ = p.N_Q, NKV = p.N_KV, qoff = 0;
+    int64_t q_row0 = (int64_t(b) * p.H_Q) * p.N_Q;     // first row of head 0 in q / out, in rows of 128
+    int q_stride = D;                                  // elements between consecutive positions of a head
+    if (PAGED) {
+        const int first = p.cu_seqlens_q[b];
+        NQ = p.cu_seqlens_q[b + 1] - first;
+        NKV = p.seq_lens[b];
+        NKV = NKV < 0 ? 0 : (NKV > (p.max_blocks << p.bs_log2) ? (p.max_blocks << p.bs_log2) : NKV);
+        qoff = NKV - NQ > 0 ? NKV - NQ : 0;
+        q_row0 = int64_t(first) * p.H_Q;
+        q_stride = p.H_Q * D;
+        if (NQ <= 0) return;
+    }
+
     // ---- units --------------------------------------------------------------------------
-    const int nblk = (p.N_Q + 31) >> 5;
+    const int nblk = (NQ + 31) >> 5;
     const int units = nblk * p.G;
     const int wg = int(gridDim.x) - 1 - int(blockIdx.x);   // late (long) query blocks start first
+    if (PAGED && 8 * wg >= units) return;                  // the grid is sized for the longest sequence
     const int unit_raw = 8 * wg + w;
     const bool unit_live = unit_raw < units;
     const int unit = unit_live ? unit_raw : units - 1;
@@ -92,13 +119,13 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const int pos0 = 32 * (unit / p.G);
     const int last_unit = 8 * wg + 7 < units - 1 ? 8 * wg + 7 : units - 1;
     int wg_maxpos = 32 * (last_unit / p.G) + 31;
-    wg_maxpos = wg_maxpos < p.N_Q - 1 ? wg_maxpos : p.N_Q - 1;
-    int my_maxpos = pos0 + 31 < p.N_Q - 1 ? pos0 + 31 : p.N_Q - 1;
-    const int all_tiles = (p.N_KV + 63) >> 6;
+    wg_maxpos = wg_maxpos < NQ - 1 ? wg_maxpos : NQ - 1;
+    int my_maxpos = pos0 + 31 < NQ - 1 ? pos0 + 31 : NQ - 1;
+    const int all_tiles = (NKV + 63) >> 6;
     int ntiles = all_tiles, my_tiles = all_tiles;
     if (p.causal) {
-        ntiles = (wg_maxpos >> 6) + 1 < all_tiles ? (wg_maxpos >> 6) + 1 : all_tiles;
-        my_tiles = (my_maxpos >> 6) + 1 < all_tiles ? (my_maxpos >> 6) + 1 : all_tiles;
+        ntiles = ((qoff + wg_maxpos) >> 6) + 1 < all_tiles ? ((qoff + wg_maxpos) >> 6) + 1 : all_tiles;
+        my_tiles = ((qoff + my_maxpos) >> 6) + 1 < all_tiles ? ((qoff + my_maxpos) >> 6) + 1 : all_tiles;
     }
     if (!unit_live) my_tiles = 0;
 
@@ -108,7 +135,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const uint32_t lk = 4u * (lane & 31), lv = 128u + lk;
 
     // ---- dequantisation plan ------------------------------------------------------------------
-    const int64_t kv_row0 = (int64_t(b) * p.H_KV + hkv) * p.N_KV;
+    const int64_t kv_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.N_KV;
     const uint8_t* kp = p.k_packed + kv_row0 * 64;
     const uint8_t* vp = p.v_packed + kv_row0 * 64;
     const float* knp = p.k_norms + kv_row0;
@@ -133,17 +160,39 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     float nk, nv0, nv1;
     auto issue_loads = [&](int tile_raw) {
         const int tile = tile_raw < ntiles ? tile_raw : ntiles - 1;   // past the end: the last tile again, never used
-        const int t0 = tile * 64;
-        const int last = p.N_KV - 1;
+        const int t0 = tile > 0 ? tile * 64 : 0;
+        const int last = NKV > 0 ? NKV - 1 : 0;
         const int tkk = t0 + tk < last ? t0 + tk : last;
         const int ta = t0 + 2 * tp < last ? t0 + 2 * tp : last;
         const int tb = t0 + 2 * tp + 1 < last ? t0 + 2 * tp + 1 : last;
-        kraw = *reinterpret_cast<const uint2v*>(kp + int64_t(tkk) * 64 + 8 * gqk);
-        nk = knp[tkk];
-        vra = *reinterpret_cast<const uint32_t*>(vp + int64_t(ta) * 64 + 4 * jv);
-        vrb = *reinterpret_cast<const uint32_t*>(vp + int64_t(tb) * 64 + 4 * jv);
-        nv0 = vnp[ta];
-        nv1 = vnp[tb];
+        if (PAGED) {
+            // token t of the sequence: row t % BS of page block_table[t / BS]; the row holds
+            // [K idx H*64 | K norm H*4 | V idx H*64 | V norm H*4]
+            const int H = p.H_KV;
+            const int64_t row_bytes = int64_t(H) * 136;
+            const int32_t* bt = p.block_table + int64_t(b) * p.max_blocks;
+            auto row_ptr = [&](int t) {
+                int pg = bt[t >> p.bs_log2];
+                pg = pg < 0 ? 0 : (pg >= p.num_blocks ? p.num_blocks - 1 : pg);
+                return p.cache + ((int64_t(pg) << p.bs_log2) + (t & ((1 << p.bs_log2) - 1))) * row_bytes;
+            };
+            const uint8_t* rk = row_ptr(tkk);
+            const uint8_t* ra = row_ptr(ta);
+            const uint8_t* rb2 = row_ptr(tb);
+            kraw = *reinterpret_cast<const uint2v*>(rk + hkv * 64 + 8 * gqk);
+            nk = *reinterpret_cast<const float*>(rk + H * 64 + 4 * hkv);
+            vra = *reinterpret_cast<const uint32_t*>(ra + H * 68 + hkv * 64 + 4 * jv);
+            vrb = *reinterpret_cast<const uint32_t*>(rb2 + H * 68 + hkv * 64 + 4 * jv);
+            nv0 = *reinterpret_cast<const float*>(ra + H * 132 + 4 * hkv);
+            nv1 = *reinterpret_cast<const float*>(rb2 + H * 132 + 4 * hkv);
+        } else {
+            kraw = *reinterpret_cast<const uint2v*>(kp + int64_t(tkk) * 64 + 8 * gqk);
+            nk = knp[tkk];
+            vra = *reinterpret_cast<const uint32_t*>(vp + int64_t(ta) * 64 + 4 * jv);
+            vrb = *reinterpret_cast<const uint32_t*>(vp + int64_t(tb) * 64 + 4 * jv);
+            nv0 = vnp[ta];
+            nv1 = vnp[tb];
+        }
     };
     auto dequant = [&](int buf) {
         uint8_t* dst = bufs + buf * kPfBufBytes;
@@ -176,7 +225,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     half8 qb[8];
     float krow;
     {
-        const uint16_t* qbase = p.q + ((int64_t(b) * p.H_Q + hq) * p.N_Q) * D;
+        const uint16_t* qbase = PAGED ? p.q + (q_row0 + hq) * D : p.q + (q_row0 + int64_t(hq) * NQ) * D;
         uint16_t* st = reinterpret_cast<uint16_t*>(bufs + w * kPfStageBytes);   // (32 rows, 128) raw 16-bit
         // the rows are exact in fp16 up to a power of two: fp16-split MFMA, two terms
         half8 a[2][4];
@@ -184,10 +233,10 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             int pos = pos0 + 16 * rb + n16;
-            pos = pos < p.N_Q ? pos : p.N_Q - 1;
+            pos = pos < NQ ? pos : NQ - 1;
             uint4v raw[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) raw[j] = *reinterpret_cast<const uint4v*>(qbase + int64_t(pos) * D + 32 * j + 8 * g4);
+            for (int j = 0; j < 4; ++j) raw[j] = *reinterpret_cast<const uint4v*>(qbase + int64_t(pos) * q_stride + 32 * j + 8 * g4);
             rows_as_f16<D, DT>(raw, a[rb], up[rb]);
         }
         for (int cb = 0; cb < 8; ++cb) {
@@ -246,7 +295,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
         for (int r = 0; r < 16; ++r) O[ob][r] = 0.0f;
     float m_run = -__builtin_inff();
     float l_run = 0.0f;
-    const int qpos = pos0 + m32;
+    const int qpos = qoff + pos0 + m32;            // position among the keys
 
     auto compute = [&](int tile, int buf) {
         const uint8_t* kt = bufs + buf * kPfBufBytes;
@@ -262,9 +311,9 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             }
         }
         const int t0 = tile * 64;
-        const bool need_mask = (t0 + 63 >= p.N_KV) || (p.causal && t0 + 63 > pos0);   // wavefront-uniform
+        const bool need_mask = (t0 + 63 >= NKV) || (p.causal && t0 + 63 > qoff + pos0);   // wavefront-uniform
         if (need_mask) {
-            int lim = p.N_KV - 1;
+            int lim = NKV - 1;
             if (p.causal && qpos < lim) lim = qpos;
             lim -= t0;                         // token offsets <= lim are visible
 #pragma unroll
@@ -340,7 +389,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const float l_tot = l_run + xor_shuffle(l_run, 32);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     float* stf = reinterpret_cast<float*>(bufs + w * kPfStageBytes);   // (16 rows, 128) float32
-    uint16_t* obase = p.out + ((int64_t(b) * p.H_Q + hq) * p.N_Q) * D;
+    uint16_t* obase = PAGED ? p.out + (q_row0 + hq) * D : p.out + (q_row0 + int64_t(hq) * NQ) * D;
     for (int half_rows = 0; half_rows < 2; ++half_rows) {
         __syncthreads();
         if ((m32 >> 4) == half_rows) {
@@ -348,7 +397,11 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             for (int ob = 0; ob < 4; ++ob)
 #pragma unroll
                 for (int rq = 0; rq < 4; ++rq) {
-                    const float4v v = {O[ob][4 * rq] * inv, O[ob][4 * rq + 1] * inv, O[ob][4 * rq + 2] * inv, O[ob][4 * rq + 3] * inv};
+                    float4v v = {O[ob][4 * rq] * inv, O[ob][4 * rq + 1] * inv, O[ob][4 * rq + 2] * inv, O[ob][4 * rq + 3] * inv};
+                    if (PAGED) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = load_elem<DT>(store_elem<DT>(v[e]));
+                    }
                     *reinterpret_cast<float4v*>(stf + (m32 & 15) * D + 32 * ob + 8 * rq + 4 * hf) = v;
                 }
         }
@@ -374,7 +427,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int pos = pos0 + 16 * half_rows + 4 * g4 + i;
-                if (unit_live && pos < p.N_Q) obase[int64_t(pos) * D + 16 * cb + n16] = store_elem<DT>(acc[i] * up);
+                if (unit_live && pos < NQ) obase[int64_t(pos) * q_stride + 16 * cb + n16] = store_elem<DT>(acc[i] * up);
             }
         }
     }
@@ -418,12 +471,68 @@ extern "C" int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, con
     const dim3 grid(static_cast<unsigned>(wgs), H_KV, B), block(512);
     const size_t lds = 2 * size_t(kPfBufBytes);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    p.cu_seqlens_q = nullptr; p.seq_lens = nullptr; p.block_table = nullptr; p.cache = nullptr;
+    p.max_blocks = 0; p.num_blocks = 0; p.bs_log2 = 0;
     if (dtype == FQ_F16) {
-        auto kern = fused_tq_attention_kernel<FQ_F16>;
+        auto kern = fused_tq_attention_kernel<FQ_F16, false>;
         if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, grid, block, lds, s, p);
     } else {
-        auto kern = fused_tq_attention_kernel<FQ_BF16>;
+        auto kern = fused_tq_attention_kernel<FQ_BF16, false>;
+        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
+    }
+    return fq_host::check_launch();
+}
+
+extern "C" int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, const uint8_t* kv_cache,
+                                    const int32_t* block_table, const int32_t* seq_lens,
+                                    const float* centroids_k, const float* centroids_v,
+                                    const float* rotation, int rotation_col_major, void* out,
+                                    int num_seqs, int max_q_len, int H_Q, int H_KV, int D, int block_size,
+                                    int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int is_causal,
+                                    int dtype, void* stream) {
+    using namespace fq;
+    if (num_seqs < 0 || max_q_len < 0 || H_Q <= 0 || H_KV <= 0 || H_Q % H_KV != 0 || max_blocks_per_seq <= 0 ||
+        num_blocks <= 0 || num_blocks > 0x7fffffffLL)
+        return FQ_ERR_BAD_SHAPE;
+    if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
+    if (D != 128) return FQ_ERR_UNSUPPORTED_DIM;
+    if (block_size != 8 && block_size != 16 && block_size != 32) return FQ_ERR_UNSUPPORTED_BLOCK;
+    if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
+    if (num_seqs == 0 || max_q_len == 0) return FQ_OK;
+    if (!q || !cu_seqlens_q || !kv_cache || !block_table || !seq_lens || !centroids_k || !centroids_v || !rotation || !out)
+        return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(q, 16) || !fq_host::aligned(kv_cache, 16) || !fq_host::aligned(rotation, 16) ||
+        !fq_host::aligned(out, 2))
+        return FQ_ERR_MISALIGNED;
+    if (num_seqs > 65535 || H_KV > 65535) return FQ_ERR_BAD_SHAPE;
+
+    PrefillParams p;
+    p.q = static_cast<const uint16_t*>(q);
+    p.k_packed = nullptr; p.k_norms = nullptr; p.v_packed = nullptr; p.v_norms = nullptr;
+    p.centroids_k = centroids_k; p.centroids_v = centroids_v;
+    p.rotation = rotation; p.rot_col_major = rotation_col_major;
+    p.out = static_cast<uint16_t*>(out);
+    p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.N_Q = 0; p.N_KV = 0;
+    p.causal = is_causal ? 1 : 0;
+    p.scale_log2e = sm_scale * kLog2e;
+    p.cu_seqlens_q = cu_seqlens_q; p.seq_lens = seq_lens; p.block_table = block_table; p.cache = kv_cache;
+    p.max_blocks = max_blocks_per_seq; p.num_blocks = int(num_blocks);
+    p.bs_log2 = block_size == 8 ? 3 : (block_size == 16 ? 4 : 5);
+
+    const int64_t units = int64_t((max_q_len + 31) / 32) * p.G;
+    const int64_t wgs = (units + 7) / 8;
+    if (wgs > 0x7fffffffLL) return FQ_ERR_BAD_SHAPE;
+    const dim3 grid(static_cast<unsigned>(wgs), H_KV, num_seqs), block(512);
+    const size_t lds = 2 * size_t(kPfBufBytes);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == FQ_F16) {
+        auto kern = fused_tq_attention_kernel<FQ_F16, true>;
+        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
+    } else {
+        auto kern = fused_tq_attention_kernel<FQ_BF16, true>;
         if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, grid, block, lds, s, p);
     }

@@ -132,6 +132,38 @@ int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, const float* k
                           float sm_scale, int is_causal, int dtype, void* stream);
 
 /*
+ * Prefill over the packed paged TQ4 cache: un-rotated queries of several
+ * sequences packed along the token axis, keys and values read from the cache
+ * through the block table, original-space output.  One launch for what the
+ * serving backend does in four steps: rotate the query, decompress the whole
+ * cache to fp16/bf16, variable-length attention through the block table,
+ * rotate the result back (src/flashquant/vllm/impl.py:317-336 and 470-512;
+ * the decompression is impl.py:265-315).  The tokens' own keys and values must
+ * already be in the cache (fq_tq4_compress_store), as in the reference, which
+ * stores before it attends (impl.py:320-323).
+ *
+ *   q             (total_q, H_Q, D) fp16/bf16, contiguous, 16-byte aligned
+ *   cu_seqlens_q  (num_seqs + 1,) int32, first query token of every sequence,
+ *                 non-decreasing, cu_seqlens_q[num_seqs] == total_q
+ *   kv_cache, block_table, seq_lens   as in fq_split_k_paged_decode; seq_lens
+ *                 counts the new tokens too, so seq_lens[s] >= the sequence's
+ *                 query count
+ *   out           (total_q, H_Q, D) same dtype as q
+ *   max_q_len     the largest query count of a sequence (sizes the grid)
+ *   is_causal     query j of n in a sequence of L keys sees keys 0 .. L - n + j
+ * The attention result is rounded to the query dtype before the rotation back,
+ * as the attention library's output is in the reference.  A sequence with no
+ * queries is skipped; with no keys its rows are zero.  D == 128.
+ */
+int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, const uint8_t* kv_cache,
+                         const int32_t* block_table, const int32_t* seq_lens,
+                         const float* centroids_k, const float* centroids_v,
+                         const float* rotation, int rotation_col_major, void* out,
+                         int num_seqs, int max_q_len, int H_Q, int H_KV, int D, int block_size,
+                         int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int is_causal,
+                         int dtype, void* stream);
+
+/*
  * Split-K paged decode from the packed TQ4 cache, un-rotated query in,
  * original-space output out.  Takes the roles of paged_tq4_decode_cuda
  * (csrc/cuda/paged_decode.cu:346-368) and split_k_reduce_cuda

@@ -30,6 +30,10 @@ Pinned by (see tests/test_oracle_*.py):
       torch.nn.functional.scaled_dot_product_attention, rotated-space identity.
   paged_decode_loop / paged_decode_gather
       each other, block-table permutation invariance, SDPA over gathered rows.
+  paged_prefill
+      fused_tq_attention on the same tokens (one page run per sequence, full
+      queries), paged_decode_gather for one query per sequence, SDPA with an
+      explicit bottom-right mask for a chunked prefill.
   prod_quantize / prod_inner_product
       unbiasedness of the estimator over many draws, sign/zero rule.
   prod_paged_decode
@@ -475,6 +479,63 @@ def split_k_paged_decode(
     fn = paged_decode_loop if faithful_loop else paged_decode_gather
     out_rot = fn(q_rot, kv_cache, block_table, seq_lens, centroids_k, centroids_v,
                  num_kv_heads, head_dim, block_size, sm_scale=sm_scale)
+    return torch.matmul(out_rot.float(), rotation).to(q.dtype)
+
+
+def paged_prefill(
+    q: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    kv_cache: torch.Tensor,
+    block_table: torch.Tensor,
+    seq_lens: torch.Tensor,
+    centroids_k: torch.Tensor,
+    centroids_v: torch.Tensor,
+    rotation: torch.Tensor,
+    num_kv_heads: int,
+    head_dim: int,
+    block_size: int,
+    sm_scale: Optional[float] = None,
+    causal: bool = True,
+) -> torch.Tensor:
+    """Prefill over the packed paged cache as the serving backend computes it
+    (src/flashquant/vllm/impl.py:317-336 and 470-512): the queries of all
+    sequences are packed along the token axis, q (T, HQ, D); q_rot =
+    (q.float() @ R.T).to(q.dtype); the cache is decompressed in rotated space
+    to q.dtype (impl.py:298-305); a variable-length attention over
+    (cu_seqlens_q, seq_lens, block_table) gives a q.dtype result, which is
+    multiplied by R in float32 and cast to q.dtype (impl.py:506-510).
+
+    The attention call itself belongs to vllm's flash-attention library, which
+    is not in the reference checkout; its published semantics are restated:
+    float32 scores and softmax, a causal mask aligned to the bottom-right
+    corner (query j of n sees keys 0 .. L - n + j), result cast to q.dtype.
+    """
+    total, hq, d = q.shape
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(head_dim)
+    rep = hq // num_kv_heads
+    q_rot = torch.matmul(q.float(), rotation.T).to(q.dtype)
+    out_rot = torch.zeros_like(q_rot)
+    for s in range(seq_lens.shape[0]):
+        first, end = int(cu_seqlens_q[s]), int(cu_seqlens_q[s + 1])
+        n, length = end - first, int(seq_lens[s])
+        if n == 0 or length == 0:
+            continue
+        k, v = gather_sequence(kv_cache, block_table[s], length, centroids_k, centroids_v,
+                               num_kv_heads, head_dim, block_size)
+        k = k.to(q.dtype).float()
+        v = v.to(q.dtype).float()
+        if rep > 1:
+            k = k.repeat_interleave(rep, dim=0)
+            v = v.repeat_interleave(rep, dim=0)
+        qs = q_rot[first:end].float().permute(1, 0, 2)                 # (HQ, n, D)
+        sc = torch.bmm(qs, k.transpose(-2, -1)) * sm_scale             # (HQ, n, L)
+        if causal:
+            key_pos = torch.arange(length)[None, :]
+            q_pos = (length - n + torch.arange(n))[:, None]
+            sc = sc.masked_fill((key_pos > q_pos)[None], float("-inf"))
+        w = torch.softmax(sc, dim=-1)
+        out_rot[first:end] = torch.bmm(w, v).permute(1, 0, 2).to(q.dtype)
     return torch.matmul(out_rot.float(), rotation).to(q.dtype)
 
 

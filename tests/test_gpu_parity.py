@@ -312,6 +312,102 @@ def test_fused_attention_rejects_bad_arguments():
         K.fused_tq_attention(q, *dev[1:5], dev[5], dev[5], dev[6])                  # CPU query
 
 
+# ---- prefill over the packed paged cache -------------------------------------------------
+
+def _check_paged_prefill(q_lens, kv_lens, hq, hkv, bs=16, dtype=torch.bfloat16, causal=True, seed=21, scale=None,
+                         kv_scale=1.0, cv=None):
+    """q_lens[s] new tokens at the end of a sequence of kv_lens[s] keys."""
+    c, bnd, r = book(128)
+    cv = c if cv is None else cv
+    _, cache, table, sl = build_paged_case(kv_lens, hq, hkv, bs=bs, seed=seed, dtype=dtype, kv_scale=kv_scale)
+    g = torch.Generator().manual_seed(seed + 100)
+    total = sum(q_lens)
+    q = torch.randn(total, hq, 128, generator=g).to(dtype)
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    want = O.paged_prefill(q, cu, cache, table, sl, c, cv, r, hkv, 128, bs, sm_scale=scale, causal=causal)
+    out = torch.full_like(q, 7.0).to(DEV)
+    got = K.paged_tq4_prefill(q.to(DEV), cu.to(DEV), max(q_lens), cache.to(DEV), table.to(DEV), sl.to(DEV),
+                              c.to(DEV), cv.to(DEV), r.to(DEV), hkv, 128, bs, sm_scale=scale, causal=causal, out=out)
+    torch.cuda.synchronize()
+    assert got.data_ptr() == out.data_ptr() and got.dtype == dtype and got.shape == q.shape
+    got = got.cpu().float()
+    for s, (n, L) in enumerate(zip(q_lens, kv_lens)):
+        if n and not L:                      # no keys: zero rows
+            assert (got[int(cu[s]):int(cu[s + 1])] == 0).all()
+    err = (got - want.float()).abs().max().item()
+    tol = 2e-2 * max(1.0, want.float().abs().max().item())
+    assert math.isfinite(err) and err <= tol, f"max abs error {err} (tolerance {tol})"
+    return err
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+def test_paged_prefill_llama_heads_full_prompts(dtype, causal):
+    _check_paged_prefill([70, 33, 200, 1], [70, 33, 200, 1], hq=32, hkv=8, dtype=dtype, causal=causal)
+
+
+def test_paged_prefill_chunks_on_existing_context():
+    # new tokens after a cached prefix: the mask is aligned to the bottom-right corner
+    _check_paged_prefill([7, 64, 1, 130, 32], [45, 64, 300, 131, 500], hq=32, hkv=8)
+
+
+def test_paged_prefill_mixed_with_decode_and_idle_sequences():
+    # one query (a decode step), no queries (skipped), no keys (zero rows)
+    _check_paged_prefill([1, 0, 5, 96, 3], [257, 40, 5, 96, 0], hq=16, hkv=8)
+
+
+@pytest.mark.parametrize("bs", [8, 16, 32])
+def test_paged_prefill_page_sizes(bs):
+    _check_paged_prefill([50, 129], [77, 129], hq=8, hkv=2, bs=bs)
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 8), (4, 1), (12, 4), (5, 1), (64, 8)])
+def test_paged_prefill_group_sizes(hq, hkv):
+    _check_paged_prefill([40, 65], [40, 100], hq=hq, hkv=hkv)
+
+
+def test_paged_prefill_scaled_inputs_custom_scale_and_value_codebook():
+    c, _, _ = book(128)
+    _check_paged_prefill([90, 31], [120, 31], hq=8, hkv=2, dtype=torch.float16, kv_scale=6.0, scale=0.05,
+                         cv=(c * 1.25).contiguous())
+
+
+def test_paged_prefill_long_sequence_equals_decode_on_last_token():
+    """Size-independent property: the last query of a prefill sees what a decode step
+    with the same query sees."""
+    c, bnd, r = book(128)
+    L, hq, hkv, bs = 2100, 32, 8, 16
+    _, cache, table, sl = build_paged_case([L], hq, hkv, bs=bs, seed=33)
+    g = torch.Generator().manual_seed(34)
+    q = torch.randn(L, hq, 128, generator=g).to(torch.bfloat16).to(DEV)
+    cu = torch.tensor([0, L], dtype=torch.int32, device=DEV)
+    dev = [t.to(DEV) for t in (cache, table, sl, c, r)]
+    full = K.paged_tq4_prefill(q, cu, L, dev[0], dev[1], dev[2], dev[3], dev[3], dev[4], hkv, 128, bs)
+    dec = K.split_k_paged_decode(q[-1:].contiguous(), dev[0], dev[1], dev[2], dev[3], dev[3], dev[4], hkv, 128, bs)
+    assert (full[-1:].float() - dec.float()).abs().max().item() <= 2e-2
+    # and a chunk of the last 100 tokens reproduces the full prefill's last 100 rows bit for bit
+    cu2 = torch.tensor([0, 100], dtype=torch.int32, device=DEV)
+    part = K.paged_tq4_prefill(q[-100:].contiguous(), cu2, 100, dev[0], dev[1], dev[2], dev[3], dev[3], dev[4],
+                               hkv, 128, bs)
+    assert (part.float() - full[-100:].float()).abs().max().item() <= 2e-2
+
+
+def test_paged_prefill_rejects_bad_arguments():
+    c, bnd, r = book(128)
+    _, cache, table, sl = build_paged_case([20, 30], 8, 2, seed=35)
+    q = torch.randn(50, 8, 128).to(torch.bfloat16)
+    cu = torch.tensor([0, 20, 50], dtype=torch.int32)
+    dev = [t.to(DEV) for t in (q, cu, cache, table, sl, c, r)]
+    with pytest.raises(ValueError):
+        K.paged_tq4_prefill(dev[0][:, :7].contiguous(), dev[1], 30, dev[2], dev[3], dev[4], dev[5], dev[5], dev[6], 2, 128, 16)
+    with pytest.raises(ValueError):
+        K.paged_tq4_prefill(dev[0], dev[1][:2], 30, dev[2], dev[3], dev[4], dev[5], dev[5], dev[6], 2, 128, 16)
+    with pytest.raises(ValueError):
+        K.paged_tq4_prefill(dev[0], dev[1], 30, dev[2], dev[3], dev[4], dev[5], dev[5], dev[6], 2, 128, 8)   # page size
+    with pytest.raises(RuntimeError):
+        K.paged_tq4_prefill(q, dev[1], 30, dev[2], dev[3], dev[4], dev[5], dev[5], dev[6], 2, 128, 16)      # CPU query
+
+
 # ---- fused compress-and-store into the paged cache -----------------------------------
 
 @pytest.mark.parametrize("h,d,dtype", [(8, 128, torch.bfloat16), (8, 128, torch.float16), (1, 64, torch.bfloat16),

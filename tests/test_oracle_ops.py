@@ -220,6 +220,63 @@ def test_paged_block_table_permutation_invariance(book):
     assert torch.equal(base, loop)
 
 
+# ---- paged prefill ----------------------------------------------------------
+
+def test_paged_prefill_one_query_is_paged_decode(book):
+    c, b, r = book
+    q, cache, bt, lens = _paged_case(book, [37, 16, 5])
+    cu = torch.arange(4, dtype=torch.int32)
+    got = O.paged_prefill(q, cu, cache, bt, lens, c, c, r, 2, 128, 16)
+    want = O.split_k_paged_decode(q, cache, bt, lens, c, c, r, 2, 128, 16)
+    assert torch.allclose(got.float(), want.float(), atol=1e-2)
+
+
+def test_paged_prefill_full_queries_is_fused_attention(book):
+    """Every token of a sequence is a query: the same numbers as the fused
+    operator on that sequence's packed K/V, causal from the top-left corner."""
+    c, b, r = book
+    hkv, hq, bs, L = 2, 4, 16, 40
+    q1, cache, bt, lens = _paged_case(book, [L], hq=hq, hkv=hkv, bs=bs, dtype=torch.float32)
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(L, hq, 128, generator=g)
+    cu = torch.tensor([0, L], dtype=torch.int32)
+    got = O.paged_prefill(q, cu, cache, bt, lens, c, c, r, hkv, 128, bs)
+    t = torch.arange(L)
+    rows = cache.view(-1, hkv * 136)[bt[0].long()[t // bs] * bs + t % bs]
+    kp = rows[:, :hkv * 64].reshape(L, hkv, 64).permute(1, 0, 2)[None]
+    kn = rows[:, hkv * 64:hkv * 68].contiguous().view(torch.float32).reshape(L, hkv, 1).permute(1, 0, 2)[None]
+    vp = rows[:, hkv * 68:hkv * 132].reshape(L, hkv, 64).permute(1, 0, 2)[None]
+    vn = rows[:, hkv * 132:].contiguous().view(torch.float32).reshape(L, hkv, 1).permute(1, 0, 2)[None]
+    want = O.fused_tq_attention(q.permute(1, 0, 2)[None], kp, kn, vp, vn, c, c, r, is_causal=True)
+    assert torch.allclose(got, want[0].permute(1, 0, 2), atol=2e-5)
+
+
+def test_paged_prefill_chunk_mask_is_bottom_right(book):
+    """A chunked prefill: 7 new tokens on a context of 45.  Checked against
+    SDPA with the mask written out by hand, and against the full prefill of
+    the same sequence, whose last 7 rows it must reproduce."""
+    c, b, r = book
+    hkv, hq, bs, L, n = 2, 4, 16, 45, 7
+    _, cache, bt, lens = _paged_case(book, [L], hq=hq, hkv=hkv, bs=bs, dtype=torch.float32)
+    g = torch.Generator().manual_seed(12)
+    q_all = torch.randn(L, hq, 128, generator=g)
+    full = O.paged_prefill(q_all, torch.tensor([0, L], dtype=torch.int32), cache, bt, lens, c, c, r, hkv, 128, bs)
+    part = O.paged_prefill(q_all[L - n:], torch.tensor([0, n], dtype=torch.int32), cache, bt, lens, c, c, r,
+                           hkv, 128, bs)
+    assert torch.allclose(part, full[L - n:], atol=1e-6)
+    k, v = O.gather_sequence(cache, bt[0], L, c, c, hkv, 128, bs)
+    mask = torch.zeros(n, L, dtype=torch.bool)
+    for j in range(n):
+        mask[j, : L - n + j + 1] = True
+    q_rot = (q_all[L - n:] @ r.T).permute(1, 0, 2)
+    want = F.scaled_dot_product_attention(q_rot, k.repeat_interleave(2, 0), v.repeat_interleave(2, 0), attn_mask=mask)
+    assert torch.allclose(part, want.permute(1, 0, 2) @ r, atol=2e-5)
+    no_mask = O.paged_prefill(q_all[L - n:], torch.tensor([0, n], dtype=torch.int32), cache, bt, lens, c, c, r,
+                              hkv, 128, bs, causal=False)
+    assert not torch.allclose(no_mask[:-1], part[:-1], atol=1e-3)
+    assert torch.allclose(no_mask[-1], part[-1], atol=1e-6)     # the last query sees every key either way
+
+
 # ---- TurboQuantProd ---------------------------------------------------------
 
 def test_prod_signs_and_shapes():
