@@ -255,7 +255,15 @@ def main():
         vx = outlier_rows(pb * pn, H_KV, D, 1023, dev)
         kp3, kn3 = K.tq4_compress(kx, rot_d, bnd_d)
         vp3, vn3 = K.tq4_compress(vx, rot_d, bnd_d)
-        del kx, vx
+        # the same tokens in a paged cache behind a shuffled block table, for the paged prefill
+        pages3 = pb * pn // BS
+        cache3 = torch.zeros(pages3, BS, ROW_BYTES, dtype=torch.uint8, device=dev)
+        table3 = torch.randperm(pages3, generator=torch.Generator().manual_seed(1033)).to(torch.int32)
+        table3 = table3.reshape(pb, pn // BS).to(dev)
+        t3 = torch.arange(pn, device=dev)
+        slots3 = torch.cat([table3[b_i].long()[t3 // BS] * BS + t3 % BS for b_i in range(pb)])
+        K.tq4_compress_and_store(kx, vx, rot_d, bnd_d, cache3, slots3)
+        del kx, vx, slots3, t3
 
         def to_bhnd(t):                                            # (B*N, H, X) -> (B, H, N, X)
             return t.reshape(pb, pn, H_KV, -1).permute(0, 2, 1, 3).contiguous()
@@ -272,7 +280,24 @@ def main():
             "prefill_pct_fp16_mfma_peak": 100.0 * p_flops / (p_ms * 1e-3) / 2.5e15,
             "prefill_tokens_per_s": pb * pn / (p_ms * 1e-3),
         })
-        del q3, kp3, kn3, vp3, vn3
+        q3v = q3.permute(0, 2, 1, 3).reshape(pb * pn, H_Q, D).contiguous()      # (tokens, heads, D)
+        cu3 = torch.arange(pb + 1, dtype=torch.int32, device=dev) * pn
+        lens3 = torch.full((pb,), pn, dtype=torch.int32, device=dev)
+        out3 = torch.empty_like(q3v)
+
+        def paged_prefill_step(i):
+            K.paged_tq4_prefill(q3v, cu3, pn, cache3, table3, lens3, cent_d, cent_d, rot_d, H_KV, D, BS,
+                                sm_scale=scale, causal=True, out=out3)
+
+        for i in range(2):
+            paged_prefill_step(i)
+        pp_ms = time_events(paged_prefill_step, 5)
+        extra.update({
+            "paged_prefill_ms": pp_ms,
+            "paged_prefill_tflops": p_flops / (pp_ms * 1e-3) / 1e12,
+            "paged_prefill_pct_fp16_mfma_peak": 100.0 * p_flops / (pp_ms * 1e-3) / 2.5e15,
+        })
+        del q3, q3v, out3, cache3, kp3, kn3, vp3, vn3
         torch.cuda.empty_cache()
 
         # ---- long-context decode over TurboQuantProd key / TQ4 value pages (configs[4]) ----------

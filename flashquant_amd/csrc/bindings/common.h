@@ -50,4 +50,3 @@ void* current_stream(const at::Tensor& like);
 void bind_kernels(pybind11::module_& m);
 void bind_codebook(pybind11::module_& m);
 void bind_quantizer(pybind11::module_& m);
-void bind_packing(pybind11::module_& m);

@@ -10,4 +10,6 @@ PYBIND11_MODULE(_C, m) {
     m.doc() = "TurboQuant KV-cache kernels for MI355X (gfx950)";
     m.attr("abi_version") = fq_abi_version();
     bind_kernels(m);
+    bind_codebook(m);
+    bind_quantizer(m);
 }

@@ -50,6 +50,52 @@ const char* fq_status_string(int status);
 const char* fq_last_hip_error(void);
 
 /*
+ * Lloyd-Max codebook of a rotated unit vector's coordinates: N(0, 1/dim) truncated
+ * to +-3.5 sigma, 2^bits levels.  Host code, no GPU work.  Follows the solver the
+ * reference's Python layer defines the kernel inputs with
+ * (_gaussian_centroids_boundaries, src/flashquant/core/codebook.py:58-140), not
+ * the numerically different csrc/core/codebook.cpp:64-121.
+ *   centroids   (2^bits,) float32 out, host memory
+ *   boundaries  (2^bits - 1,) float32 out, host memory: midpoints of the centroids
+ * bits in 1..8.
+ */
+int fq_lloyd_max_gaussian(int dim, int bits, float* centroids, float* boundaries);
+
+/*
+ * TurboQuantMSE.quantize / dequantize for any bit width up to 4
+ * (src/flashquant/core/quantizer.py:125-195; C++ twin csrc/core/quantizer.cpp:24-72),
+ * float32 arithmetic on the GPU.
+ *
+ * fq_mse_quantize:    n = ||x||, y = (x / (n + 1e-10)) R^T, idx = #{boundaries < y}
+ *   x            (M, D) fp16 / bf16 / float32 rows, contiguous
+ *   rotation     (D, D) float32, 16-byte aligned; rotation_col_major != 0 when the
+ *                buffer holds the transpose (layout as in fq_split_k_paged_decode)
+ *   boundaries   (num_boundaries,) float32 ascending, 1 <= num_boundaries <= 15
+ *   indices      (M, D) int64 out;  norms (M,) float32 out
+ * fq_mse_dequantize:  out = (centroids[idx] R) n
+ *   indices      (M, D) int64, clamped to [0, num_centroids - 1]
+ *   out          (M, D) float32, original space
+ * fq_mse_residual:    residual = x - (centroids[idx] R) n,  residual_norms = ||residual||
+ *                     (the first half of TurboQuantProd.quantize, quantizer.py:287-295)
+ * fq_project_rows:    out = x M^T in float32, or sign(x M^T) with 0 -> +1 when
+ *                     signs_only != 0 (the sketch of TurboQuantProd, quantizer.py:297-304
+ *                     and 357-359); matrix (D, D) float32
+ * D in {64, 128, 256}.  M == 0 is a no-op.
+ */
+int fq_mse_quantize(const void* x, int x_dtype, const float* rotation, int rotation_col_major,
+                    const float* boundaries, int num_boundaries, int64_t* indices, float* norms,
+                    int64_t M, int D, void* stream);
+int fq_mse_dequantize(const int64_t* indices, const float* norms, const float* rotation,
+                      int rotation_col_major, const float* centroids, int num_centroids, float* out,
+                      int64_t M, int D, void* stream);
+int fq_mse_residual(const void* x, int x_dtype, const int64_t* indices, const float* norms,
+                    const float* rotation, int rotation_col_major, const float* centroids,
+                    int num_centroids, float* residual, float* residual_norms, int64_t M, int D,
+                    void* stream);
+int fq_project_rows(const void* x, int x_dtype, const float* matrix, int matrix_col_major, int signs_only,
+                    float* out, int64_t M, int D, void* stream);
+
+/*
  * TQ4 compress.  Takes the role of tq4_compress_cuda
  * (csrc/cuda/compress.cuh:38-48); operator defined by compress_reference
  * (src/flashquant/kernels/cpu_reference.py:22-61).

@@ -610,3 +610,111 @@ def test_nibble_pack_rejects_bad_input():
     with pytest.raises(ValueError):
         K.nibble_pack(torch.tensor([-1, 3], dtype=torch.int32, device=DEV))
     assert K.nibble_pack(torch.zeros(0, 8, dtype=torch.uint8, device=DEV)).shape == (0, 4)
+
+
+# ---- quantizer classes: TurboQuantMSE / TurboQuantProd at any bit width ----------------------
+
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mse_quantizer_matches_oracle(dim, bits, dtype):
+    from flashquant_amd import core
+    qz = core.TurboQuantMSE(dim, bits, seed=42)
+    c, b = O.lloyd_max_gaussian(dim, bits)
+    r = O.haar_orthogonal(dim, 42)
+    x = outlier_rows(37, 5, dim, 90 + bits).to(dtype)              # 185 rows: a ragged last tile
+    want_idx, want_n = O.mse_quantize(x, r, b)
+    idx, n = qz.quantize(x.to(DEV))
+    assert idx.dtype == torch.int64 and idx.shape == x.shape and n.shape == (37, 5, 1)
+    mism = (idx.cpu() != want_idx).float().mean().item()
+    assert mism <= 1e-4, f"index mismatch rate {mism}"
+    assert torch.allclose(n.cpu(), want_n, rtol=1e-6, atol=0)
+    assert int(idx.max()) < (1 << bits) and int(idx.min()) >= 0
+    rec = qz.dequantize(idx, n)
+    want_rec = O.mse_dequantize(idx.cpu(), n.cpu(), r, c)
+    assert rec.dtype == torch.float32
+    scale = want_rec.abs().max().item()
+    assert (rec.cpu() - want_rec).abs().max().item() <= 1e-5 * scale
+
+
+def test_config0_round_trip_on_the_gpu():
+    """The reference's CPU-runnable case (4096 tokens, 8 heads, float32, seed 1000):
+    relative MSE of the 4-bit round trip through the quantizer class."""
+    from flashquant_amd import core
+    qz = core.TurboQuantMSE(128, 4, seed=42)
+    x = outlier_rows(4096, 8, 128, 1000)
+    idx, n = qz.quantize(x.to(DEV))
+    rec = qz.dequantize(idx, n).cpu()
+    rel = ((x - rec) ** 2).sum().item() / (x ** 2).sum().item()
+    c, b, r = book(128)
+    oi, on = O.mse_quantize(x, r, b)
+    want = O.mse_dequantize(oi, on, r, c)
+    rel_want = ((x - want) ** 2).sum().item() / (x ** 2).sum().item()
+    assert abs(rel - rel_want) <= 1e-5 and 0.0085 <= rel <= 0.0105
+    assert (idx.cpu() != oi).float().mean().item() <= 1e-4
+
+
+@pytest.mark.parametrize("dim,bits", [(128, 4), (64, 3), (256, 4)])
+def test_prod_quantizer_matches_oracle(dim, bits):
+    from flashquant_amd import core
+    qz = core.TurboQuantProd(dim, bits, seed=42)
+    c, b = O.lloyd_max_gaussian(dim, bits - 1)
+    r, s = O.haar_orthogonal(dim, 42), O.qjl_matrix(dim, 42)
+    x = outlier_rows(50, 3, dim, 120 + dim)
+    wi, wn, ws, wg = O.prod_quantize(x, r, b, c, s)
+    idx, n, signs, gam = qz.quantize(x.to(DEV))
+    assert signs.dtype == torch.float32 and signs.shape == x.shape and gam.shape == (50, 3, 1)
+    assert (idx.cpu() != wi).float().mean().item() <= 1e-4
+    same_rows = (idx.cpu() == wi).all(dim=-1)                       # rows whose indices agree share the residual
+    assert (signs.cpu()[same_rows] != ws[same_rows]).float().mean().item() <= 1e-3
+    assert set(signs.unique().tolist()) <= {-1.0, 1.0}
+    assert torch.allclose(gam.cpu()[same_rows], wg[same_rows], rtol=1e-4)
+    q = torch.randn(50, 3, dim, generator=torch.Generator().manual_seed(5))
+    est = qz.estimate_inner_product(q.to(DEV), idx, n, signs, gam).cpu()
+    want = O.prod_inner_product(q, idx.cpu(), n.cpu(), signs.cpu(), gam.cpu(), r, c, s)
+    assert est.shape == (50, 3, 1)
+    assert (est - want).abs().max().item() <= 1e-4 * max(1.0, want.abs().max().item())
+
+
+def test_prod_estimator_bias_bound_on_the_gpu():
+    """The property the reference tests for the estimator (tests/test_quantizer_prod.py:32-99):
+    averaged over many keys the relative bias of the estimate of <q, k> is below 0.05, and the
+    sketch term moves the MSE-only product towards the true one.  (With the sketch divided by
+    sqrt(m) and the sum by m, as the reference has them, the correction is 1 / sqrt(m) of
+    <q, residual>: it narrows the bias, it does not remove it.)"""
+    from flashquant_amd import core
+    qz = core.TurboQuantProd(128, 4, seed=42)
+    g = torch.Generator().manual_seed(77)
+    k = torch.randn(20000, 128, generator=g)
+    q = k * 0.5 + torch.randn(20000, 128, generator=g) * 0.5         # correlated with the key
+    idx, n, signs, gam = qz.quantize(k.to(DEV))
+    est = qz.estimate_inner_product(q.to(DEV), idx, n, signs, gam).cpu().squeeze(-1)
+    true = (q * k).sum(-1)
+    mse_only = (q * qz.dequantize(idx, n, signs, gam).cpu()).sum(-1)
+    bias, bias_mse = (est - true).mean().item(), (mse_only - true).mean().item()
+    assert abs(bias) / true.abs().mean().item() < 0.05
+    assert abs(bias) < abs(bias_mse)
+    expected_gain = -bias_mse / math.sqrt(128)                       # the 1 / sqrt(m) share of <q, residual>
+    assert abs((bias - bias_mse) - expected_gain) < 0.1 * abs(expected_gain) + 0.02
+
+
+def test_compressors_shapes_and_scores():
+    from flashquant_amd import core
+    kc, vc = core.KeyCompressor(128, 4), core.ValueCompressor(128, 4)
+    g = torch.Generator().manual_seed(9)
+    keys = torch.randn(2, 4, 33, 128, generator=g).to(torch.float16).to(DEV)
+    vals = torch.randn(2, 4, 33, 128, generator=g).to(torch.float16).to(DEV)
+    qry = torch.randn(2, 4, 5, 128, generator=g).to(torch.float16).to(DEV)
+    ck, cv = kc.compress(keys), vc.compress(vals)
+    assert ck.indices.shape == keys.shape and ck.residual_norms.shape == (2, 4, 33, 1) and ck.original_dtype == torch.float16
+    rec = vc.decompress(cv)
+    assert rec.dtype == torch.float16
+    rel = ((rec.float() - vals.float()) ** 2).sum().item() / (vals.float() ** 2).sum().item()
+    assert rel < 0.012
+    scores = kc.asymmetric_attention_scores(qry, ck)
+    assert scores.shape == (2, 4, 5, 33) and scores.dtype == torch.float16
+    r, s = O.haar_orthogonal(128, 42), O.qjl_matrix(128, 42)
+    c3, _ = O.lloyd_max_gaussian(128, 3)
+    want = O.prod_inner_product(qry.cpu()[:, :, :, None, :], ck.indices.cpu()[:, :, None], ck.norms.cpu()[:, :, None],
+                                ck.qjl_signs.cpu()[:, :, None], ck.residual_norms.cpu()[:, :, None], r, c3, s)
+    assert (scores.cpu().float() - want.squeeze(-1)).abs().max().item() <= 2e-2

@@ -55,3 +55,60 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".cpp", ".hip", ".hpp", ".h")):
                 text = open(os.path.join(dirpath, f), errors="ignore").read()
                 assert "tq_oracle" not in text and "import oracle" not in text and "from oracle" not in text, f
+
+
+# ---- host set-up of the product against the oracle ---------------------------------------
+
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("bits", [1, 2, 3, 4])
+def test_codebook_solver_equals_the_oracle(dim, bits):
+    from flashquant_amd import core
+    from oracle import tq_oracle as O
+    c, b = core.solve_lloyd_max(dim, bits)
+    oc, ob = O.lloyd_max_gaussian(dim, bits)
+    assert c.dtype == torch.float32 and c.shape == (1 << bits,) and b.shape == ((1 << bits) - 1,)
+    assert torch.equal(c, oc)
+    # the middle boundary is the mean of two opposite levels: zero up to the last bit of the doubles
+    assert (b - ob).abs().max().item() < 1e-12
+
+
+def test_codebook_registry_and_value_quantizer():
+    from flashquant_amd import core
+    reg = core.CodebookRegistry()
+    cb = reg.get(128, 4)
+    assert reg.get(128, 4) is cb and cb.bits == 4 and cb.dim == 128
+    x = torch.tensor([-1.0, 0.0, float(cb.boundaries[3]), 1.0])
+    idx = cb.quantize(x)
+    assert idx.tolist() == [0, int((cb.boundaries < 0).sum()), 3, 15]          # a tie goes to the lower cell
+    assert torch.equal(cb.dequantize(idx), cb.centroids[idx])
+    reg.clear()
+    assert reg.get(128, 4) is not cb
+
+
+@pytest.mark.parametrize("dim,seed", [(128, 42), (128, 43), (64, 42), (256, 5)])
+def test_rotation_and_sketch_equal_the_oracle(dim, seed):
+    from flashquant_amd import core
+    from oracle import tq_oracle as O
+    r = core.haar_orthogonal(dim, seed)
+    assert torch.equal(r, O.haar_orthogonal(dim, seed))
+    assert torch.equal(core.qjl_matrix(dim, seed), O.qjl_matrix(dim, seed))
+    e, o = core.split_rotation(r)
+    oe, oo = O.split_rotation(r)
+    assert torch.equal(e, oe) and torch.equal(o, oo) and e.is_contiguous()
+
+
+def test_quantizer_classes_hold_reference_state_and_refuse_cpu_tensors():
+    from flashquant_amd import core
+    from oracle import tq_oracle as O
+    q = core.TurboQuantProd(128, 4, seed=42)
+    assert q.mse_quantizer.bits == 3 and q.qjl_dim == 128
+    assert torch.equal(q.mse_quantizer.rotation, O.haar_orthogonal(128, 42))
+    assert torch.equal(q.qjl_matrix, O.qjl_matrix(128, 42))
+    with pytest.raises(ValueError):
+        core.TurboQuantProd(128, 1)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        q.quantize(torch.zeros(2, 128))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        core.TurboQuantMSE(64, 2).dequantize(torch.zeros(2, 64, dtype=torch.long), torch.ones(2, 1))
+    assert core.KeyCompressor(128).quantizer.mse_quantizer.bits == 3
+    assert torch.equal(core.ValueCompressor(128).quantizer.rotation, O.haar_orthogonal(128, 43))
