@@ -419,6 +419,53 @@ at::Tensor nibble_unpack(const at::Tensor& packed) {
     return out;
 }
 
+at::Tensor pack_2bit(const at::Tensor& indices) {
+    fqbind::require_gpu(indices, "indices");
+    require(indices.dim() >= 1 && indices.size(-1) % 4 == 0, "Last dim must be divisible by 4");
+    int bytes = 0;
+    switch (indices.scalar_type()) {
+        case at::kByte: bytes = 1; break;
+        case at::kInt: bytes = 4; break;
+        case at::kLong: bytes = 8; break;
+        default: throw std::invalid_argument("pack_2bit: indices must be uint8, int32 or int64");
+    }
+    c10::DeviceGuard guard(indices.device());
+    const at::Tensor ic = indices.contiguous();
+    auto shape = ic.sizes().vec();
+    shape.back() /= 4;
+    at::Tensor packed = at::empty(shape, ic.options().dtype(at::kByte));
+    at::Tensor bad = at::zeros({1}, ic.options().dtype(at::kInt));
+    const int st = fq_pack_2bit(ic.data_ptr(), bytes, packed.data_ptr<uint8_t>(), packed.numel(), bad.data_ptr<int>(),
+                                fqbind::current_stream(indices));
+    fqbind::raise_on_error(st, "pack_2bit");
+    if (bad.item<int>() != 0) throw std::invalid_argument("Indices out of range for 2-bit packing. Expected [0, 3]");
+    return packed;
+}
+
+at::Tensor unpack_2bit(const at::Tensor& packed) {
+    fqbind::require_gpu(packed, "packed");
+    require(packed.scalar_type() == at::kByte, "unpack_2bit: packed must be uint8");
+    c10::DeviceGuard guard(packed.device());
+    const at::Tensor pc = packed.contiguous();
+    auto shape = pc.sizes().vec();
+    shape.back() *= 4;
+    at::Tensor out = at::empty(shape, pc.options().dtype(at::kLong));
+    const int st = fq_unpack_2bit(pc.data_ptr<uint8_t>(), out.data_ptr<int64_t>(), pc.numel(),
+                                  fqbind::current_stream(packed));
+    fqbind::raise_on_error(st, "unpack_2bit");
+    return out;
+}
+
+// validate_indices (csrc/core/packing.cpp:8-19): raises when an index lies outside [0, 2^bits).
+void validate_indices(const at::Tensor& indices, int64_t bits) {
+    fqbind::require_gpu(indices, "indices");
+    require(bits >= 1 && bits <= 8, "bits must lie in 1..8");
+    if (indices.numel() == 0) return;
+    const int64_t lo = indices.min().item<int64_t>(), hi = indices.max().item<int64_t>();
+    if (lo < 0 || hi >= (int64_t(1) << bits))
+        throw std::invalid_argument("Indices out of range for " + std::to_string(bits) + "-bit packing");
+}
+
 at::Tensor rotate_query(const at::Tensor& q, const at::Tensor& rotation) {
     fqbind::require_gpu(q, "q");
     require(q.dim() == 3 && (q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16),
@@ -548,6 +595,14 @@ void bind_kernels(py::module_& m) {
           "Split-K paged decode over TurboQuantProd key / TQ4 value pages");
     m.def("nibble_pack", &nibble_pack, py::arg("indices"), "Pack pairs of 4-bit indices (..., D) into bytes (..., D/2)");
     m.def("nibble_unpack", &nibble_unpack, py::arg("packed"), "Unpack bytes (..., D/2) into int64 indices (..., D)");
+    {
+        py::module_ pk = m.def_submodule("packing", "Index packing on the GPU");
+        pk.def("nibble_pack", &nibble_pack, py::arg("indices"));
+        pk.def("nibble_unpack", &nibble_unpack, py::arg("packed"));
+        pk.def("pack_2bit", &pack_2bit, py::arg("indices"), "Four 2-bit indices per byte, the first in the top bits");
+        pk.def("unpack_2bit", &unpack_2bit, py::arg("packed"), "Inverse of pack_2bit, int64");
+        pk.def("validate_indices", &validate_indices, py::arg("indices"), py::arg("bits"));
+    }
     m.def("rotate_query", &rotate_query, py::arg("q"), py::arg("rotation"),
           "q_rot = (q @ rotation.T) rounded to q's dtype.");
     m.def("paged_tq4_decode_partials", &paged_tq4_decode_partials, py::arg("q_rot"), py::arg("kv_cache"),

@@ -20,3 +20,19 @@ def nibble_unpack(packed: torch.Tensor) -> torch.Tensor:
     """Unpack ``(..., D // 2)`` uint8 into int64 indices ``(..., D)``."""
     require_gpu(packed, "packed")
     return native().nibble_unpack(packed)
+
+
+def pack_2bit(indices: torch.Tensor) -> torch.Tensor:
+    """Pack four 2-bit indices per byte, the first in the top bits
+    (csrc/core/packing.cpp:48-64).  Raises ValueError for a last dimension not
+    divisible by 4 or an index outside [0, 3]."""
+    require_gpu(indices, "indices")
+    if indices.shape[-1] % 4 != 0:
+        raise ValueError(f"Last dim must be divisible by 4, got {indices.shape[-1]}")
+    return native().packing.pack_2bit(indices)
+
+
+def unpack_2bit(packed: torch.Tensor) -> torch.Tensor:
+    """Inverse of ``pack_2bit``: int64 indices ``(..., 4 * bytes)``."""
+    require_gpu(packed, "packed")
+    return native().packing.unpack_2bit(packed)

@@ -298,6 +298,16 @@ int fq_nibble_pack(const void* indices, int index_bytes, uint8_t* packed, int64_
 int fq_nibble_unpack(const uint8_t* packed, int64_t* indices, int64_t n_packed, void* stream);
 
 /*
+ * 2-bit packing, four indices per byte with the first in the top bits
+ * (pack_2bit / unpack_2bit, csrc/core/packing.cpp:48-79).  Arguments as for the
+ * nibble pair; n_packed = number of bytes; indices outside [0, 3] are counted in
+ * *bad_count.
+ */
+int fq_pack_2bit(const void* indices, int index_bytes, uint8_t* packed, int64_t n_packed,
+                 int* bad_count, void* stream);
+int fq_unpack_2bit(const uint8_t* packed, int64_t* indices, int64_t n_packed, void* stream);
+
+/*
  * TurboQuantProd keys (3-bit Lloyd-Max index + 1-bit sign sketch of the residual) with
  * TQ4 values, as pages.  The reference defines the quantizer
  * (TurboQuantProd.quantize / estimate_inner_product, src/flashquant/core/quantizer.py:285-370;

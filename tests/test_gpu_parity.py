@@ -612,6 +612,29 @@ def test_nibble_pack_rejects_bad_input():
     assert K.nibble_pack(torch.zeros(0, 8, dtype=torch.uint8, device=DEV)).shape == (0, 4)
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int32, torch.int64])
+def test_2bit_pack_unpack_bit_exact(dtype):
+    g = torch.Generator().manual_seed(6)
+    idx = torch.randint(0, 4, (5, 3, 132), generator=g).to(dtype)
+    packed = K.pack_2bit(idx.to(DEV))
+    assert packed.dtype == torch.uint8 and packed.shape == (5, 3, 33)
+    assert torch.equal(packed.cpu(), O.pack_2bit(idx))
+    back = K.unpack_2bit(packed)
+    assert back.dtype == torch.int64 and torch.equal(back.cpu(), idx.long())
+    allb = torch.arange(256, dtype=torch.uint8)
+    assert torch.equal(K.unpack_2bit(allb.to(DEV)).cpu(), O.unpack_2bit(allb))
+    assert K.pack_2bit(torch.tensor([3, 0, 2, 1], dtype=dtype, device=DEV)).cpu().tolist() == [0b11001001]
+    with pytest.raises(ValueError):
+        K.pack_2bit(torch.zeros(2, 6, dtype=dtype, device=DEV))
+    with pytest.raises(ValueError):
+        K.pack_2bit(torch.tensor([0, 1, 2, 4], dtype=dtype, device=DEV))
+    import flashquant_amd
+    pk = flashquant_amd.load_native().packing
+    pk.validate_indices(idx.to(DEV), 2)
+    with pytest.raises(ValueError):
+        pk.validate_indices(torch.tensor([0, 4], device=DEV), 2)
+
+
 # ---- quantizer classes: TurboQuantMSE / TurboQuantProd at any bit width ----------------------
 
 @pytest.mark.parametrize("dim", [64, 128, 256])
