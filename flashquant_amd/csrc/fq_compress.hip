@@ -48,6 +48,17 @@ struct CompressCfg {
 
 constexpr float kLoScale = 1.0f / 4096.0f;
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// top 16 bits of a float as bf16 (truncation: the next term of the split takes up the rest)
+__device__ __forceinline__ __bf16 bf16_trunc(float f) {
+    return __builtin_bit_cast(__bf16, uint16_t(float_to_bits(f) >> 16));
+}
+__device__ __forceinline__ float bf16_value(__bf16 h) {
+    return bits_to_float(uint32_t(__builtin_bit_cast(uint16_t, h)) << 16);
+}
+
 // lane exchange inside the VALU (DPP): CTRL 0xB1 / 0x4E swap lanes inside quads, 0x141 / 0x140
 // mirror the 8- / 16-lane rows
 template <int CTRL>
@@ -154,7 +165,10 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
         return pd.cache + slot * (int64_t(pd.H) * (D + 8)) + (is_v ? int64_t(pd.H) * (D / 2 + 4) : 0);
     };
     __shared__ __attribute__((aligned(16))) uint8_t xs[2][C::TT * C::XS_STRIDE];
-    __shared__ __attribute__((aligned(16))) uint8_t outs[C::TT * C::OUT_STRIDE];
+    // bf16 rows of head_dim 128 run a software pipeline (see below) with two packed-row buffers
+    constexpr bool kPipe = DT == FQ_BF16 && D == 128;
+    constexpr int kOutBytes = C::TT * C::OUT_STRIDE;
+    __shared__ __attribute__((aligned(16))) uint8_t outs[(kPipe ? 2 : 1) * kOutBytes];
     __shared__ float inv_s[2][C::TT];
     __shared__ BucketTable table;
 
@@ -167,7 +181,13 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     const int tb0 = wave / C::CB;
 
     // ---- the rotation rows of this wave, split into two fp16 terms ----------
-    half8 a_hi[C::NK], a_lo[C::NK];
+    // fp16 rows: R = hi + lo / 4096 in fp16.  bf16 rows go to the bf16 MFMA as they are, against
+    // R = t0 + t1 + t2 in bf16 (3 x 8 bits: the float32 value exactly); bf16 terms keep the
+    // float32 exponent range, so the three products share one accumulator.
+    // (head_dim 256 would need 192 registers for the three terms: it keeps the fp16 route)
+    constexpr bool kBf16 = DT == FQ_BF16 && D <= 128;
+    half8 a_hi[kBf16 ? 1 : C::NK], a_lo[kBf16 ? 1 : C::NK];
+    bf16x8 a_t[kBf16 ? 3 : 1][kBf16 ? C::NK : 1];
     {
         const int j = 32 * cb + mfma_row_to_coord(n32);
         const float* src = (j & 1) ? rot_T_odd : rot_T_even;
@@ -178,9 +198,17 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             for (int e = 0; e < 8; ++e) {
                 const int k = 16 * ks + 8 * kg + e;
                 const float r = src[k * (D / 2) + col];
-                const _Float16 hi = _Float16(r);
-                a_hi[ks][e] = hi;
-                a_lo[ks][e] = _Float16((r - float(hi)) * 4096.0f);
+                if constexpr (kBf16) {
+                    const __bf16 t0 = bf16_trunc(r);
+                    const float r1 = r - bf16_value(t0);
+                    const __bf16 t1 = bf16_trunc(r1);
+                    const __bf16 t2 = bf16_trunc(r1 - bf16_value(t1));
+                    a_t[0][ks][e] = t0; a_t[1][ks][e] = t1; a_t[2][ks][e] = t2;
+                } else {
+                    const _Float16 hi = _Float16(r);
+                    a_hi[ks][e] = hi;
+                    a_lo[ks][e] = _Float16((r - float(hi)) * 4096.0f);
+                }
             }
         }
     }
@@ -213,41 +241,62 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             const int64_t row = tile * C::TT + r;
             float e[8];
             const uint32_t w[4] = {pre[p].x, pre[p].y, pre[p].z, pre[p].w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                e[2 * i] = load_elem<DT>(uint16_t(w[i] & 0xffffu));
-                e[2 * i + 1] = load_elem<DT>(uint16_t(w[i] >> 16));
-            }
             float ss = 0.0f, mx = 0.0f;
+            if constexpr (kBf16) {
+                // sum of squares straight from the packed pairs (v_dot2_f32_bf16)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                ss = __builtin_fmaf(e[i], e[i], ss);
-                mx = __builtin_fmaxf(mx, __builtin_fabsf(e[i]));
+                for (int i = 0; i < 4; ++i) {
+                    const bf16x2 v = __builtin_bit_cast(bf16x2, w[i]);
+                    ss = __builtin_amdgcn_fdot2_f32_bf16(v, v, ss, false);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    e[2 * i] = load_elem<DT>(uint16_t(w[i] & 0xffffu));
+                    e[2 * i + 1] = load_elem<DT>(uint16_t(w[i] >> 16));
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    ss = __builtin_fmaf(e[i], e[i], ss);
+                    mx = __builtin_fmaxf(mx, __builtin_fabsf(e[i]));
+                }
             }
             // all-reduce over the CPR lanes of the row, in the VALU (quad swaps, mirrors, row swap)
-            ss += dpp_f32<0xB1>(ss); mx = __builtin_fmaxf(mx, dpp_f32<0xB1>(mx));      // lane ^ 1
-            ss += dpp_f32<0x4E>(ss); mx = __builtin_fmaxf(mx, dpp_f32<0x4E>(mx));      // lane ^ 2
-            ss += dpp_f32<0x141>(ss); mx = __builtin_fmaxf(mx, dpp_f32<0x141>(mx));    // mirror of 8: the other quad
-            if (C::CPR >= 16) { ss += dpp_f32<0x140>(ss); mx = __builtin_fmaxf(mx, dpp_f32<0x140>(mx)); }   // mirror of 16
+            ss += dpp_f32<0xB1>(ss);      // lane ^ 1
+            ss += dpp_f32<0x4E>(ss);      // lane ^ 2
+            ss += dpp_f32<0x141>(ss);     // mirror of 8: the other quad
+            if (C::CPR >= 16) ss += dpp_f32<0x140>(ss);   // mirror of 16
             if (C::CPR >= 32) {
                 const auto sw = __builtin_amdgcn_permlane16_swap(float_to_bits(ss), float_to_bits(ss), false, false);
                 ss = bits_to_float(sw[0]) + bits_to_float(sw[1]);
-                const auto mw = __builtin_amdgcn_permlane16_swap(float_to_bits(mx), float_to_bits(mx), false, false);
-                mx = __builtin_fmaxf(bits_to_float(mw[0]), bits_to_float(mw[1]));
             }
-            const float nrm = __builtin_sqrtf(ss);
-            int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
-            if (ex < -126 || ex > 126) ex = 0;   // zero / subnormal / non-finite rows: no scaling
-            const float down = bits_to_float(uint32_t(127 - ex) << 23);
-            const float up = bits_to_float(uint32_t(127 + ex) << 23);
-            uint4v h;
-            h.x = pack_h2(_Float16(e[0] * down), _Float16(e[1] * down));
-            h.y = pack_h2(_Float16(e[2] * down), _Float16(e[3] * down));
-            h.z = pack_h2(_Float16(e[4] * down), _Float16(e[5] * down));
-            h.w = pack_h2(_Float16(e[6] * down), _Float16(e[7] * down));
+            // v_sqrt_f32 (1 ulp), with a sum of squares in the subnormal range scaled into the normal one
+            const bool tiny = ss < 0x1p-96f;
+            const float nrm_s = __builtin_amdgcn_sqrtf(tiny ? ss * 0x1p64f : ss);
+            const float nrm = tiny ? nrm_s * 0x1p-32f : nrm_s;
+            float up = 1.0f;
+            uint4v h = pre[p];
+            if constexpr (!kBf16) {
+                mx = __builtin_fmaxf(mx, dpp_f32<0xB1>(mx));
+                mx = __builtin_fmaxf(mx, dpp_f32<0x4E>(mx));
+                mx = __builtin_fmaxf(mx, dpp_f32<0x141>(mx));
+                if (C::CPR >= 16) mx = __builtin_fmaxf(mx, dpp_f32<0x140>(mx));
+                if (C::CPR >= 32) {
+                    const auto mw = __builtin_amdgcn_permlane16_swap(float_to_bits(mx), float_to_bits(mx), false, false);
+                    mx = __builtin_fmaxf(bits_to_float(mw[0]), bits_to_float(mw[1]));
+                }
+                int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+                if (ex < -126 || ex > 126) ex = 0;   // zero / subnormal / non-finite rows: no scaling
+                const float down = bits_to_float(uint32_t(127 - ex) << 23);
+                up = bits_to_float(uint32_t(127 + ex) << 23);
+                h.x = pack_h2(_Float16(e[0] * down), _Float16(e[1] * down));
+                h.y = pack_h2(_Float16(e[2] * down), _Float16(e[3] * down));
+                h.z = pack_h2(_Float16(e[4] * down), _Float16(e[5] * down));
+                h.w = pack_h2(_Float16(e[6] * down), _Float16(e[7] * down));
+            }
             *reinterpret_cast<uint4v*>(&xs[buf][r * C::XS_STRIDE + chunk * 16]) = h;
             if (chunk == 0) {
-                inv_s[buf][r] = up / (nrm + 1e-10f);
+                inv_s[buf][r] = up * __builtin_amdgcn_rcpf(nrm + 1e-10f);
                 if (row < M) {
                     if (PAGED) {
                         int head, is_v;
@@ -261,56 +310,15 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
         }
     };
 
-    int64_t tile = blockIdx.x;
-    if (tile < num_tiles) {
-        issue_loads(tile);
-        stage(tile, 0);
-    }
-    __syncthreads();
-
-    for (int it = 0; tile < num_tiles; tile += gridDim.x, ++it) {
-        const int cur = it & 1;
-        const int64_t next = tile + gridDim.x;
-        if (next < num_tiles) issue_loads(next);
-
-        // ---- rotate + bucketize + pack ---------------------------------------
-        for (int tb = tb0; tb < C::TB; tb += C::TB_STEP) {
-            float16v acc_hi = {}, acc_lo = {};
-            const uint8_t* brow = &xs[cur][(32 * tb + n32) * C::XS_STRIDE + kg * 16];
-#pragma unroll
-            for (int ks = 0; ks < C::NK; ++ks) {
-                const half8 b = *reinterpret_cast<const half8*>(brow + ks * 32);
-                acc_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[ks], b, acc_hi, 0, 0, 0);
-                acc_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_lo[ks], b, acc_lo, 0, 0, 0);
-            }
-            const float inv = inv_s[cur][32 * tb + n32];
-            uint32_t idx[16];
-            if (!slow) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    idx[i] = bucket_fast(table, __builtin_fmaf(acc_lo[i], kLoScale, acc_hi[i]) * inv, inv_w, offset);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    idx[i] = bucket_slow(table, __builtin_fmaf(acc_lo[i], kLoScale, acc_hi[i]) * inv);
-            }
-            uint2v o;
-            o.x = (idx[0] << 4 | idx[1]) | (idx[2] << 4 | idx[3]) << 8 | (idx[4] << 4 | idx[5]) << 16 |
-                  (idx[6] << 4 | idx[7]) << 24;
-            o.y = (idx[8] << 4 | idx[9]) | (idx[10] << 4 | idx[11]) << 8 | (idx[12] << 4 | idx[13]) << 16 |
-                  (idx[14] << 4 | idx[15]) << 24;
-            *reinterpret_cast<uint2v*>(&outs[(32 * tb + n32) * C::OUT_STRIDE + 16 * cb + 8 * kg]) = o;
-        }
-        __syncthreads();
-
-        // ---- packed rows of this tile: LDS -> global, 16 bytes per lane ------
+    // packed rows of a tile: LDS -> global, 16 bytes per lane
+    auto store_tile = [&](int64_t tile, const uint8_t* ob) {
         constexpr int OC = D / 32;   // 16-byte chunks per packed row
         for (int c = tid; c < C::TT * OC; c += C::THREADS) {
             const int r = c / OC, q = c % OC;
             const int64_t row = tile * C::TT + r;
             if (row < M) {
-                const uint2v lo = *reinterpret_cast<const uint2v*>(&outs[r * C::OUT_STRIDE + q * 16]);
-                const uint2v hi = *reinterpret_cast<const uint2v*>(&outs[r * C::OUT_STRIDE + q * 16 + 8]);
+                const uint2v lo = *reinterpret_cast<const uint2v*>(&ob[r * C::OUT_STRIDE + q * 16]);
+                const uint2v hi = *reinterpret_cast<const uint2v*>(&ob[r * C::OUT_STRIDE + q * 16 + 8]);
                 uint4v v = {lo.x, lo.y, hi.x, hi.y};
                 if (PAGED) {
                     int head, is_v;
@@ -329,6 +337,145 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                 }
             }
         }
+    };
+
+    int64_t tile = blockIdx.x;
+
+    // ---- software pipeline (bf16, head_dim 128) ------------------------------------------------
+    // The unit of work is a block of 32 rows.  The matrix instructions of block u + 1 are issued
+    // between the lookups and compares that bucketize block u, so that a wavefront keeps both the
+    // matrix pipe and the vector ALU busy instead of alternating between them (two wavefronts
+    // share a SIMD; phases that alternate fall into step and leave one of the two units idle).
+    // Per tile: [MFMA (tile, 1) | finish (tile, 0)], stage tile + 1, barrier,
+    //           [MFMA (tile + 1, 0) | finish (tile, 1)], barrier, store tile.
+    if constexpr (kPipe) {
+        if (!slow && tile < num_tiles) {
+            const int64_t G = gridDim.x;
+            auto pipe = [&](int mbuf, int mtb, float16v& acc_out, int fbuf, int ftb,
+                            const float16v& acc_in, uint8_t* ob) {
+                const uint8_t* brow = &xs[mbuf][(32 * mtb + n32) * C::XS_STRIDE + kg * 16];
+                const float inv = inv_s[fbuf][32 * ftb + n32];
+                float16v acc = {};
+                uint32_t idx[16];
+                uint2v cell[16];
+                float yv[16];
+                // element e: address and lookup at step e, compare at step e + 4
+#pragma unroll
+                for (int st = 0; st < 24; ++st) {
+                    {
+                        const int ks = st / 3, t = 2 - st % 3;
+                        const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc, 0, 0, 0);
+                    }
+                    if (st < 16) {
+                        yv[st] = acc_in[st] * inv;
+                        const float pos = __builtin_fmaf(yv[st], inv_w, offset);
+                        const int c = int(__builtin_amdgcn_fmed3f(pos, 0.0f, 255.0f));
+                        cell[st] = table.cell[c];
+                    }
+                    if (st >= 4 && st < 20) {
+                        const int e = st - 4;
+                        idx[e] = cell[e].y + (bits_to_float(cell[e].x) < yv[e] ? 1u : 0u);
+                    }
+                }
+                uint2v o;
+                o.x = (idx[0] << 4 | idx[1]) | (idx[2] << 4 | idx[3]) << 8 | (idx[4] << 4 | idx[5]) << 16 |
+                      (idx[6] << 4 | idx[7]) << 24;
+                o.y = (idx[8] << 4 | idx[9]) | (idx[10] << 4 | idx[11]) << 8 | (idx[12] << 4 | idx[13]) << 16 |
+                      (idx[14] << 4 | idx[15]) << 24;
+                *reinterpret_cast<uint2v*>(&ob[(32 * ftb + n32) * C::OUT_STRIDE + 16 * cb + 8 * kg]) = o;
+                acc_out = acc;
+            };
+
+            issue_loads(tile);
+            stage(tile, 0);
+            if (tile + G < num_tiles) issue_loads(tile + G);
+            __syncthreads();
+            float16v acc_a = {}, acc_b = {};
+            {   // block (tile, 0): nothing to overlap with yet
+                const uint8_t* brow = &xs[0][n32 * C::XS_STRIDE + kg * 16];
+#pragma unroll
+                for (int st = 0; st < 24; ++st) {
+                    const int ks = st / 3, t = 2 - st % 3;
+                    const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
+                    acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc_a, 0, 0, 0);
+                }
+            }
+            for (int it = 0; tile < num_tiles; tile += G, ++it) {
+                const int cur = it & 1;
+                const int64_t next = tile + G;
+                const bool has_next = next < num_tiles;
+                uint8_t* ob = outs + cur * kOutBytes;
+                pipe(cur, 1, acc_b, cur, 0, acc_a, ob);
+                if (has_next) {
+                    stage(next, cur ^ 1);
+                    if (next + G < num_tiles) issue_loads(next + G);
+                }
+                __syncthreads();                      // tile + 1 is staged
+                // past the last tile the matrix instructions run on stale rows and their result is dropped
+                pipe(cur ^ 1, 0, acc_a, cur, 1, acc_b, ob);
+                __syncthreads();                      // the packed rows of this tile are complete
+                store_tile(tile, ob);
+            }
+            return;
+        }
+    }
+
+    if (tile < num_tiles) {
+        issue_loads(tile);
+        stage(tile, 0);
+    }
+    __syncthreads();
+
+    for (int it = 0; tile < num_tiles; tile += gridDim.x, ++it) {
+        const int cur = it & 1;
+        const int64_t next = tile + gridDim.x;
+        if (next < num_tiles) issue_loads(next);
+
+        // ---- rotate + bucketize + pack ---------------------------------------
+        for (int tb = tb0; tb < C::TB; tb += C::TB_STEP) {
+            float16v acc_hi = {}, acc_lo = {};
+            const uint8_t* brow = &xs[cur][(32 * tb + n32) * C::XS_STRIDE + kg * 16];
+            if constexpr (kBf16) {
+                // the small terms first, so that they are not rounded away against the large one
+#pragma unroll
+                for (int t = 2; t >= 0; --t)
+#pragma unroll
+                    for (int ks = 0; ks < C::NK; ++ks) {
+                        const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
+                        acc_hi = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc_hi, 0, 0, 0);
+                    }
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < C::NK; ++ks) {
+                    const half8 b = *reinterpret_cast<const half8*>(brow + ks * 32);
+                    acc_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[ks], b, acc_hi, 0, 0, 0);
+                    acc_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_lo[ks], b, acc_lo, 0, 0, 0);
+                }
+            }
+            const float inv = inv_s[cur][32 * tb + n32];
+            float yv[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                yv[i] = (kBf16 ? acc_hi[i] : __builtin_fmaf(acc_lo[i], kLoScale, acc_hi[i])) * inv;
+            uint32_t idx[16];
+            if (!slow) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) idx[i] = bucket_fast(table, yv[i], inv_w, offset);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) idx[i] = bucket_slow(table, yv[i]);
+            }
+            uint2v o;
+            o.x = (idx[0] << 4 | idx[1]) | (idx[2] << 4 | idx[3]) << 8 | (idx[4] << 4 | idx[5]) << 16 |
+                  (idx[6] << 4 | idx[7]) << 24;
+            o.y = (idx[8] << 4 | idx[9]) | (idx[10] << 4 | idx[11]) << 8 | (idx[12] << 4 | idx[13]) << 16 |
+                  (idx[14] << 4 | idx[15]) << 24;
+            *reinterpret_cast<uint2v*>(&outs[(32 * tb + n32) * C::OUT_STRIDE + 16 * cb + 8 * kg]) = o;
+        }
+        __syncthreads();
+
+        store_tile(tile, outs);
         if (next < num_tiles) stage(next, cur ^ 1);
         __syncthreads();
     }
