@@ -58,6 +58,7 @@ namespace fq_host {
 // FQ_DECODE_DIRECT=1 in the environment routes every shape to the direct kernel
 // (both kernels are kept tested).
 bool force_direct_decode();
+int device_cu_count();
 }
 
 namespace fq {
@@ -82,6 +83,8 @@ struct DecodeParams {
     int num_splits;
     int two_tables;             // centroids_v differs from centroids_k
     float scale_log2e;          // sm_scale * log2(e)
+    int balance_slots;          // staged kernel: > 0 lets the workgroups size the token chunks from the actual
+                                // sequence lengths, for this many workgroups running at a time (num_seqs <= 64)
 };
 
 
@@ -620,8 +623,12 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     const int g = lane >> 4;
     const int hd = n % GP;
     const int cls = n / GP;               // column class: GP=4 -> 2*block + half, GP=8 -> block, GP=16 -> 0
-    const int split = blockIdx.x;
-    const int seq = blockIdx.y;
+    // Sequence fastest: workgroups are handed to the CUs in the order of their linear index, and
+    // a workgroup that finds its split empty and leaves at once does not make room for a later one
+    // on another CU.  With the split index slow, the empty splits (beyond a sequence's length)
+    // come last instead of alternating with the live ones.
+    int seq = blockIdx.x;
+    int split = blockIdx.y;
 
     // Every load that depends on nothing is asked for first, so that the memory
     // latencies of the prologue overlap instead of adding up: the centroids, the
@@ -634,13 +641,87 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     const uint8_t* lut_v = lut_k;
     const uint32_t lane_off = 4u * (lane & 31);
     const uint32_t lane_off_v = 128u + lane_off;
-    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + int64_t(seq) * p.H_Q * 128;
     float rot_b[4][8];
     float rot_s[4][8];
-    uint4v q_pre[2][4];
     if (p.rotation != nullptr) {
         load_rotation_any<128>(p.rotation, p.rot_col_major != 0, true, 16 * h, n, g, rot_b);
         if constexpr (PROD) load_rotation_any<128>(p.sketch, false, true, 16 * h, n, g, rot_s);
+    }
+
+    const int NS = p.num_splits;
+    const bool rowwide = p.max_blocks <= 64 * PVR;
+    // every sequence is cut into the same token chunks (those of the longest possible context):
+    // the work of a workgroup does not depend on its sequence's length, short sequences just
+    // leave their last splits empty
+    int chunk = (((p.max_blocks * BS + NS - 1) / NS) + 63) & ~63;
+    int L_known = -1;
+    if (p.balance_slots > 0) {
+        // Ragged batches of long contexts (at most 64 sequences, one lane each).  With the chunk
+        // of the longest possible context the live workgroups are all the same size and their
+        // count is whatever the lengths add up to, e.g. 2.1 rounds over the chip, which costs 3.
+        // Every workgroup evaluates the same 64 candidate chunk sizes (one per lane) on the
+        // actual lengths, cost = rounds x (chunk + a prologue's worth of tokens), and takes the
+        // cheapest: same inputs, same arithmetic, same answer in every workgroup.  Larger chunks
+        // only: the split count bounds the chunk from below.
+        const int cap = rowwide ? chunk * NS : 64 * PVR * BS;       // page ids of a split: 64 * PVR lanes
+        const int step = ((chunk >> 4) + 63) & ~63;
+        int cand = chunk + lane * step;
+        cand = cand < cap ? cand : cap;
+        cand = cand > chunk ? cand : chunk;
+        const float rc = __builtin_amdgcn_rcpf(float(cand));
+        const int nseq = int(gridDim.x);
+        int l_mine = lane < nseq ? p.seq_lens[lane] : 0;
+        l_mine = l_mine < 0 ? 0 : (l_mine > p.max_blocks * BS ? p.max_blocks * BS : l_mine);
+        float groups = 0.0f;
+        for (int sq = 0; sq < nseq; ++sq)
+            groups += __builtin_ceilf(float(__builtin_amdgcn_readlane(l_mine, sq)) * rc - 0.0009765625f);
+        const float rounds = __builtin_ceilf(groups * __builtin_amdgcn_rcpf(float(p.balance_slots)) - 0.0009765625f);
+        const float cost = (rounds < 1.0f ? 1.0f : rounds) * float(cand + 96);
+        uint32_t key = (uint32_t(cost) << 6) | uint32_t(lane);
+#pragma unroll
+        for (int mask = 1; mask < 64; mask <<= 1) {
+            const uint32_t other = uint32_t(__shfl_xor(int(key), mask, kWave));
+            key = other < key ? other : key;
+        }
+        const int best = chunk + int(key & 63u) * step;
+        chunk = best < cap ? best : (cap > chunk ? cap : chunk);
+
+        // The live (sequence, split) pairs first, in sequence order, then the empty ones: the w-th
+        // workgroup of the grid takes the w-th pair of that list.  Live workgroups are all of one
+        // size and now consecutive, so they spread evenly over the XCDs and CUs whatever the lengths.
+        auto scan = [&](int v) {
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int t = __shfl_up(v, d, kWave);
+                v += lane >= d ? t : 0;
+            }
+            return v;
+        };
+        int n_mine = lane < nseq ? (l_mine + chunk - 1) / chunk : 0;
+        n_mine = n_mine < NS ? n_mine : NS;
+        const int live_incl = scan(n_mine);
+        const int total_live = __builtin_amdgcn_readlane(live_incl, 63);
+        const int w = int(blockIdx.x) + int(gridDim.x) * int(blockIdx.y);
+        if (w < total_live) {
+            const int s_idx = __builtin_popcountll(__ballot(live_incl <= w));
+            seq = s_idx;
+            split = w - __builtin_amdgcn_readlane(live_incl - n_mine, s_idx);
+        } else {
+            const int e = w - total_live;
+            const int dead_mine = lane < nseq ? NS - n_mine : 0;
+            const int dead_incl = scan(dead_mine);
+            int s_idx = __builtin_popcountll(__ballot(dead_incl <= e));
+            s_idx = s_idx < nseq ? s_idx : nseq - 1;
+            seq = s_idx;
+            split = __builtin_amdgcn_readlane(n_mine, s_idx) + (e - __builtin_amdgcn_readlane(dead_incl - dead_mine, s_idx));
+            split = split < NS ? split : NS - 1;
+        }
+        L_known = __builtin_amdgcn_readlane(l_mine, seq);
+    }
+
+    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + int64_t(seq) * p.H_Q * 128;
+    uint4v q_pre[2][4];
+    if (p.rotation != nullptr) {
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
@@ -652,7 +733,6 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     // fetched now, before the sequence length is known, so that the two loads overlap;
     // otherwise the registers hold the pages of this split, which depend on the length.
     const int32_t* bt = p.block_table + int64_t(seq) * p.max_blocks;
-    const bool rowwide = p.max_blocks <= 64 * PVR;
     int pv[PVR];
     if (rowwide) {
 #pragma unroll
@@ -662,14 +742,9 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         }
     }
 
-    int L = p.seq_lens[seq];
+    int L = L_known >= 0 ? L_known : p.seq_lens[seq];
     L = L < 0 ? 0 : L;
     L = L > p.max_blocks * BS ? p.max_blocks * BS : L;
-    const int NS = p.num_splits;
-    // every sequence is cut into the same token chunks (those of the longest possible context):
-    // the work of a workgroup does not depend on its sequence's length, short sequences just
-    // leave their last splits empty
-    const int chunk = (((p.max_blocks * BS + NS - 1) / NS) + 63) & ~63;
     const int begin = split * chunk;
     const int end = L < begin + chunk ? L : begin + chunk;
     const int hq_lane = h * p.G + n;
@@ -1294,6 +1369,14 @@ int launch_with_lds(K kernel, const DecodeParams& p, dim3 grid, dim3 block, size
     return fq_host::check_launch();
 }
 
+// Workgroups that run at a time (one per CU) when the staged kernel should size its chunks from
+// the actual sequence lengths, 0 when the fixed chunks already fill the chip in one round or the
+// batch is too large for one lane per sequence.
+inline int staged_balance_slots(int num_seqs, int num_splits) {
+    const int cus = fq_host::device_cu_count();
+    return (num_seqs <= 64 && int64_t(num_seqs) * num_splits > cus) ? cus : 0;
+}
+
 // The staged kernel covers 8 KV heads of dimension 128.
 inline bool staged_applies(int D, int H_KV) {
     return D == 128 && H_KV == 8 && !fq_host::force_direct_decode();
@@ -1303,7 +1386,7 @@ template <bool PROD, typename K>
 int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream) {
     // dynamic part only; the 64 KB table is static
     const size_t lds = 2 * size_t(StagedCfg<PROD>::TILE_BYTES);
-    return launch_with_lds(kernel, p, dim3(p.num_splits, S, 1), dim3(512), lds, stream);
+    return launch_with_lds(kernel, p, dim3(S, p.num_splits, 1), dim3(512), lds, stream);
 }
 
 // Staged kernel for every page size and group size; PROD selects the TurboQuantProd page format.
@@ -1336,8 +1419,13 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
     const bool wide = chunk / BS > 64;   // begin is a multiple of 64 tokens, hence page aligned
 
     // four page-id registers also when they can hold the whole block-table row
-    if (staged_applies(D, p.H_KV))
-        return launch_staged_any<DT, false>(p, S, BS, wide || (p.max_blocks > 64 && p.max_blocks <= 256), stream);
+    if (staged_applies(D, p.H_KV)) {
+        DecodeParams ps = p;
+        ps.balance_slots = staged_balance_slots(S, p.num_splits);
+        // a chosen chunk may span up to 256 pages: four page-id registers
+        return launch_staged_any<DT, false>(ps, S, BS, wide || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256),
+                                            stream);
+    }
 
     const int waves = p.H_KV < 8 ? p.H_KV : 8;
     const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
@@ -1447,9 +1535,10 @@ extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_siz
     // KV head and split) ...
     const int64_t target_waves = int64_t(fq_host::device_cu_count()) * 8;
     const int64_t one_round = (target_waves + int64_t(num_seqs) * H_KV - 1) / (int64_t(num_seqs) * H_KV);
-    // ... and up to four rounds when the contexts are long enough for splits of 1024 tokens: the
-    // lengths of the sequences are not known here, and ragged batches leave many splits empty
-    int64_t ns = 4 * one_round < max_ctx / 1024 ? 4 * one_round : max_ctx / 1024;
+    // ... and twice that when the contexts are long enough for splits of 1024 tokens: the lengths
+    // of the sequences are not known here, a ragged batch leaves many splits empty, and the
+    // kernel can merge splits (it sizes its chunks from the actual lengths) but not divide them
+    int64_t ns = 2 * one_round < max_ctx / 1024 ? 2 * one_round : max_ctx / 1024;
     if (ns < one_round) ns = one_round;
     if (ns > tiles) ns = tiles;
     if (ns > 256) ns = 256;
@@ -1514,6 +1603,7 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
     p.num_blocks = int(num_blocks); p.num_splits = num_splits;
     p.two_tables = centroids_k != centroids_v ? 1 : 0;
     p.scale_log2e = sm_scale * kLog2e;
+    p.balance_slots = 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define FQ_DECODE_D(DD)                                                                 \
     case DD:                                                                            \
@@ -1638,10 +1728,12 @@ extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, cons
     p.num_blocks = int(num_blocks); p.num_splits = num_splits;
     p.two_tables = 1;
     p.scale_log2e = sm_scale * kLog2e;
+    p.balance_slots = staged_balance_slots(num_seqs, num_splits);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t max_ctx = int64_t(max_blocks_per_seq) * block_size;
     const int64_t chunk = (((max_ctx + num_splits - 1) / num_splits) + 63) & ~int64_t(63);
-    const bool wide = chunk / block_size > 64 || (max_blocks_per_seq > 64 && max_blocks_per_seq <= 256);
+    const bool wide = chunk / block_size > 64 || p.balance_slots > 0 ||
+                      (max_blocks_per_seq > 64 && max_blocks_per_seq <= 256);
     const int st = dtype == FQ_F16 ? launch_staged_any<FQ_F16, true>(p, num_seqs, block_size, wide, s)
                                    : launch_staged_any<FQ_BF16, true>(p, num_seqs, block_size, wide, s);
     if (st != FQ_OK) return st;

@@ -166,6 +166,20 @@ def test_paged_decode_llama8b_heads(num_splits):
     _decode_case([37, 0, 16, 300, 64, 65, 1, 129], hq=32, hkv=8, num_splits=num_splits)
 
 
+@pytest.mark.parametrize("num_splits", [40, 64])
+def test_paged_decode_ragged_batch_with_more_splits_than_cus(num_splits):
+    """More (sequence, split) workgroups than CUs: the kernel sizes its chunks from the actual
+    lengths and renumbers the workgroups, live ones first.  The result must not depend on it."""
+    lens = [1500, 0, 37, 6000, 64, 2049, 1, 3333]
+    _decode_case(lens, hq=32, hkv=8, num_splits=num_splits)
+    _decode_case(lens, hq=64, hkv=8, num_splits=num_splits, bs=32, dtype=torch.float16)
+
+
+def test_paged_decode_64_sequences_rebalanced():
+    lens = [(37 * i) % 700 for i in range(64)]            # 64 sequences: one lane each, some empty
+    _decode_case(lens, hq=8, hkv=8, num_splits=8)
+
+
 @pytest.mark.parametrize("hq,hkv", [(8, 8), (4, 2), (8, 2), (12, 4), (64, 8), (16, 1), (5, 1)])
 def test_paged_decode_group_sizes(hq, hkv):
     _decode_case([70, 5, 200], hq=hq, hkv=hkv, num_splits=2)
@@ -538,6 +552,10 @@ def _check_prod_decode(lens, hq, bs=16, num_splits=0, dtype=torch.bfloat16, seed
 @pytest.mark.parametrize("num_splits", [0, 1, 5])
 def test_prod_paged_decode_group_sizes_and_splits(hq, num_splits):
     _check_prod_decode([300, 1, 77, 0, 129], hq, num_splits=num_splits)
+
+
+def test_prod_paged_decode_ragged_batch_with_more_splits_than_cus():
+    _check_prod_decode([900, 0, 37, 2100, 64, 1025, 1, 1500], 64, num_splits=48)
 
 
 @pytest.mark.parametrize("bs", [8, 16, 32])
