@@ -78,4 +78,5 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 inline bool supported_dim(int d) { return d == 64 || d == 128 || d == 256; }
 // Raises the dynamic-LDS limit of a kernel function once per (function, device); later calls are a lookup.
 bool lds_limit_raised(const void* kernel, size_t bytes);
+int device_cu_count();
 }  // namespace fq_host

@@ -63,6 +63,7 @@ struct PrefillParams {
     const int32_t* block_table;    // (S, max_blocks)
     const uint8_t* cache;          // (num_blocks, block_size, H_KV * 136)
     int max_blocks, num_blocks, bs_log2;
+    int round_slots;               // workgroups running at a time (one per CU)
 };
 
 __device__ __forceinline__ uint32_t scale_pair(uint32_t pair, half2v n2) {
@@ -90,7 +91,15 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m32 = lane & 31, hf = lane >> 5;     // 32x32 MFMA: column (query row) and lane half
     const int n16 = lane & 15, g4 = lane >> 4;     // 16x16 MFMA of the rotations
-    const int b = blockIdx.z, hkv = blockIdx.y;
+    // Workgroups reach the CUs in the order of their linear index, round after round, and under a
+    // causal mask their durations grow with the query position.  Position fastest, (batch, head)
+    // slow, and the position order reversed in every other round over the chip: whichever way the
+    // rounds land on the CUs, each CU sees long and short workgroups alternate.
+    const int lin = int(blockIdx.x) + int(gridDim.x) * (int(blockIdx.y) + int(gridDim.y) * int(blockIdx.z));
+    const int pair = lin / int(gridDim.x);
+    const int b = pair / int(gridDim.y), hkv = pair % int(gridDim.y);
+    const int x_in_pair = lin % int(gridDim.x);
+    const bool flip = ((lin / p.round_slots) & 1) != 0;
 
     // ---- this sequence -----------------------------------------------------------------------
     int NQ = p.N_Q, NKV = p.N_KV, qoff = 0;
@@ -110,7 +119,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     // ---- units --------------------------------------------------------------------------
     const int nblk = (NQ + 31) >> 5;
     const int units = nblk * p.G;
-    const int wg = int(gridDim.x) - 1 - int(blockIdx.x);   // late (long) query blocks start first
+    const int wg = flip ? x_in_pair : int(gridDim.x) - 1 - x_in_pair;
     if (PAGED && 8 * wg >= units) return;                  // the grid is sized for the longest sequence
     const int unit_raw = 8 * wg + w;
     const bool unit_live = unit_raw < units;
@@ -473,6 +482,7 @@ extern "C" int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, con
     hipStream_t s = static_cast<hipStream_t>(stream);
     p.cu_seqlens_q = nullptr; p.seq_lens = nullptr; p.block_table = nullptr; p.cache = nullptr;
     p.max_blocks = 0; p.num_blocks = 0; p.bs_log2 = 0;
+    p.round_slots = fq_host::device_cu_count();
     if (dtype == FQ_F16) {
         auto kern = fused_tq_attention_kernel<FQ_F16, false>;
         if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
@@ -520,6 +530,7 @@ extern "C" int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, 
     p.cu_seqlens_q = cu_seqlens_q; p.seq_lens = seq_lens; p.block_table = block_table; p.cache = kv_cache;
     p.max_blocks = max_blocks_per_seq; p.num_blocks = int(num_blocks);
     p.bs_log2 = block_size == 8 ? 3 : (block_size == 16 ? 4 : 5);
+    p.round_slots = fq_host::device_cu_count();
 
     const int64_t units = int64_t((max_q_len + 31) / 32) * p.G;
     const int64_t wgs = (units + 7) / 8;
