@@ -230,7 +230,8 @@ def main():
             "compress_mtok_per_s": rows_tok / (c_ms * 1e-3) / 1e6,
             "compress_gbps": nrows * 324 / (c_ms * 1e-3) / 1e9,
             "compress_pct_hbm_peak": 100.0 * nrows * 324 / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-            "compress_tflops_fp16_mfma": nrows * 2 * 2 * D * D / (c_ms * 1e-3) / 1e12,
+            # bf16 rows against the 3-term bf16 split of the rotation: 3 x 2 D^2 flops per row on the MFMA
+            "compress_tflops_bf16_mfma": nrows * 3 * 2 * D * D / (c_ms * 1e-3) / 1e12,
         })
         del x
         torch.cuda.empty_cache()
@@ -381,7 +382,7 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a plain copy
             # (profiles/paged_decode_hbm_traffic_pmc.txt); a measured constant, not read live
-            "traffic": 150.5e6,
+            "traffic": 148.0e6,
             "kernel": "paged_decode_staged_kernel<4,4,bf16,4,false>",
         },
         "cpu_baseline": cpu,
