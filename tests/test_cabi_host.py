@@ -120,3 +120,69 @@ def test_rotation_fusion_rule(lib):
     assert lib.fq_paged_decode_fuses_rotation(128, 8, 0) == 1    # distinct K and V codebooks share the table
     assert lib.fq_paged_decode_fuses_rotation(64, 8, 1) == 0
     assert lib.fq_paged_decode_fuses_rotation(128, 4, 1) == 0
+
+
+def test_codebook_solver_runs_on_the_host_and_matches_the_committed_levels(lib):
+    import json
+    f = lib.fq_lloyd_max_gaussian
+    f.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
+    golden = json.load(open(os.path.join(ROOT, "tests", "golden", "codebook_d128.json")))
+    for bits in (2, 3, 4):
+        c = (ctypes.c_float * (1 << bits))()
+        b = (ctypes.c_float * ((1 << bits) - 1))()
+        assert f(128, bits, c, b) == FQ_OK
+        want = golden[str(bits)]
+        assert max(abs(x - y) for x, y in zip(c, want["centroids"])) < 1e-8
+        assert max(abs(x - y) for x, y in zip(b, want["boundaries"])) < 1e-8
+        assert all(c[i] < c[i + 1] for i in range(len(c) - 1))
+    c = (ctypes.c_float * 2)()
+    b = (ctypes.c_float * 1)()
+    assert f(128, 0, c, b) == FQ_SHAPE and f(0, 2, c, b) == FQ_SHAPE and f(128, 9, c, b) == FQ_SHAPE
+    assert f(128, 1, None, b) == FQ_NULL
+
+
+def test_quantizer_and_packing_argument_errors(lib):
+    q = lib.fq_mse_quantize
+    q.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+                  ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    assert q(_p(), 2, _p(), 0, _p(), 15, _p(), _p(), 0, 128, _p()) == FQ_OK
+    assert q(_p(), 2, _p(), 0, _p(), 16, _p(), _p(), 4, 128, _p()) == FQ_SHAPE       # at most 15 boundaries
+    assert q(_p(), 2, _p(), 0, _p(), 15, _p(), _p(), 4, 96, _p()) == FQ_DIM
+    assert q(_p(), 5, _p(), 0, _p(), 15, _p(), _p(), 4, 128, _p()) == FQ_DTYPE
+    assert q(_p(), 2, _p(), 0, _p(), 15, _p(), _p(), 4, 128, _p()) == FQ_NULL
+    assert q(_p(16), 2, _p(8), 0, _p(16), 15, _p(16), _p(16), 4, 128, _p()) == FQ_ALIGN
+    d = lib.fq_mse_dequantize
+    d.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+                  ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    assert d(_p(), _p(), _p(), 0, _p(), 1, _p(), 4, 128, _p()) == FQ_SHAPE            # fewer than 2 levels
+    assert d(_p(), _p(), _p(), 0, _p(), 16, _p(), 4, 128, _p()) == FQ_NULL
+    pr = lib.fq_project_rows
+    pr.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                   ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    assert pr(_p(), 2, _p(), 0, 1, _p(), -1, 128, _p()) == FQ_SHAPE
+    assert pr(_p(), 2, _p(), 0, 1, _p(), 3, 32, _p()) == FQ_DIM
+    p2 = lib.fq_pack_2bit
+    p2.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    assert p2(_p(), 8, _p(), 0, _p(), _p()) == FQ_OK
+    assert p2(_p(), 2, _p(), 4, _p(), _p()) == FQ_DTYPE                               # 16-bit indices
+    assert p2(_p(), 8, _p(), 4, _p(), _p()) == FQ_NULL
+
+
+def test_paged_prefill_argument_errors(lib):
+    f = lib.fq_paged_tq4_prefill
+    f.argtypes = ([ctypes.c_void_p] * 8 + [ctypes.c_int, ctypes.c_void_p] + [ctypes.c_int] * 7 +
+                  [ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
+
+    def call(S=2, maxq=64, HQ=32, HKV=8, D=128, BS=16, MB=4, NB=64, dtype=1, ptr=0, out=None):
+        o = ptr if out is None else out
+        return f(_p(ptr), _p(ptr), _p(ptr), _p(ptr), _p(ptr), _p(ptr), _p(ptr), _p(ptr), 0, _p(o), S, maxq, HQ, HKV, D,
+                 BS, MB, NB, 0.088, 1, dtype, _p())
+
+    assert call(S=0) == FQ_OK and call(maxq=0) == FQ_OK
+    assert call(HQ=30) == FQ_SHAPE
+    assert call(D=64) == FQ_DIM and call(D=100) == FQ_DIM
+    assert call(BS=12) == FQ_BLOCK
+    assert call(dtype=2) == FQ_DTYPE
+    assert call(S=-1) == FQ_SHAPE and call(MB=0) == FQ_SHAPE
+    assert call() == FQ_NULL
+    assert call(ptr=4096 + 8) == FQ_ALIGN
