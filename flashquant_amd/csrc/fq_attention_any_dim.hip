@@ -1,0 +1,323 @@
+// Fused TQ4 attention for head_dim 64 and 256 (and, as a cross-check, 128): the operator of
+// fq_fused_attention.hip (src/flashquant/kernels/cpu_reference.py:154-227, the launcher
+// csrc/cuda/fused_tq_attention.cu:468-511 takes all three dimensions) in a plainer shape.
+// The tuned kernel's tile layout is written for 128 coordinates; this one trades speed for
+// generality and shares nothing with it but the arithmetic rules:
+//   q_rot = (q @ R^T) rounded to the query dtype (float32 MFMA)
+//   K, V  = fp16(centroid[idx] * norm), scores and P.V on v_mfma_f32_16x16x32_f16
+//   out   = (softmax(...) V) @ R, rounded once (contiguous operands) or rounded before and after
+//           the rotation (paged operands, as the serving path rounds)
+//
+// A workgroup of 4 wavefronts owns 64 query rows of one query head, 16 per wavefront.  Per
+// 32-token tile all threads dequantise K (row-major) and V (transposed) into LDS; a wavefront
+// then computes S = q K^T in the MFMA accumulator layout (lane = token column, registers = 4 query
+// rows), keeps the running maximum per row with row-wide DPP reductions, moves P through a
+// private LDS patch into the A-operand layout, and accumulates O (registers = the same 4 rows,
+// so the rescale needs no cross-lane traffic).
+#include <cstdlib>
+
+#include "fq_common.hpp"
+#include "fq_device.hpp"
+#include "fq_attention_any_dim.hpp"
+
+namespace fq {
+
+
+// maximum over the 16 lanes of a DPP row
+__device__ __forceinline__ float row16_max(float v) {
+    v = __builtin_fmaxf(v, dpp_mov<0x121>(v));
+    v = __builtin_fmaxf(v, dpp_mov<0x122>(v));
+    v = __builtin_fmaxf(v, dpp_mov<0x124>(v));
+    v = __builtin_fmaxf(v, dpp_mov<0x128>(v));
+    return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_mov<0x121>(v);
+    v += dpp_mov<0x122>(v);
+    v += dpp_mov<0x124>(v);
+    v += dpp_mov<0x128>(v);
+    return v;
+}
+
+template <int D>
+struct AnyDimCfg {
+    static constexpr int KSTRIDE = D + 8;                 // halves per K tile row (padded)
+    static constexpr int VSTRIDE = 32 + 8;                // halves per V^T tile row
+    static constexpr int K_BYTES = 32 * KSTRIDE * 2;
+    static constexpr int V_BYTES = D * VSTRIDE * 2;
+    static constexpr int P_BYTES = 4 * 16 * VSTRIDE * 2;  // one 16 x 32 patch per wavefront
+    static constexpr int Q_BYTES = 4 * 16 * KSTRIDE * 2;  // rotated query rows, fp16
+    static constexpr int LOOP_BYTES = K_BYTES + V_BYTES + P_BYTES + Q_BYTES;
+    static constexpr int O_BYTES = 4 * 16 * (D + 4) * 4;  // float32 rows for the rotation back
+    static constexpr int LDS_BYTES = LOOP_BYTES > O_BYTES ? LOOP_BYTES : O_BYTES;
+};
+
+template <int D, int DT, bool PAGED>
+__global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimParams p) {
+    using C = AnyDimCfg<D>;
+    constexpr int NJ = D / 32;          // k-steps of the score product
+    constexpr int NCB = D / 16;         // 16-coordinate output blocks
+    constexpr int CPT = D / 8;          // coordinates per thread in the dequantisation (8 threads per token)
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ _Float16 cent_k[16], cent_v[16];
+    _Float16* ks = reinterpret_cast<_Float16*>(smem);
+    _Float16* vt = reinterpret_cast<_Float16*>(smem + C::K_BYTES);
+    _Float16* ps = reinterpret_cast<_Float16*>(smem + C::K_BYTES + C::V_BYTES);
+    _Float16* qs = reinterpret_cast<_Float16*>(smem + C::K_BYTES + C::V_BYTES + C::P_BYTES);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = tid >> 6;
+    const int n16 = lane & 15, g4 = lane >> 4;
+    const int hq = blockIdx.y, b = blockIdx.z;
+    const int hkv = hq / p.G;
+
+    int NQ = p.N_Q, NKV = p.N_KV, qoff = 0;
+    int64_t q_row0 = (int64_t(b) * p.H_Q + hq) * p.N_Q;   // first row of this head, in rows of D
+    int q_stride = D;
+    if (PAGED) {
+        const int first = p.cu_seqlens_q[b];
+        NQ = p.cu_seqlens_q[b + 1] - first;
+        NKV = p.seq_lens[b];
+        NKV = NKV < 0 ? 0 : (NKV > (p.max_blocks << p.bs_log2) ? (p.max_blocks << p.bs_log2) : NKV);
+        qoff = NKV - NQ > 0 ? NKV - NQ : 0;
+        q_row0 = int64_t(first) * p.H_Q + hq;
+        q_stride = p.H_Q * D;
+    }
+    const int pos_wg = 64 * blockIdx.x;
+    if (pos_wg >= NQ) return;                         // uniform: the grid is sized for the longest sequence
+    const int pos0 = pos_wg + 16 * w;                 // first row of this wavefront
+
+    if (tid < 16) cent_k[tid] = _Float16(p.centroids_k[tid]);
+    else if (tid < 32) cent_v[tid - 16] = _Float16(p.centroids_v[tid - 16]);
+
+    // ---- rotate the 16 query rows of this wavefront, round to the query dtype, stage as fp16 ------
+    float up = 1.0f;
+    {
+        int pos = pos0 + n16;
+        pos = pos < NQ ? pos : NQ - 1;
+        const uint16_t* src = p.q + (q_row0 * D) + int64_t(pos) * q_stride;
+        float a[NJ][8];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int k = 0; k < 8; ++k) a[j][k] = load_elem<DT>(src[32 * j + 8 * g4 + k]);
+        float qr[NCB][4];
+        float mx = 0.0f;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            float rb[NJ][8];
+            load_rotation_any<D>(p.rotation, p.rot_col_major != 0, true, 16 * cb, n16, g4, rb);
+            const float4v acc = rotate_block<D>(a, rb);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                qr[cb][i] = load_elem<DT>(store_elem<DT>(acc[i]));
+                mx = __builtin_fmaxf(mx, __builtin_fabsf(qr[cb][i]));
+            }
+        }
+        // one power of two for the wavefront's 16 rows, so that the rounded values are exact in fp16
+        mx = wave_max(mx);
+        int ex = int((float_to_bits(mx) >> 23) & 0xffu) - 127;
+        if (ex < -100 || ex > 100) ex = 0;
+        const float down = bits_to_float(uint32_t(127 - ex) << 23);
+        up = bits_to_float(uint32_t(127 + ex) << 23);
+        _Float16* mine = qs + w * 16 * C::KSTRIDE;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mine[(4 * g4 + i) * C::KSTRIDE + 16 * cb + n16] = _Float16(qr[cb][i] * down);
+    }
+    __syncthreads();
+    half8 qa[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+        qa[j] = *reinterpret_cast<const half8*>(qs + (w * 16 + n16) * C::KSTRIDE + 32 * j + 8 * g4);
+    const float qscale = p.scale_log2e * up;
+
+    // ---- tiles --------------------------------------------------------------------------------------
+    const int all_tiles = (NKV + 31) >> 5;
+    int ntiles = all_tiles;
+    if (p.causal) {
+        int last_pos = pos_wg + 63 < NQ - 1 ? pos_wg + 63 : NQ - 1;
+        const int t = ((qoff + last_pos) >> 5) + 1;
+        ntiles = t < all_tiles ? t : all_tiles;
+    }
+    float4v O[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) O[cb] = float4v{0.f, 0.f, 0.f, 0.f};
+    float m_run[4], l_run[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { m_run[i] = -__builtin_inff(); l_run[i] = 0.0f; }
+
+    const int tok_d = tid >> 3, part = tid & 7;       // dequantisation: token of the tile, eighth of its row
+    const int64_t kv_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.N_KV;
+    _Float16* pw = ps + w * 16 * C::VSTRIDE;
+
+    for (int tile = 0; tile < ntiles; ++tile) {
+        const int t0 = tile * 32;
+        // ---- dequantise: thread = (token, D/8 coordinates) -----------------------------------------
+        {
+            int tok = t0 + tok_d;
+            const bool live = tok < NKV;
+            tok = live ? tok : (NKV > 0 ? NKV - 1 : 0);
+            const uint8_t *kp, *vp;
+            float nk, nv;
+            if (PAGED) {
+                const int H = p.H_KV;
+                int pg = p.block_table[int64_t(b) * p.max_blocks + (tok >> p.bs_log2)];
+                pg = pg < 0 ? 0 : (pg >= p.num_blocks ? p.num_blocks - 1 : pg);
+                const uint8_t* row = p.cache + ((int64_t(pg) << p.bs_log2) + (tok & ((1 << p.bs_log2) - 1))) * (int64_t(H) * (D + 8));
+                kp = row + hkv * (D / 2);
+                nk = *reinterpret_cast<const float*>(row + H * (D / 2) + 4 * hkv);
+                vp = row + H * (D / 2 + 4) + hkv * (D / 2);
+                nv = *reinterpret_cast<const float*>(row + H * (D + 4) + 4 * hkv);
+            } else {
+                kp = p.k_packed + (kv_row0 + tok) * (D / 2);
+                vp = p.v_packed + (kv_row0 + tok) * (D / 2);
+                nk = p.k_norms[kv_row0 + tok];
+                nv = p.v_norms[kv_row0 + tok];
+            }
+            if (!live) { nk = 0.0f; nv = 0.0f; }
+#pragma unroll
+            for (int c = 0; c < CPT / 8; ++c) {       // 4 bytes = 8 coordinates at a time
+                const int byte0 = part * (CPT / 2) + 4 * c;
+                const uint32_t kw = *reinterpret_cast<const uint32_t*>(kp + byte0);
+                const uint32_t vw = *reinterpret_cast<const uint32_t*>(vp + byte0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t kb = (kw >> (8 * e)) & 0xffu, vb = (vw >> (8 * e)) & 0xffu;
+                    const int d = 2 * (byte0 + e);
+                    // fp16(centroid) * norm, rounded to fp16: the same values as the tuned kernel's tiles
+                    ks[tok_d * C::KSTRIDE + d] = _Float16(float(cent_k[kb >> 4]) * nk);
+                    ks[tok_d * C::KSTRIDE + d + 1] = _Float16(float(cent_k[kb & 15]) * nk);
+                    vt[d * C::VSTRIDE + tok_d] = _Float16(float(cent_v[vb >> 4]) * nv);
+                    vt[(d + 1) * C::VSTRIDE + tok_d] = _Float16(float(cent_v[vb & 15]) * nv);
+                }
+            }
+        }
+        __syncthreads();
+
+        // ---- scores: two blocks of 16 tokens ----------------------------------------------------------
+        float4v s[2];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+            s[tb] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const half8 kb = *reinterpret_cast<const half8*>(ks + (16 * tb + n16) * C::KSTRIDE + 32 * j + 8 * g4);
+                s[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[j], kb, s[tb], 0, 0, 0);
+            }
+        }
+        // lane (n16, g4): rows 4 g4 + i, tokens t0 + n16 and t0 + 16 + n16
+        float pv[2][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int qpos = qoff + pos0 + 4 * g4 + i;
+            float sc[2];
+            float mx = -__builtin_inff();
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb) {
+                const int tok = t0 + 16 * tb + n16;
+                const bool ok = tok < NKV && (!p.causal || tok <= qpos);
+                sc[tb] = ok ? s[tb][i] * qscale : -__builtin_inff();
+                mx = __builtin_fmaxf(mx, sc[tb]);
+            }
+            mx = row16_max(mx);
+            const float m_new = __builtin_fmaxf(m_run[i], mx);
+            const float m_use = m_new == -__builtin_inff() ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[i] - m_use);
+            m_run[i] = m_new;
+            float rs = 0.0f;
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb) {
+                pv[tb][i] = __builtin_amdgcn_exp2f(sc[tb] - m_use);
+                rs += pv[tb][i];
+            }
+            l_run[i] = __builtin_fmaf(l_run[i], alpha, rs);     // per-lane partial; summed over the row at the end
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) O[cb][i] *= alpha;
+        }
+        // P (C layout) -> LDS patch -> A layout
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pw[(4 * g4 + i) * C::VSTRIDE + 16 * tb + n16] = _Float16(pv[tb][i]);
+        const half8 pa = *reinterpret_cast<const half8*>(pw + n16 * C::VSTRIDE + 8 * g4);
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            const half8 vb = *reinterpret_cast<const half8*>(vt + (16 * cb + n16) * C::VSTRIDE + 8 * g4);
+            O[cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, O[cb], 0, 0, 0);
+        }
+        __syncthreads();                               // the tiles are free again
+    }
+
+    // ---- normalise, rotate back, store ------------------------------------------------------------------
+    __syncthreads();                                   // the staging rows overlay the tiles and the query rows
+    float* os = reinterpret_cast<float*>(smem) + w * 16 * (D + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float l = row16_sum(l_run[i]);
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            float v = O[cb][i] * inv;
+            if (PAGED) v = load_elem<DT>(store_elem<DT>(v));
+            os[(4 * g4 + i) * (D + 4) + 16 * cb + n16] = v;
+        }
+    }
+    __syncthreads();
+    float a[NJ][8];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a[j][k] = os[n16 * (D + 4) + 32 * j + 8 * g4 + k];
+    uint16_t* obase = p.out + q_row0 * D;
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+        float rb[NJ][8];
+        load_rotation_any<D>(p.rotation, p.rot_col_major != 0, false, 16 * cb, n16, g4, rb);
+        const float4v acc = rotate_block<D>(a, rb);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int pos = pos0 + 4 * g4 + i;
+            if (pos < NQ) obase[int64_t(pos) * q_stride + 16 * cb + n16] = store_elem<DT>(acc[i]);
+        }
+    }
+}
+
+template <int D, bool PAGED>
+int launch_any_dim(const AnyDimParams& p, int max_q, int batch, int dtype, hipStream_t s) {
+    const dim3 grid((max_q + 63) / 64, p.H_Q, batch), block(256);
+    const size_t lds = AnyDimCfg<D>::LDS_BYTES;
+    if (dtype == FQ_F16) {
+        auto kern = tq_attention_any_dim_kernel<D, FQ_F16, PAGED>;
+        if (lds > 32768 && !fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
+    } else {
+        auto kern = tq_attention_any_dim_kernel<D, FQ_BF16, PAGED>;
+        if (lds > 32768 && !fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
+    }
+    return fq_host::check_launch();
+}
+
+// Entry for the two host functions of fq_fused_attention.hip: every argument already checked.
+int launch_attention_any_dim(const AnyDimParams& p, int D, bool paged, int max_q, int batch, int dtype, void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (p.H_Q > 65535 || batch > 65535) return FQ_ERR_BAD_SHAPE;
+    switch (D) {
+        case 64: return paged ? launch_any_dim<64, true>(p, max_q, batch, dtype, s) : launch_any_dim<64, false>(p, max_q, batch, dtype, s);
+        case 128: return paged ? launch_any_dim<128, true>(p, max_q, batch, dtype, s) : launch_any_dim<128, false>(p, max_q, batch, dtype, s);
+        case 256: return paged ? launch_any_dim<256, true>(p, max_q, batch, dtype, s) : launch_any_dim<256, false>(p, max_q, batch, dtype, s);
+        default: return FQ_ERR_UNSUPPORTED_DIM;
+    }
+}
+
+}  // namespace fq
+
+namespace fq_host {
+bool force_any_dim_attention() {
+    const char* v = getenv("FQ_ATTENTION_ANY_DIM");
+    return v && v[0] == '1';
+}
+}

@@ -34,6 +34,7 @@
 // with operands split into two fp16 terms, staged through the tile buffers.
 #include "fq_common.hpp"
 #include "fq_device.hpp"
+#include "fq_attention_any_dim.hpp"
 
 namespace fq {
 
@@ -453,7 +454,6 @@ extern "C" int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, con
     using namespace fq;
     if (B < 0 || H_Q <= 0 || H_KV <= 0 || N_Q < 0 || N_KV < 0 || H_Q % H_KV != 0) return FQ_ERR_BAD_SHAPE;
     if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
-    if (D != 128) return FQ_ERR_UNSUPPORTED_DIM;   // the tile layout is written for 128 coordinates
     if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
     if (B == 0 || N_Q == 0) return FQ_OK;
     if (N_KV == 0) return FQ_ERR_BAD_SHAPE;          // softmax over no keys is undefined
@@ -463,6 +463,19 @@ extern "C" int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, con
         !fq_host::aligned(rotation, 16) || !fq_host::aligned(out, 2))
         return FQ_ERR_MISALIGNED;
     if (B > 65535 || H_KV > 65535) return FQ_ERR_BAD_SHAPE;
+
+    if (D != 128 || fq_host::force_any_dim_attention()) {   // the tuned tile layout is written for 128 coordinates
+        AnyDimParams a{};
+        a.q = static_cast<const uint16_t*>(q);
+        a.k_packed = k_packed; a.k_norms = k_norms; a.v_packed = v_packed; a.v_norms = v_norms;
+        a.centroids_k = centroids_k; a.centroids_v = centroids_v;
+        a.rotation = rotation; a.rot_col_major = rotation_col_major;
+        a.out = static_cast<uint16_t*>(out);
+        a.H_Q = H_Q; a.H_KV = H_KV; a.G = H_Q / H_KV; a.N_Q = N_Q; a.N_KV = N_KV;
+        a.causal = (is_causal && N_Q > 1) ? 1 : 0;
+        a.scale_log2e = sm_scale * kLog2e;
+        return launch_attention_any_dim(a, D, false, N_Q, B, dtype, stream);
+    }
 
     PrefillParams p;
     p.q = static_cast<const uint16_t*>(q);
@@ -507,7 +520,6 @@ extern "C" int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, 
         num_blocks <= 0 || num_blocks > 0x7fffffffLL)
         return FQ_ERR_BAD_SHAPE;
     if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
-    if (D != 128) return FQ_ERR_UNSUPPORTED_DIM;
     if (block_size != 8 && block_size != 16 && block_size != 32) return FQ_ERR_UNSUPPORTED_BLOCK;
     if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
     if (num_seqs == 0 || max_q_len == 0) return FQ_OK;
@@ -517,6 +529,21 @@ extern "C" int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, 
         !fq_host::aligned(out, 2))
         return FQ_ERR_MISALIGNED;
     if (num_seqs > 65535 || H_KV > 65535) return FQ_ERR_BAD_SHAPE;
+
+    if (D != 128 || fq_host::force_any_dim_attention()) {
+        AnyDimParams a{};
+        a.q = static_cast<const uint16_t*>(q);
+        a.centroids_k = centroids_k; a.centroids_v = centroids_v;
+        a.rotation = rotation; a.rot_col_major = rotation_col_major;
+        a.out = static_cast<uint16_t*>(out);
+        a.H_Q = H_Q; a.H_KV = H_KV; a.G = H_Q / H_KV;
+        a.causal = is_causal ? 1 : 0;
+        a.scale_log2e = sm_scale * kLog2e;
+        a.cu_seqlens_q = cu_seqlens_q; a.seq_lens = seq_lens; a.block_table = block_table; a.cache = kv_cache;
+        a.max_blocks = max_blocks_per_seq; a.num_blocks = int(num_blocks);
+        a.bs_log2 = block_size == 8 ? 3 : (block_size == 16 ? 4 : 5);
+        return launch_attention_any_dim(a, D, true, max_q_len, num_seqs, dtype, stream);
+    }
 
     PrefillParams p;
     p.q = static_cast<const uint16_t*>(q);

@@ -166,9 +166,10 @@ int fq_tq4_decompress(const uint8_t* packed, const float* norms,
  *   out        (B, H_Q, N_Q, D) same dtype as q
  *   is_causal  key j > query i (counted from the top-left corner) is hidden;
  *              ignored when N_Q == 1, as in the reference
- * D == 128 (FQ_ERR_UNSUPPORTED_DIM otherwise); H_Q a multiple of H_KV; N_KV >= 1.
- * K and V are dequantised to fp16 with the norm folded in, so a row norm times a
- * centroid must stay below 65504.
+ * D in {64, 128, 256}: 128 runs the tuned kernel, 64 and 256 a general one
+ * (FQ_ATTENTION_ANY_DIM=1 in the environment sends 128 there too).  H_Q a multiple
+ * of H_KV; N_KV >= 1.  K and V are dequantised to fp16 with the norm folded in, so a
+ * row norm times a centroid must stay below 65504.
  */
 int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, const float* k_norms,
                           const uint8_t* v_packed, const float* v_norms,
@@ -199,7 +200,8 @@ int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, const float* k
  *   is_causal     query j of n in a sequence of L keys sees keys 0 .. L - n + j
  * The attention result is rounded to the query dtype before the rotation back,
  * as the attention library's output is in the reference.  A sequence with no
- * queries is skipped; with no keys its rows are zero.  D == 128.
+ * queries is skipped; with no keys its rows are zero.  D in {64, 128, 256} as for
+ * fq_fused_tq_attention.
  */
 int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, const uint8_t* kv_cache,
                          const int32_t* block_table, const int32_t* seq_lens,

@@ -180,7 +180,7 @@ def test_paged_prefill_argument_errors(lib):
 
     assert call(S=0) == FQ_OK and call(maxq=0) == FQ_OK
     assert call(HQ=30) == FQ_SHAPE
-    assert call(D=64) == FQ_DIM and call(D=100) == FQ_DIM
+    assert call(D=100) == FQ_DIM and call(D=64) == FQ_NULL          # 64, 128 and 256 are all served
     assert call(BS=12) == FQ_BLOCK
     assert call(dtype=2) == FQ_DTYPE
     assert call(S=-1) == FQ_SHAPE and call(MB=0) == FQ_SHAPE

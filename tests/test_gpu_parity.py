@@ -246,20 +246,20 @@ def test_paged_decode_distinct_value_codebook():
 
 # ---- fused TQ4 attention (prefill) ------------------------------------------------
 
-def _prefill_case(b, hq, hkv, nq, nkv, dtype, seed, kv_scale=1.0, v_seed_rot=None):
-    c, bnd, r = book(128)
+def _prefill_case(b, hq, hkv, nq, nkv, dtype, seed, kv_scale=1.0, v_seed_rot=None, d=128):
+    c, bnd, r = book(d)
     g = torch.Generator().manual_seed(seed)
-    q = torch.randn(b, hq, nq, 128, generator=g).to(dtype)
-    k = outlier_rows(b * hkv * nkv, 1, 128, seed + 1).reshape(b, hkv, nkv, 128) * kv_scale
-    v = outlier_rows(b * hkv * nkv, 1, 128, seed + 2).reshape(b, hkv, nkv, 128) * kv_scale
-    kp, kn = O.compress(k.reshape(-1, 1, 128), r, bnd)
-    vp, vn = O.compress(v.reshape(-1, 1, 128), r, bnd)
-    shape_p, shape_n = (b, hkv, nkv, 64), (b, hkv, nkv, 1)
+    q = torch.randn(b, hq, nq, d, generator=g).to(dtype)
+    k = outlier_rows(b * hkv * nkv, 1, d, seed + 1).reshape(b, hkv, nkv, d) * kv_scale
+    v = outlier_rows(b * hkv * nkv, 1, d, seed + 2).reshape(b, hkv, nkv, d) * kv_scale
+    kp, kn = O.compress(k.reshape(-1, 1, d), r, bnd)
+    vp, vn = O.compress(v.reshape(-1, 1, d), r, bnd)
+    shape_p, shape_n = (b, hkv, nkv, d // 2), (b, hkv, nkv, 1)
     return q, kp.reshape(shape_p), kn.reshape(shape_n), vp.reshape(shape_p), vn.reshape(shape_n), c, r
 
 
-def _check_prefill(b, hq, hkv, nq, nkv, dtype, causal, seed=11, kv_scale=1.0, scale=None, cv=None):
-    q, kp, kn, vp, vn, c, r = _prefill_case(b, hq, hkv, nq, nkv, dtype, seed, kv_scale)
+def _check_prefill(b, hq, hkv, nq, nkv, dtype, causal, seed=11, kv_scale=1.0, scale=None, cv=None, d=128):
+    q, kp, kn, vp, vn, c, r = _prefill_case(b, hq, hkv, nq, nkv, dtype, seed, kv_scale, d=d)
     cv = c if cv is None else cv
     want = O.fused_tq_attention(q, kp, kn, vp, vn, c, cv, r, sm_scale=scale, is_causal=causal)
     got = K.fused_tq_attention(q.to(DEV), kp.to(DEV), kn.to(DEV), vp.to(DEV), vn.to(DEV), c.to(DEV), cv.to(DEV),
@@ -315,6 +315,30 @@ def test_fused_attention_matches_dequantize_then_sdpa():
     assert (got.float() - ref.float()).abs().max().item() <= 2e-2 * max(1.0, ref.float().abs().max().item())
 
 
+@pytest.mark.parametrize("d", [64, 256])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_fused_attention_other_head_dims(d, dtype, causal):
+    _check_prefill(2, 8, 2, 150, 150, dtype, causal, d=d, seed=81)
+    _check_prefill(1, 4, 4, 37, 99, dtype, False, d=d, seed=82, cv=(book(d)[0] * 1.25).contiguous())
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_fused_attention_general_kernel_agrees_at_head_dim_128(causal, monkeypatch):
+    """The kernel that serves head_dim 64 and 256 also takes 128: against the oracle and against the
+    tuned kernel on the same inputs."""
+    q, kp, kn, vp, vn, c, r = _prefill_case(2, 8, 2, 200, 200, torch.bfloat16, 83)
+    dev = [t.to(DEV) for t in (q, kp, kn, vp, vn, c, r)]
+    tuned = K.fused_tq_attention(*dev[:5], dev[5], dev[5], dev[6], is_causal=causal)
+    monkeypatch.setenv("FQ_ATTENTION_ANY_DIM", "1")
+    general = K.fused_tq_attention(*dev[:5], dev[5], dev[5], dev[6], is_causal=causal)
+    torch.cuda.synchronize()
+    want = O.fused_tq_attention(q, kp, kn, vp, vn, c, c, r, is_causal=causal)
+    tol = 2e-2 * max(1.0, want.float().abs().max().item())
+    assert (general.cpu().float() - want.float()).abs().max().item() <= tol
+    assert (general.float() - tuned.float()).abs().max().item() <= tol
+
+
 def test_fused_attention_rejects_bad_arguments():
     q, kp, kn, vp, vn, c, r = _prefill_case(1, 8, 2, 16, 16, torch.bfloat16, 71)
     dev = [t.to(DEV) for t in (q, kp, kn, vp, vn, c, r)]
@@ -329,19 +353,19 @@ def test_fused_attention_rejects_bad_arguments():
 # ---- prefill over the packed paged cache -------------------------------------------------
 
 def _check_paged_prefill(q_lens, kv_lens, hq, hkv, bs=16, dtype=torch.bfloat16, causal=True, seed=21, scale=None,
-                         kv_scale=1.0, cv=None):
+                         kv_scale=1.0, cv=None, d=128):
     """q_lens[s] new tokens at the end of a sequence of kv_lens[s] keys."""
-    c, bnd, r = book(128)
+    c, bnd, r = book(d)
     cv = c if cv is None else cv
-    _, cache, table, sl = build_paged_case(kv_lens, hq, hkv, bs=bs, seed=seed, dtype=dtype, kv_scale=kv_scale)
+    _, cache, table, sl = build_paged_case(kv_lens, hq, hkv, d=d, bs=bs, seed=seed, dtype=dtype, kv_scale=kv_scale)
     g = torch.Generator().manual_seed(seed + 100)
     total = sum(q_lens)
-    q = torch.randn(total, hq, 128, generator=g).to(dtype)
+    q = torch.randn(total, hq, d, generator=g).to(dtype)
     cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
-    want = O.paged_prefill(q, cu, cache, table, sl, c, cv, r, hkv, 128, bs, sm_scale=scale, causal=causal)
+    want = O.paged_prefill(q, cu, cache, table, sl, c, cv, r, hkv, d, bs, sm_scale=scale, causal=causal)
     out = torch.full_like(q, 7.0).to(DEV)
     got = K.paged_tq4_prefill(q.to(DEV), cu.to(DEV), max(q_lens), cache.to(DEV), table.to(DEV), sl.to(DEV),
-                              c.to(DEV), cv.to(DEV), r.to(DEV), hkv, 128, bs, sm_scale=scale, causal=causal, out=out)
+                              c.to(DEV), cv.to(DEV), r.to(DEV), hkv, d, bs, sm_scale=scale, causal=causal, out=out)
     torch.cuda.synchronize()
     assert got.data_ptr() == out.data_ptr() and got.dtype == dtype and got.shape == q.shape
     got = got.cpu().float()
@@ -384,6 +408,18 @@ def test_paged_prefill_scaled_inputs_custom_scale_and_value_codebook():
     c, _, _ = book(128)
     _check_paged_prefill([90, 31], [120, 31], hq=8, hkv=2, dtype=torch.float16, kv_scale=6.0, scale=0.05,
                          cv=(c * 1.25).contiguous())
+
+
+@pytest.mark.parametrize("d", [64, 256])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_paged_prefill_other_head_dims(d, dtype):
+    _check_paged_prefill([7, 64, 1, 0, 130], [45, 64, 300, 20, 131], hq=8, hkv=2, d=d, dtype=dtype)
+    _check_paged_prefill([50, 3], [77, 0], hq=4, hkv=4, d=d, dtype=dtype, bs=8, causal=False)
+
+
+def test_paged_prefill_general_kernel_agrees_at_head_dim_128(monkeypatch):
+    monkeypatch.setenv("FQ_ATTENTION_ANY_DIM", "1")
+    _check_paged_prefill([7, 64, 1, 130, 32], [45, 64, 300, 131, 500], hq=32, hkv=8)
 
 
 def test_paged_prefill_long_sequence_equals_decode_on_last_token():
