@@ -783,15 +783,18 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     // the table is filled while the page ids are on their way
     fill_pair_tables<8>(lut, cent_k_mine, cent_v_mine, PROD ? 7 : 15, h, lane);
 
-    // ---- copy plan: chunk c = tid + 512 k of the tile, k = 0..4 (the last round only
-    // for the first 128 threads) -----------------------------------------------------------
+    // ---- copy plan: chunk c = tid + 512 k of the tile, k = 0..3; the remaining chunks go out as
+    // one dword per thread where that comes out even (128 chunks = 512 dwords: every wavefront
+    // then moves the same amount), else as whole chunks by the first wavefronts ------------------
     constexpr int ROUNDS = 5;
+    constexpr bool kSpreadTail = (kChunksPerTile - 4 * 512) * 4 == 512;
     uint32_t src_off[ROUNDS];    // byte offset from the base of the chunk's page
     int src_page[ROUNDS];        // which of the tile's pages (lane constant)
     int dst_off[ROUNDS];         // byte offset inside the LDS tile slot
 #pragma unroll
     for (int k = 0; k < ROUNDS; ++k) {
         int c = tid + 512 * k;
+        if (kSpreadTail && k == 4) c = 4 * 512 + (tid >> 2);
         c = c < kChunksPerTile ? c : kChunksPerTile - 1;
         // rows of a page are contiguous: chunk c of the tile is chunk c - page * (chunks per page) of its page
         constexpr int PC = BS * kChunksPerRow;
@@ -799,10 +802,11 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
 #pragma unroll
         for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
         src_page[k] = pg;
-        src_off[k] = uint32_t(16 * (c - pg * PC));
-        dst_off[k] = kChunkDst<PROD>.off[c];
+        const int sub = (kSpreadTail && k == 4) ? 4 * (tid & 3) : 0;
+        src_off[k] = uint32_t(16 * (c - pg * PC) + sub);
+        dst_off[k] = kChunkDst<PROD>.off[c] + sub;
     }
-    const bool has_round4 = tid < kChunksPerTile - 4 * 512;   // 128 threads, whole wavefronts
+    const bool has_round4 = kSpreadTail || tid < kChunksPerTile - 4 * 512;   // else whole wavefronts
 
     uint4v stage_reg[ROUNDS];
     auto issue_loads = [&](int t0) {
@@ -820,14 +824,16 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             const uint8_t* b = base[0];
 #pragma unroll
             for (int i = 1; i < PPT; ++i) b = pg_k == i ? base[i] : b;
-            if (k < 4 || has_round4) stage_reg[k] = *reinterpret_cast<const uint4v*>(b + in_page + src_off[k]);
+            if (kSpreadTail && k == 4) stage_reg[k].x = *reinterpret_cast<const uint32_t*>(b + in_page + src_off[k]);
+            else if (k < 4 || has_round4) stage_reg[k] = *reinterpret_cast<const uint4v*>(b + in_page + src_off[k]);
         }
     };
     auto write_slot = [&](int slot) {
         uint8_t* dst = slots + slot * kTileBytes;
 #pragma unroll
         for (int k = 0; k < ROUNDS; ++k)
-            if (k < 4 || has_round4) *reinterpret_cast<uint4v*>(dst + dst_off[k]) = stage_reg[k];
+            if (kSpreadTail && k == 4) *reinterpret_cast<uint32_t*>(dst + dst_off[k]) = stage_reg[k].x;
+            else if (k < 4 || has_round4) *reinterpret_cast<uint4v*>(dst + dst_off[k]) = stage_reg[k];
     };
 
 #pragma unroll
