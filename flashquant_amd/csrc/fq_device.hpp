@@ -201,6 +201,40 @@ __device__ __forceinline__ float4v rotate_block_f16(const half8 (&a)[D / 32], co
     return acc_hi + acc_lo * (1.0f / 4096.0f);
 }
 
+// The same for rows that are bfloat16: they go to the bf16 MFMA as they are, against the matrix
+// block split into three bf16 terms (3 x 8 bits: the float32 value exactly; bf16 keeps the float32
+// exponent range, so the terms need no scaling and share one accumulator).
+typedef __bf16 bf16v8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ __bf16 bf16_top(float f) {          // truncation: the next term takes up the rest
+    return __builtin_bit_cast(__bf16, uint16_t(float_to_bits(f) >> 16));
+}
+__device__ __forceinline__ float bf16_as_float(__bf16 h) {
+    return bits_to_float(uint32_t(__builtin_bit_cast(uint16_t, h)) << 16);
+}
+template <int D>
+__device__ __forceinline__ void split_rotation_block_bf16(const float (&b)[D / 32][8], bf16v8 (&t)[3][D / 32]) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const __bf16 t0 = bf16_top(b[j][e]);
+            const float r1 = b[j][e] - bf16_as_float(t0);
+            const __bf16 t1 = bf16_top(r1);
+            t[0][j][e] = t0;
+            t[1][j][e] = t1;
+            t[2][j][e] = bf16_top(r1 - bf16_as_float(t1));
+        }
+}
+template <int D>
+__device__ __forceinline__ float4v rotate_block_bf16(const bf16v8 (&a)[D / 32], const bf16v8 (&t)[3][D / 32]) {
+    float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 2; k >= 0; --k)       // the small terms first
+#pragma unroll
+        for (int j = 0; j < D / 32; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], t[k][j], acc, 0, 0, 0);
+    return acc;
+}
+
 // Wavefront-wide maximum (all 64 lanes receive it), in the VALU: rotations inside the rows
 // of 16 lanes, then the row swaps.
 __device__ __forceinline__ float wave_max(float v) {

@@ -862,10 +862,19 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             // float32 sketched query (H_Q <= 64) takes the first slot and a barrier of its own.
             uint16_t* qs = reinterpret_cast<uint16_t*>(slots + kTileBytes);
             float* qs2 = reinterpret_cast<float*>(slots);
-            // this wavefront's 16 matrix columns as two fp16 terms each
+            // This wavefront's 16 matrix columns.  bfloat16 heads go to the bf16 MFMA as loaded, against
+            // the columns in three bf16 terms; fp16 heads are scaled by a power of two and go to the fp16
+            // MFMA against two fp16 terms.  Either way the products are exact.
+            constexpr bool kRawBf16 = DT == FQ_BF16;
             half8 rot_hi[KS], rot_lo[KS], sk_hi[KS], sk_lo[KS];
-            split_rotation_block<D>(rot_b, rot_hi, rot_lo);
-            if constexpr (PROD) split_rotation_block<D>(rot_s, sk_hi, sk_lo);
+            bf16v8 rot_t[3][KS], sk_t[3][KS];
+            if constexpr (kRawBf16) {
+                split_rotation_block_bf16<D>(rot_b, rot_t);
+                if constexpr (PROD) split_rotation_block_bf16<D>(rot_s, sk_t);
+            } else {
+                split_rotation_block<D>(rot_b, rot_hi, rot_lo);
+                if constexpr (PROD) split_rotation_block<D>(rot_s, sk_hi, sk_lo);
+            }
             for (int rb = 0; 16 * rb < p.H_Q; ++rb) {
                 const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
                 uint4v raw[KS];
@@ -873,17 +882,26 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
                 for (int j = 0; j < KS; ++j)
                     raw[j] = rb < 2 ? q_pre[rb & 1][j]
                                     : *reinterpret_cast<const uint4v*>(qseq + row * D + 32 * j + 8 * g);
-                half8 a[KS];
-                float up;
-                rows_as_f16<D, DT>(raw, a, up);
-                const float4v acc = rotate_block_f16<D>(a, rot_hi, rot_lo);
+                float4v acc, acc2 = {0.f, 0.f, 0.f, 0.f};
+                float up = 1.0f;
+                if constexpr (kRawBf16) {
+                    bf16v8 a[KS];
+#pragma unroll
+                    for (int j = 0; j < KS; ++j) a[j] = __builtin_bit_cast(bf16v8, raw[j]);
+                    acc = rotate_block_bf16<D>(a, rot_t);
+                    if constexpr (PROD) acc2 = rotate_block_bf16<D>(a, sk_t);
+                } else {
+                    half8 a[KS];
+                    rows_as_f16<D, DT>(raw, a, up);
+                    acc = rotate_block_f16<D>(a, rot_hi, rot_lo);
+                    if constexpr (PROD) acc2 = rotate_block_f16<D>(a, sk_hi, sk_lo);
+                }
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int head = 16 * rb + 4 * g + i;
                     if (head < p.H_Q) qs[head * D + 16 * h + n] = store_elem<DT>(acc[i] * up);
                 }
                 if constexpr (PROD) {
-                    const float4v acc2 = rotate_block_f16<D>(a, sk_hi, sk_lo);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int head = 16 * rb + 4 * g + i;
