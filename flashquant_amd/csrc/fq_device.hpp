@@ -64,19 +64,27 @@ __device__ __forceinline__ void fill_byte_table(uint32_t* table, float mine, int
 template <int WAVES>
 __device__ __forceinline__ void fill_pair_tables(uint32_t* table, float mine_k, float mine_v, int k_mask, int wave,
                                                  int lane) {
+    static_assert(WAVES == 8, "byte = wave + 8 i: the high nibble is i / 2, the low nibble wave or wave + 8");
     // the fp16 centroid of this lane; entries are then assembled on the scalar unit
     const int hk = int(__builtin_bit_cast(uint16_t, _Float16(mine_k)));
     const int hv = int(__builtin_bit_cast(uint16_t, _Float16(mine_v)));
     uint32_t* mine = table + lane;
+    // low halves of this wavefront's entries (two possible low nibbles), shifted into place once
+    const uint32_t klo[2] = {uint32_t(__builtin_amdgcn_readlane(hk, wave & k_mask)) << 16,
+                             uint32_t(__builtin_amdgcn_readlane(hk, (wave + 8) & k_mask)) << 16};
+    const uint32_t vlo[2] = {uint32_t(__builtin_amdgcn_readlane(hv, wave)) << 16,
+                             uint32_t(__builtin_amdgcn_readlane(hv, wave + 8)) << 16};
 #pragma unroll
-    for (int i = 0; i < 256 / WAVES; ++i) {
-        const int byte = wave + WAVES * i;
-        const uint32_t khi = uint32_t(__builtin_amdgcn_readlane(hk, (byte >> 4) & k_mask));
-        const uint32_t klo = uint32_t(__builtin_amdgcn_readlane(hk, byte & k_mask));
-        const uint32_t vhi = uint32_t(__builtin_amdgcn_readlane(hv, byte >> 4));
-        const uint32_t vlo = uint32_t(__builtin_amdgcn_readlane(hv, byte & 15));
-        const uint32_t ke = khi | (klo << 16), ve = vhi | (vlo << 16);
-        mine[wave * 64 + WAVES * 64 * i] = lane < 32 ? ke : ve;
+    for (int hi = 0; hi < 16; ++hi) {
+        // the high nibble is a compile-time lane index: one readlane per table and nibble
+        const uint32_t kh = uint32_t(__builtin_amdgcn_readlane(hk, hi & k_mask));
+        const uint32_t vh = uint32_t(__builtin_amdgcn_readlane(hv, hi));
+#pragma unroll
+        for (int lo = 0; lo < 2; ++lo) {
+            const int i = 2 * hi + lo;                      // byte = wave + 8 i = 16 hi + (wave + 8 lo)
+            const uint32_t ke = kh | klo[lo], ve = vh | vlo[lo];
+            mine[wave * 64 + WAVES * 64 * i] = lane < 32 ? ke : ve;
+        }
     }
 }
 __device__ __forceinline__ void build_byte_table(uint32_t* table, const float* __restrict__ centroids, int wave,
