@@ -648,6 +648,68 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         if constexpr (PROD) load_rotation_any<128>(p.sketch, false, true, 16 * h, n, g, rot_s);
     }
 
+    // Everything that depends on the lane alone is worked out here, while the first loads are on
+    // their way: the first value that comes back from memory is needed 2.5 us after entry.
+    // ---- copy plan: chunk c = tid + 512 k of the tile, k = 0..3; the remaining chunks go out as
+    // one dword per thread where that comes out even (128 chunks = 512 dwords: every wavefront
+    // then moves the same amount), else as whole chunks by the first wavefronts ------------------
+    constexpr int ROUNDS = 5;
+    constexpr bool kSpreadTail = (kChunksPerTile - 4 * 512) * 4 == 512;
+    uint32_t src_off[ROUNDS];    // byte offset from the base of the chunk's page
+    int src_page[ROUNDS];        // which of the tile's pages (lane constant)
+    int dst_off[ROUNDS];         // byte offset inside the LDS tile slot
+#pragma unroll
+    for (int k = 0; k < ROUNDS; ++k) {
+        int c = tid + 512 * k;
+        if (kSpreadTail && k == 4) c = 4 * 512 + (tid >> 2);
+        c = c < kChunksPerTile ? c : kChunksPerTile - 1;
+        // rows of a page are contiguous: chunk c of the tile is chunk c - page * (chunks per page) of its page
+        constexpr int PC = BS * kChunksPerRow;
+        int pg = 0;
+#pragma unroll
+        for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
+        src_page[k] = pg;
+        const int sub = (kSpreadTail && k == 4) ? 4 * (tid & 3) : 0;
+        src_off[k] = uint32_t(16 * (c - pg * PC) + sub);
+        dst_off[k] = kChunkDst<PROD>.off[c] + sub;
+    }
+    const bool has_round4 = kSpreadTail || tid < kChunksPerTile - 4 * 512;   // else whole wavefronts
+    // ---- lane-constant LDS read offsets (inside a tile slot) -------------------------------
+    int k_rd[2];                // K operand of block b: 16 bytes of row n, quarter g
+    int v_rd[2][4];             // V operand: dword n of rows 4g + i of block b
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        k_rd[b] = b * kStageBytes + 16 * staged_slot(h, n, g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            v_rd[b][i] = b * kStageBytes + 8192 + 16 * staged_slot(h, 4 * g + i, n >> 2) + 4 * (n & 3);
+    }
+    // the (block, row) of this lane's scores, and the slot of each score in the P operand
+    int sc_tok[NSC];            // token offset inside the tile
+    int n_rd[NSC];              // K norm offset; the V norm is 512 bytes further
+#pragma unroll
+    for (int e = 0; e < NSC; ++e) {
+        int blk, row;
+        if (GP == 4) { blk = cls >> 1; row = 4 * g + 2 * (cls & 1) + e; }
+        else if (GP == 8) { blk = cls; row = 4 * g + e; }
+        else { blk = e >> 2; row = 4 * g + (e & 3); }
+        sc_tok[e] = 16 * blk + row;
+        n_rd[e] = blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
+    }
+
+    // dword d of the P operand holds slots 2d, 2d + 1: it is this lane's when its class owns them
+    uint32_t pa_mask[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        bool mine;
+        if (GP == 4) mine = d == cls;                 // class = 2 * block + half, one dword each
+        else if (GP == 8) mine = (d >> 1) == cls;     // class = block, two dwords each
+        else mine = true;
+        pa_mask[d] = mine ? 0xffffffffu : 0u;
+    }
+
+    __builtin_amdgcn_sched_barrier(0);
+
     const int NS = p.num_splits;
     const bool rowwide = p.max_blocks <= 64 * PVR;
     // every sequence is cut into the same token chunks (those of the longest possible context):
@@ -783,30 +845,6 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     // the table is filled while the page ids are on their way
     fill_pair_tables<8>(lut, cent_k_mine, cent_v_mine, PROD ? 7 : 15, h, lane);
 
-    // ---- copy plan: chunk c = tid + 512 k of the tile, k = 0..3; the remaining chunks go out as
-    // one dword per thread where that comes out even (128 chunks = 512 dwords: every wavefront
-    // then moves the same amount), else as whole chunks by the first wavefronts ------------------
-    constexpr int ROUNDS = 5;
-    constexpr bool kSpreadTail = (kChunksPerTile - 4 * 512) * 4 == 512;
-    uint32_t src_off[ROUNDS];    // byte offset from the base of the chunk's page
-    int src_page[ROUNDS];        // which of the tile's pages (lane constant)
-    int dst_off[ROUNDS];         // byte offset inside the LDS tile slot
-#pragma unroll
-    for (int k = 0; k < ROUNDS; ++k) {
-        int c = tid + 512 * k;
-        if (kSpreadTail && k == 4) c = 4 * 512 + (tid >> 2);
-        c = c < kChunksPerTile ? c : kChunksPerTile - 1;
-        // rows of a page are contiguous: chunk c of the tile is chunk c - page * (chunks per page) of its page
-        constexpr int PC = BS * kChunksPerRow;
-        int pg = 0;
-#pragma unroll
-        for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
-        src_page[k] = pg;
-        const int sub = (kSpreadTail && k == 4) ? 4 * (tid & 3) : 0;
-        src_off[k] = uint32_t(16 * (c - pg * PC) + sub);
-        dst_off[k] = kChunkDst<PROD>.off[c] + sub;
-    }
-    const bool has_round4 = kSpreadTail || tid < kChunksPerTile - 4 * 512;   // else whole wavefronts
 
     uint4v stage_reg[ROUNDS];
     auto issue_loads = [&](int t0) {
@@ -968,40 +1006,6 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
             for (int e = 0; e < 8; ++e) qh[ks][e] = _Float16(qf[ks][e] * down);
-    }
-
-    // ---- lane-constant LDS read offsets (inside a tile slot) -------------------------------
-    int k_rd[2];                // K operand of block b: 16 bytes of row n, quarter g
-    int v_rd[2][4];             // V operand: dword n of rows 4g + i of block b
-#pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        k_rd[b] = b * kStageBytes + 16 * staged_slot(h, n, g);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            v_rd[b][i] = b * kStageBytes + 8192 + 16 * staged_slot(h, 4 * g + i, n >> 2) + 4 * (n & 3);
-    }
-    // the (block, row) of this lane's scores, and the slot of each score in the P operand
-    int sc_tok[NSC];            // token offset inside the tile
-    int n_rd[NSC];              // K norm offset; the V norm is 512 bytes further
-#pragma unroll
-    for (int e = 0; e < NSC; ++e) {
-        int blk, row;
-        if (GP == 4) { blk = cls >> 1; row = 4 * g + 2 * (cls & 1) + e; }
-        else if (GP == 8) { blk = cls; row = 4 * g + e; }
-        else { blk = e >> 2; row = 4 * g + (e & 3); }
-        sc_tok[e] = 16 * blk + row;
-        n_rd[e] = blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
-    }
-
-    // dword d of the P operand holds slots 2d, 2d + 1: it is this lane's when its class owns them
-    uint32_t pa_mask[4];
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        bool mine;
-        if (GP == 4) mine = d == cls;                 // class = 2 * block + half, one dword each
-        else if (GP == 8) mine = (d >> 1) == cls;     // class = block, two dwords each
-        else mine = true;
-        pa_mask[d] = mine ? 0xffffffffu : 0u;
     }
 
     // ---- running state ---------------------------------------------------------------------
