@@ -595,8 +595,8 @@ __device__ __forceinline__ constexpr int sign_order(int e) {
     return order[e];
 }
 
-template <int BSL, int GP, int DT, int PVR, bool PROD>
-__global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodeParams p) {
+template <int BSL, int GP, int DT, int PVR, bool PROD, int CW>
+__global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     using Cfg = StagedCfg<PROD>;
     constexpr int kStageBytes = Cfg::STAGE_BYTES;
     constexpr int kTileBytes = Cfg::TILE_BYTES;
@@ -619,6 +619,9 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int h = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront = KV head
+    // CW > 0: wavefronts 8 .. 8 + CW - 1 only move tiles from the cache to LDS and the first eight
+    // only consume them, so that no wavefront that computes ever waits for global memory.
+    const bool copier = CW > 0 && h >= 8;
     const int n = lane & 15;
     const int g = lane >> 4;
     const int hd = n % GP;
@@ -643,7 +646,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     const uint32_t lane_off_v = 128u + lane_off;
     float rot_b[4][8];
     float rot_s[4][8];
-    if (p.rotation != nullptr) {
+    if (p.rotation != nullptr && !copier) {
         load_rotation_any<128>(p.rotation, p.rot_col_major != 0, true, 16 * h, n, g, rot_b);
         if constexpr (PROD) load_rotation_any<128>(p.sketch, false, true, 16 * h, n, g, rot_s);
     }
@@ -660,8 +663,8 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     int dst_off[ROUNDS];         // byte offset inside the LDS tile slot
 #pragma unroll
     for (int k = 0; k < ROUNDS; ++k) {
-        int c = tid + 512 * k;
-        if (kSpreadTail && k == 4) c = 4 * 512 + (tid >> 2);
+        int c = (tid & 511) + 512 * k;
+        if (kSpreadTail && k == 4) c = 4 * 512 + ((tid & 511) >> 2);
         c = c < kChunksPerTile ? c : kChunksPerTile - 1;
         // rows of a page are contiguous: chunk c of the tile is chunk c - page * (chunks per page) of its page
         constexpr int PC = BS * kChunksPerRow;
@@ -783,7 +786,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
 
     const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + int64_t(seq) * p.H_Q * 128;
     uint4v q_pre[2][4];
-    if (p.rotation != nullptr) {
+    if (p.rotation != nullptr && !copier) {
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
@@ -811,7 +814,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     const int end = L < begin + chunk ? L : begin + chunk;
     const int hq_lane = h * p.G + n;
     if (begin >= end) {   // uniform over the workgroup
-        if (g == 0 && n < p.G) {
+        if (g == 0 && n < p.G && !copier) {
             const int64_t o = (int64_t(seq) * p.H_Q + hq_lane) * NS + split;
             p.part_m[o] = -__builtin_inff();
             p.part_l[o] = 0.0f;
@@ -843,7 +846,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
         return v;
     };
     // the table is filled while the page ids are on their way
-    fill_pair_tables<8>(lut, cent_k_mine, cent_v_mine, PROD ? 7 : 15, h, lane);
+    if (!copier) fill_pair_tables<8>(lut, cent_k_mine, cent_v_mine, PROD ? 7 : 15, h, lane);
 
 
     uint4v stage_reg[ROUNDS];
@@ -876,8 +879,100 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
 
 #pragma unroll
     for (int r = 0; r < PVR; ++r) pv[r] = pv[r] < 0 ? 0 : (pv[r] > max_page ? max_page : pv[r]);
+    const int last_t0 = begin + ((end - begin - 1) & ~31);
+    auto clamp_t0 = [&](int t) { return t < last_t0 ? t : last_t0; };
+
+    if constexpr (CW > 0) {
+        if (copier) {
+            // ---- the copy wavefronts: chunk c = ct + 64 CW k of a tile, the rest as 8 bytes per
+            // thread; two tiles in flight in registers (sets A and B), each written to the slot that
+            // the tile two before it has just left --------------------------------------------------
+            constexpr int CT = 64 * CW;
+            constexpr int FULL = kChunksPerTile / CT;
+            constexpr int REST = kChunksPerTile - FULL * CT;
+            constexpr bool kHalfTail = REST * 2 == CT;   // else whole chunks by the first REST threads
+            constexpr int NR = FULL + 1;
+            const int ct = tid - 512;
+            uint32_t c_src[NR];
+            int c_page[NR];
+            int c_dst[NR];
+#pragma unroll
+            for (int k = 0; k < NR; ++k) {
+                int c = k < FULL ? ct + CT * k : FULL * CT + (kHalfTail ? ct >> 1 : ct);
+                c = c < kChunksPerTile ? c : kChunksPerTile - 1;
+                constexpr int PC = BS * kChunksPerRow;
+                int pg = 0;
+#pragma unroll
+                for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
+                c_page[k] = pg;
+                const int sub = (k < FULL || !kHalfTail) ? 0 : 8 * (ct & 1);
+                c_src[k] = uint32_t(16 * (c - pg * PC) + sub);
+                c_dst[k] = kChunkDst<PROD>.off[c] + sub;
+            }
+            const bool has_rest = kHalfTail || ct < REST;
+            auto c_issue = [&](uint4v (&r)[NR], int t0) {
+                if (t0 > last_t0) return;             // beyond the split: nothing to fetch
+                const uint8_t* base[PPT];
+                const int p0 = (t0 >> BSL) - split_p0;
+#pragma unroll
+                for (int i = 0; i < PPT; ++i) base[i] = cache + int64_t(page_id(p0 + i)) * page_bytes;
+                const uint32_t in_page = BS >= 32 ? uint32_t((t0 & (BS - 1)) * ROWB) : 0u;
+#pragma unroll
+                for (int k = 0; k < NR; ++k) {
+                    constexpr bool kUniformPage = (BS * kChunksPerRow) % 64 == 0;
+                    const int pg_k = kUniformPage ? __builtin_amdgcn_readfirstlane(c_page[k]) : c_page[k];
+                    const uint8_t* b = base[0];
+#pragma unroll
+                    for (int i = 1; i < PPT; ++i) b = pg_k == i ? base[i] : b;
+                    if (k < FULL) {
+                        r[k] = *reinterpret_cast<const uint4v*>(b + in_page + c_src[k]);
+                    } else if (!kHalfTail) {
+                        if (has_rest) r[k] = *reinterpret_cast<const uint4v*>(b + in_page + c_src[k]);
+                    } else {
+                        const uint2v t = *reinterpret_cast<const uint2v*>(b + in_page + c_src[k]);
+                        r[k].x = t.x;
+                        r[k].y = t.y;
+                    }
+                }
+            };
+            auto c_write = [&](int slot, const uint4v (&r)[NR]) {
+                uint8_t* dst = slots + slot * kTileBytes;
+#pragma unroll
+                for (int k = 0; k < NR; ++k) {
+                    if (k < FULL) *reinterpret_cast<uint4v*>(dst + c_dst[k]) = r[k];
+                    else if (!kHalfTail) { if (has_rest) *reinterpret_cast<uint4v*>(dst + c_dst[k]) = r[k]; }
+                    else *reinterpret_cast<uint2v*>(dst + c_dst[k]) = uint2v{r[k].x, r[k].y};
+                }
+            };
+            uint4v ra[NR], rb[NR];
+#pragma unroll
+            for (int k = 0; k < NR; ++k) ra[k] = rb[k] = uint4v{0u, 0u, 0u, 0u};
+            c_issue(ra, begin);
+            c_issue(rb, begin + 32);
+            if constexpr (PROD) {
+                // the sketched query passes through the first slot: two barriers, then the tile
+                if (p.rotation != nullptr) { __syncthreads(); __syncthreads(); }
+                c_write(0, ra);
+                c_issue(ra, begin + 64);
+            } else {
+                c_write(0, ra);                       // the first slot is not part of the query exchange
+                c_issue(ra, begin + 64);
+                if (p.rotation != nullptr) __syncthreads();   // the barrier of the query exchange
+            }
+            for (int t0 = begin; t0 < end; t0 += 64) {
+                __syncthreads();                      // tile i is in LDS; the slot of tile i - 1 is free
+                c_write(1, rb);                       // tile i + 1
+                c_issue(rb, t0 + 96);                 // tile i + 3
+                if (t0 + 32 >= end) break;
+                __syncthreads();
+                c_write(0, ra);                       // tile i + 2
+                c_issue(ra, t0 + 128);                // tile i + 4
+            }
+            return;
+        }
+    }
     // the loads of the first tile fly while the query is prepared
-    issue_loads(begin);
+    if constexpr (CW == 0) issue_loads(begin);
 
     // ---- query operand ------------------------------------------------------------------
     // With a rotation matrix the workgroup first rotates all query heads of its sequence:
@@ -1176,9 +1271,7 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
     };
 
     // ---- tiles ------------------------------------------------------------------------------------
-    {
-        const int last_t0 = begin + ((end - begin - 1) & ~31);
-        auto clamp_t0 = [&](int t) { return t < last_t0 ? t : last_t0; };
+    if constexpr (CW == 0) {
         write_slot(0);                            // tile 0, loaded before the query was prepared
         issue_loads(clamp_t0(begin + 32));
         int i = 0;
@@ -1186,6 +1279,12 @@ __global__ __launch_bounds__(512) void paged_decode_staged_kernel(const DecodePa
             __syncthreads();                      // tile i is in LDS; slot of tile i - 1 is free
             write_slot((i + 1) & 1);              // tile i + 1 (its loads ran during tile i - 1)
             issue_loads(clamp_t0(t0 + 64));       // tile i + 2
+            compute_tile(t0, i & 1);
+        }
+    } else {
+        int i = 0;
+        for (int t0 = begin; t0 < end; t0 += 32, ++i) {
+            __syncthreads();                      // the copy wavefronts have put tile i in LDS
             compute_tile(t0, i & 1);
         }
     }
@@ -1411,18 +1510,33 @@ inline bool staged_applies(int D, int H_KV) {
 }
 
 template <bool PROD, typename K>
-int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream) {
+int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream, int copy_waves = 0) {
     // dynamic part only; the 64 KB table is static
     const size_t lds = 2 * size_t(StagedCfg<PROD>::TILE_BYTES);
-    return launch_with_lds(kernel, p, dim3(S, p.num_splits, 1), dim3(512), lds, stream);
+    return launch_with_lds(kernel, p, dim3(S, p.num_splits, 1), dim3(512 + 64 * copy_waves), lds, stream);
+}
+
+// The staged kernel runs with four more wavefronts that only copy; FQ_DECODE_COPY_WAVES=0
+// selects the form in which the eight wavefronts copy and compute in turn.
+inline int staged_copy_waves() {
+    static const int v = [] {
+        const char* e = std::getenv("FQ_DECODE_COPY_WAVES");
+        return (e != nullptr && e[0] == '0') ? 0 : 4;
+    }();
+    return v;
 }
 
 // Staged kernel for every page size and group size; PROD selects the TurboQuantProd page format.
 template <int DT, bool PROD>
 int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream_t stream) {
 #define FQ_STAGED_GP(BSL, GPV)                                                                                  \
-    return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD>, p, S, stream)        \
-                : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD>, p, S, stream)
+    /* TurboQuantProd pages with 16 query heads per KV head do not fit three waves' registers */                \
+    if constexpr (!(PROD && GPV == 16))                                                                         \
+    if (staged_copy_waves() == 4)                                                                               \
+        return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4>, p, S, stream, 4) \
+                    : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 4>, p, S, stream, 4); \
+    return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 0>, p, S, stream)     \
+                : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 0>, p, S, stream)
 #define FQ_STAGED_BS(BSL)                         \
     do {                                          \
         if (p.G <= 4) { FQ_STAGED_GP(BSL, 4); }   \
