@@ -1519,24 +1519,23 @@ int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream, in
 // The staged kernel runs with four more wavefronts that only copy; FQ_DECODE_COPY_WAVES=0
 // selects the form in which the eight wavefronts copy and compute in turn.
 inline int staged_copy_waves() {
-    static const int v = [] {
-        const char* e = std::getenv("FQ_DECODE_COPY_WAVES");
-        return (e != nullptr && e[0] == '0') ? 0 : 4;
-    }();
-    return v;
+    const char* e = std::getenv("FQ_DECODE_COPY_WAVES");
+    return (e != nullptr && e[0] == '0') ? 0 : 4;
 }
 
 // Staged kernel for every page size and group size; PROD selects the TurboQuantProd page format.
 template <int DT, bool PROD>
 int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream_t stream) {
 #define FQ_STAGED_GP(BSL, GPV)                                                                                  \
-    /* TurboQuantProd pages with 16 query heads per KV head do not fit three waves' registers */                \
-    if constexpr (!(PROD && GPV == 16))                                                                         \
-    if (staged_copy_waves() == 4)                                                                               \
-        return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4>, p, S, stream, 4) \
-                    : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 4>, p, S, stream, 4); \
-    return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 0>, p, S, stream)     \
-                : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 0>, p, S, stream)
+    /* TurboQuantProd pages come with at most 64 query heads (8 per KV head) */                                 \
+    if constexpr (PROD && GPV == 16) return FQ_ERR_BAD_SHAPE;                                                   \
+    else {                                                                                                      \
+        if (staged_copy_waves() == 4)                                                                           \
+            return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4>, p, S, stream, 4) \
+                        : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 4>, p, S, stream, 4); \
+        return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 0>, p, S, stream) \
+                    : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 0>, p, S, stream); \
+    }
 #define FQ_STAGED_BS(BSL)                         \
     do {                                          \
         if (p.G <= 4) { FQ_STAGED_GP(BSL, 4); }   \

@@ -166,6 +166,18 @@ def test_paged_decode_llama8b_heads(num_splits):
     _decode_case([37, 0, 16, 300, 64, 65, 1, 129], hq=32, hkv=8, num_splits=num_splits)
 
 
+@pytest.mark.parametrize("hq,bs", [(32, 16), (64, 8), (128, 32)])
+def test_paged_decode_without_copy_wavefronts(hq, bs, monkeypatch):
+    """FQ_DECODE_COPY_WAVES=0: the eight wavefronts of the staged kernel copy and compute in turn."""
+    monkeypatch.setenv("FQ_DECODE_COPY_WAVES", "0")
+    _decode_case([37, 0, 16, 300, 64, 65, 1, 129], hq=hq, hkv=8, bs=bs, num_splits=3)
+
+
+def test_prod_paged_decode_without_copy_wavefronts(monkeypatch):
+    monkeypatch.setenv("FQ_DECODE_COPY_WAVES", "0")
+    _check_prod_decode([300, 1, 77, 0, 129], 32, num_splits=5)
+
+
 @pytest.mark.parametrize("num_splits", [40, 64])
 def test_paged_decode_ragged_batch_with_more_splits_than_cus(num_splits):
     """More (sequence, split) workgroups than CUs: the kernel sizes its chunks from the actual
