@@ -595,6 +595,20 @@ __device__ __forceinline__ constexpr int sign_order(int e) {
     return order[e];
 }
 
+// Counting flags in LDS: wavefronts that have to meet without holding up the rest of the workgroup
+// (a workgroup barrier would make the copy wavefronts wait for the query rotation and the
+// computing ones for the first tile).  signal: every earlier LDS write of the wavefront is done
+// first.  wait: bounded, so that a wavefront always reaches the end of the kernel.
+__device__ __forceinline__ void lds_flag_signal(uint32_t* flag, int lane) {
+    if (lane == 0) __hip_atomic_fetch_add(flag, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void lds_flag_wait(uint32_t* flag, uint32_t count) {
+    for (int spin = 0; spin < (1 << 20); ++spin) {
+        if (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= count) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
 template <int BSL, int GP, int DT, int PVR, bool PROD, int CW>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     using Cfg = StagedCfg<PROD>;
@@ -615,6 +629,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // that folds into the offset field of every lookup; the tile slots are dynamic.
     __shared__ __attribute__((aligned(256))) uint32_t lut[kLutWords];
     extern __shared__ __attribute__((aligned(16))) uint8_t slots[];   // two tile slots
+    __shared__ uint32_t flags[2];   // CW > 0: rotated heads stored / sketched heads read back
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -646,10 +661,15 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     const uint32_t lane_off_v = 128u + lane_off;
     float rot_b[4][8];
     float rot_s[4][8];
-    if (p.rotation != nullptr && !copier) {
-        load_rotation_any<128>(p.rotation, p.rot_col_major != 0, true, 16 * h, n, g, rot_b);
-        if constexpr (PROD) load_rotation_any<128>(p.sketch, false, true, 16 * h, n, g, rot_s);
-    }
+    auto load_matrix_columns = [&]() {
+        if (p.rotation != nullptr && !copier) {
+            load_rotation_any<128>(p.rotation, p.rot_col_major != 0, true, 16 * h, n, g, rot_b);
+            if constexpr (PROD) load_rotation_any<128>(p.sketch, false, true, 16 * h, n, g, rot_s);
+        }
+    };
+    // With copy wavefronts the sequence length and the page ids are asked for first (below): the
+    // first tile hangs on them, the query rotation has time.
+    if constexpr (CW == 0) load_matrix_columns();
 
     // Everything that depends on the lane alone is worked out here, while the first loads are on
     // their way: the first value that comes back from memory is needed 2.5 us after entry.
@@ -663,6 +683,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     int dst_off[ROUNDS];         // byte offset inside the LDS tile slot
 #pragma unroll
     for (int k = 0; k < ROUNDS; ++k) {
+        if constexpr (CW > 0) {   // the copy wavefronts have a plan of their own
+            src_off[k] = 0u;
+            src_page[k] = 0;
+            dst_off[k] = 0;
+            continue;
+        }
         int c = (tid & 511) + 512 * k;
         if (kSpreadTail && k == 4) c = 4 * 512 + ((tid & 511) >> 2);
         c = c < kChunksPerTile ? c : kChunksPerTile - 1;
@@ -712,7 +738,6 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     }
 
     __builtin_amdgcn_sched_barrier(0);
-
     const int NS = p.num_splits;
     const bool rowwide = p.max_blocks <= 64 * PVR;
     // every sequence is cut into the same token chunks (those of the longest possible context):
@@ -786,20 +811,26 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 
     const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + int64_t(seq) * p.H_Q * 128;
     uint4v q_pre[2][4];
-    if (p.rotation != nullptr && !copier) {
+    auto load_first_heads = [&]() {
+        if (p.rotation != nullptr && !copier) {
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-            const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
+            for (int rb = 0; rb < 2; ++rb) {
+                const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) q_pre[rb][j] = *reinterpret_cast<const uint4v*>(qseq + row * 128 + 32 * j + 8 * g);
+                for (int j = 0; j < 4; ++j) q_pre[rb][j] = *reinterpret_cast<const uint4v*>(qseq + row * 128 + 32 * j + 8 * g);
+            }
         }
-    }
+    };
+    if constexpr (CW == 0) load_first_heads();
     // Page ids.  When the whole block-table row fits the registers (64 * PVR pages) it is
     // fetched now, before the sequence length is known, so that the two loads overlap;
     // otherwise the registers hold the pages of this split, which depend on the length.
     const int32_t* bt = p.block_table + int64_t(seq) * p.max_blocks;
     int pv[PVR];
-    if (rowwide) {
+#pragma unroll
+    for (int r = 0; r < PVR; ++r) pv[r] = 0;
+    const bool copies = CW == 0 || copier;   // this wavefront moves tiles: it needs the page ids
+    if (rowwide && copies) {
 #pragma unroll
         for (int r = 0; r < PVR; ++r) {
             const int idx = 64 * r + lane < p.max_blocks ? 64 * r + lane : p.max_blocks - 1;
@@ -807,7 +838,17 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         }
     }
 
-    int L = L_known >= 0 ? L_known : p.seq_lens[seq];
+    int L = L_known;
+    if (L_known < 0) L = p.seq_lens[seq];
+    if constexpr (CW > 0) {
+        // The flags are cleared behind a barrier placed where nobody waits for anybody: every
+        // wavefront has just asked for its sequence length and page ids and none has used them yet
+        // (the barrier does not wait for loads from global memory).
+        if (tid == 0) { flags[0] = 0u; flags[1] = 0u; }
+        __syncthreads();
+        load_matrix_columns();
+        load_first_heads();
+    }
     L = L < 0 ? 0 : L;
     L = L > p.max_blocks * BS ? p.max_blocks * BS : L;
     const int begin = split * chunk;
@@ -828,7 +869,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 
     // ---- page ids of the split in registers (see the direct kernel) ---------------------
     const int split_p0 = rowwide ? 0 : begin >> BSL;   // page index held by lane 0 of pv[0]
-    if (!rowwide) {
+    if (!rowwide && copies) {
 #pragma unroll
         for (int r = 0; r < PVR; ++r) {
             int idx = split_p0 + 64 * r + lane;
@@ -949,16 +990,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             for (int k = 0; k < NR; ++k) ra[k] = rb[k] = uint4v{0u, 0u, 0u, 0u};
             c_issue(ra, begin);
             c_issue(rb, begin + 32);
+            // The query exchange of the computing wavefronts goes through the second slot and, with a
+            // sketch, the first: that one is free when all eight have read their sketched heads back.
             if constexpr (PROD) {
-                // the sketched query passes through the first slot: two barriers, then the tile
-                if (p.rotation != nullptr) { __syncthreads(); __syncthreads(); }
-                c_write(0, ra);
-                c_issue(ra, begin + 64);
-            } else {
-                c_write(0, ra);                       // the first slot is not part of the query exchange
-                c_issue(ra, begin + 64);
-                if (p.rotation != nullptr) __syncthreads();   // the barrier of the query exchange
+                if (p.rotation != nullptr) lds_flag_wait(&flags[1], 8u);
             }
+            c_write(0, ra);
+            c_issue(ra, begin + 64);
             for (int t0 = begin; t0 < end; t0 += 64) {
                 __syncthreads();                      // tile i is in LDS; the slot of tile i - 1 is free
                 c_write(1, rb);                       // tile i + 1
@@ -1042,7 +1080,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                     }
                 }
             }
-            __syncthreads();
+            if constexpr (CW > 0) {
+                lds_flag_signal(&flags[0], lane);
+                lds_flag_wait(&flags[0], 8u);
+            } else {
+                __syncthreads();
+            }
             const uint16_t* src = qs + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -1077,7 +1120,10 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
                     for (int e = 0; e < 8; ++e) qsh[ks][e] = _Float16(qf2[ks][e] * down2);
             }
-            if constexpr (PROD) __syncthreads();   // the first slot is about to receive a tile
+            if constexpr (PROD) {                  // the first slot is about to receive a tile
+                if constexpr (CW > 0) lds_flag_signal(&flags[1], lane);
+                else __syncthreads();
+            }
         } else {
             const uint16_t* qsrc = qseq + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
