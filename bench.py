@@ -383,7 +383,7 @@ def main():
             # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a plain copy
             # (profiles/paged_decode_hbm_traffic_pmc.txt); a measured constant, not read live
             "traffic": 148.0e6,
-            "kernel": "paged_decode_staged_kernel<4,4,bf16,4,false>",
+            "kernel": "paged_decode_staged_kernel<4,4,bf16,4,false,4>",
         },
         "cpu_baseline": cpu,
         "extra": extra,
