@@ -8,10 +8,10 @@
 // Launches on the caller's stream:
 //   rotate_q_kernel              q_rot = (q @ R^T) rounded to the query dtype; only for
 //                                shapes whose decode kernel does not rotate the query itself
-//   paged_decode_staged_kernel   8 KV heads of 128 coordinates: one workgroup of 8 wavefronts
-//                                per (split, sequence) copies whole token rows to LDS and
-//                                wavefront h works on KV head h; rotates the query in its
-//                                prologue; also serves TurboQuantProd pages
+//   paged_decode_staged_kernel   8 KV heads of 128 coordinates: one workgroup per (split,
+//                                sequence); 4 wavefronts copy whole token rows to LDS and
+//                                wavefront h of 8 more works on KV head h; rotates the query
+//                                in its prologue; also serves TurboQuantProd pages
 //   paged_decode_kernel          every other shape: one wavefront per (split, sequence, KV
 //                                head), operands read straight from global memory
 //   reduce_rotate_kernel         log-sum-exp combine of the split partials (m, l, acc[D]),
@@ -248,10 +248,10 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 #pragma unroll
         for (int blk = 0; blk < 4; ++blk) {
             const uint8_t* src = (k_hi ? hi[blk] : lo[blk]) + k_off;
-            if (KW == 4) {
+            if constexpr (KW == 4) {
                 const uint4v w = *reinterpret_cast<const uint4v*>(src);
                 t.k[blk][0] = w.x; t.k[blk][1] = w.y; t.k[blk][2] = w.z; t.k[blk][3] = w.w;
-            } else if (KW == 2) {
+            } else if constexpr (KW == 2) {
                 const uint2v w = *reinterpret_cast<const uint2v*>(src);
                 t.k[blk][0] = w.x; t.k[blk][1] = w.y;
             } else {
@@ -504,9 +504,9 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 // The direct kernel above lets every wavefront fetch its own head's bytes, which are
 // 64-byte halves of cache lines it shares with the neighbouring head and 4-byte norms
 // inside 32-byte strips shared by all heads: the vector L1 then spends its time on
-// requests for lines that are already in flight.  Here the workgroup (8 wavefronts, one
-// per KV head) copies whole token rows: thread t moves the 16-byte chunks t, t + 512, ...
-// of a 32-token tile, so every wavefront request covers eight complete cache lines and
+// requests for lines that are already in flight.  Here the workgroup (8 computing
+// wavefronts, one per KV head) copies whole token rows: a copying thread t of T moves the
+// 16-byte chunks t, t + T, ... of a 32-token tile, so every wavefront request covers eight complete cache lines and
 // each line is asked for exactly once.  The chunks land in LDS in a swizzled layout from
 // which the wavefronts read their MFMA operands without bank conflicts:
 //
@@ -518,9 +518,13 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 // the banks; the eight rows read together by a K operand load fall in eight different
 // 16-byte bank groups; the eight chunks a quarter-wave writes together do too).
 //
-// Pipeline, one workgroup barrier per tile: at iteration i the registers holding tile
-// i + 1 (loaded during iteration i - 1) are written to the LDS slot that tile i - 1 has
-// just vacated, the loads of tile i + 2 are issued, and tile i is consumed from LDS.
+// Pipeline, one workgroup barrier per tile.  With copy wavefronts (CW = 4, the default) four
+// more wavefronts do nothing but move tiles: each keeps two tiles in flight in registers and
+// writes tile i + 1 to the LDS slot that tile i - 1 has just left, while the eight computing
+// wavefronts consume tile i and never wait for global memory.  Without them (CW = 0) the eight
+// wavefronts do both: at iteration i the registers holding tile i + 1 (loaded during
+// iteration i - 1) are written to the free slot, the loads of tile i + 2 are issued, and tile
+// i is consumed from LDS.
 // A tile is 32 tokens: two 16-token blocks; with 4 query heads per KV head the 16 MFMA
 // columns carry (head, block, half of the block's rows), so that all lanes own distinct
 // (head, token) scores.
@@ -621,7 +625,6 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     constexpr int KS = 4;                 // k-steps of the score product
     constexpr int DPL = 8;                // V coordinates per lane
     constexpr int NSC = GP / 2;           // scores per lane per tile
-    constexpr int H = 8;
     constexpr int ROWB = Cfg::ROWB;       // 1088, or 1120 with residual norms
     constexpr int PPT = BS >= 32 ? 1 : 32 / BS;   // pages per tile
 
