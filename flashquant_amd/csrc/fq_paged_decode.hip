@@ -1331,10 +1331,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             compute_tile(t0, i & 1);
         }
     } else {
-        int i = 0;
-        for (int t0 = begin; t0 < end; t0 += 32, ++i) {
+        // two tiles per trip, so that the slot is a constant and folds into the offsets of the LDS reads
+        for (int t0 = begin; t0 < end; t0 += 64) {
             __syncthreads();                      // the copy wavefronts have put tile i in LDS
-            compute_tile(t0, i & 1);
+            compute_tile(t0, 0);
+            if (t0 + 32 >= end) break;
+            __syncthreads();
+            compute_tile(t0 + 32, 1);
         }
     }
 
@@ -1435,14 +1438,39 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
         const int64_t row = row0 + r < rows ? row0 + r : rows - 1;
         const int64_t base = row * NS;
         float mstar = -__builtin_inff();
+        // bit c: the chunk of eight splits c (mod 64) holds a split that wrote something.  Splits
+        // beyond a sequence's length are empty (m = -inf), whole chunks of them when the split count
+        // was chosen for the longest possible context: those are not read at all.
+        uint64_t live_chunks = ~0ull;
         if (NS > 8) {
-            for (int s0 = 0; s0 < NS; s0 += 8) {
-                float mv[8];
+            // the 16 threads of a row share the maxima: thread t reads those of splits t, t + 16, ...,
+            // four at a time, so that up to 64 splits cost one round trip
+            const int t16 = threadIdx.x & 15;
+            uint32_t live_lo = 0u, live_hi = 0u;
+            for (int s0 = 0; s0 < NS; s0 += 64) {
+                float mv[4];
 #pragma unroll
-                for (int k = 0; k < 8; ++k) mv[k] = part_m[base + (s0 + k < NS ? s0 + k : NS - 1)];
+                for (int k = 0; k < 4; ++k) {
+                    const int idx = s0 + t16 + 16 * k;
+                    mv[k] = part_m[base + (idx < NS ? idx : NS - 1)];
+                }
 #pragma unroll
-                for (int k = 0; k < 8; ++k) mstar = __builtin_fmaxf(mstar, mv[k]);
+                for (int k = 0; k < 4; ++k) {
+                    const int idx = s0 + t16 + 16 * k;
+                    const bool wrote = idx < NS && mv[k] != -__builtin_inff();
+                    mstar = wrote ? __builtin_fmaxf(mstar, mv[k]) : mstar;
+                    const int chunk = (idx >> 3) & 63;
+                    live_lo |= (wrote && chunk < 32) ? 1u << chunk : 0u;
+                    live_hi |= (wrote && chunk >= 32) ? 1u << (chunk - 32) : 0u;
+                }
             }
+#pragma unroll
+            for (int mask = 1; mask < 16; mask <<= 1) {
+                mstar = __builtin_fmaxf(mstar, xor_shuffle(mstar, mask));
+                live_lo |= uint32_t(__shfl_xor(int(live_lo), mask, kWave));
+                live_hi |= uint32_t(__shfl_xor(int(live_hi), mask, kWave));
+            }
+            live_chunks = (uint64_t(live_hi) << 32) | live_lo;
         }
         for (int c0 = 8 * (threadIdx.x & 15); c0 < D; c0 += 128) {
             float num[8];
@@ -1450,6 +1478,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
             for (int e = 0; e < 8; ++e) num[e] = 0.0f;
             float den = 0.0f;
             for (int s0 = 0; s0 < NS; s0 += 8) {
+                if (!((live_chunks >> ((s0 >> 3) & 63)) & 1ull)) continue;
                 float mv[8], lv[8];
                 float4v lo[8], hi[8];
 #pragma unroll
