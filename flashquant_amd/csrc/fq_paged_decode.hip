@@ -1331,13 +1331,10 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             compute_tile(t0, i & 1);
         }
     } else {
-        // two tiles per trip, so that the slot is a constant and folds into the offsets of the LDS reads
-        for (int t0 = begin; t0 < end; t0 += 64) {
+        int i = 0;
+        for (int t0 = begin; t0 < end; t0 += 32, ++i) {
             __syncthreads();                      // the copy wavefronts have put tile i in LDS
-            compute_tile(t0, 0);
-            if (t0 + 32 >= end) break;
-            __syncthreads();
-            compute_tile(t0 + 32, 1);
+            compute_tile(t0, i & 1);
         }
     }
 
