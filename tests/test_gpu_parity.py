@@ -166,6 +166,12 @@ def test_paged_decode_llama8b_heads(num_splits):
     _decode_case([37, 0, 16, 300, 64, 65, 1, 129], hq=32, hkv=8, num_splits=num_splits)
 
 
+@pytest.mark.parametrize("num_splits", [100, 200])
+def test_paged_decode_split_counts_beyond_64(num_splits):
+    """More splits than the combine kernel reads maxima for in one pass, most of them empty."""
+    _decode_case([3300, 100, 0, 2000, 640], hq=32, hkv=8, num_splits=num_splits)
+
+
 @pytest.mark.parametrize("hq,bs", [(32, 16), (64, 8), (128, 32)])
 def test_paged_decode_without_copy_wavefronts(hq, bs, monkeypatch):
     """FQ_DECODE_COPY_WAVES=0: the eight wavefronts of the staged kernel copy and compute in turn."""
