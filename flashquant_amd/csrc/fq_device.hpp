@@ -109,6 +109,17 @@ __device__ __forceinline__ float max_xor32(float v) {
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return __builtin_fmaxf(bits_to_float(r[0]), bits_to_float(r[1]));
 }
+// sum over lanes l and l ^ 16, l and l ^ 32: one cross-lane vector instruction each, no LDS round trip
+__device__ __forceinline__ float sum_xor16(float v) {
+    const uint32_t u = float_to_bits(v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return bits_to_float(r[0]) + bits_to_float(r[1]);
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+    const uint32_t u = float_to_bits(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return bits_to_float(r[0]) + bits_to_float(r[1]);
+}
 // max over all lanes that share lane % GP
 template <int GP>
 __device__ __forceinline__ float max_same_head(float v) {

@@ -1339,15 +1339,18 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     }
 
     // ---- publish the partial of this split (as in the direct kernel) -----------------------------
+    auto sum_xor = [](float v, int mask) {
+        return mask == 16 ? sum_xor16(v) : (mask == 32 ? sum_xor32(v) : v + xor_shuffle(v, mask));
+    };
 #pragma unroll
-    for (int mask = GP; mask < 64; mask <<= 1) lsum += xor_shuffle(lsum, mask);
+    for (int mask = GP; mask < 64; mask <<= 1) lsum = sum_xor(lsum, mask);
 #pragma unroll
     for (int db = 0; db < DPL; ++db)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float v = O[db][i];
 #pragma unroll
-            for (int mask = 4 * GP; mask < 64; mask <<= 1) v += xor_shuffle(v, mask);
+            for (int mask = 4 * GP; mask < 64; mask <<= 1) v = sum_xor(v, mask);
             O[db][i] = v;
         }
     if (g == 0 && n < p.G) {
