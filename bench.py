@@ -33,7 +33,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published peak
 H_Q, H_KV, D, BS = 32, 8, 128, 16
 BATCH, CTX = 32, 4096
+EXTRA_ITERS = 20              # timed calls of every leg other than the headline
 ROW_BYTES = H_KV * (D + 8)
+DOMINANT_KERNEL = "paged_decode_staged_kernel<4,4,bf16,4,false,4>"
 
 
 def log(*a):
@@ -81,15 +83,33 @@ def build_cache(K, book, seed, device):
 
 
 def time_events(fn, iters):
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
+    """Median and mean time of a call in ms, from GPU events recorded on the stream the calls are
+    launched on (torch's current stream) around every call."""
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(iters + 1)]
     torch.cuda.synchronize()
-    start.record()
+    marks[0].record()
     for i in range(iters):
         fn(i)
-    stop.record()
+        marks[i + 1].record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) / iters   # ms per call
+    each = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(iters))
+    median = each[iters // 2] if iters % 2 else 0.5 * (each[iters // 2 - 1] + each[iters // 2])
+    return median, marks[0].elapsed_time(marks[iters]) / iters
+
+
+def committed_traffic(kernel_prefix):
+    """HBM bytes per launch of the dominant kernel as the committed counter summary states them
+    (a line `TRAFFIC_BYTES_PER_LAUNCH <kernel> <bytes>` in profiles/paged_decode_hbm_traffic_pmc.txt,
+    written from the FETCH_SIZE / WRITE_SIZE runs); None when the summary does not cover the kernel."""
+    path = os.path.join(ROOT, "profiles", "paged_decode_hbm_traffic_pmc.txt")
+    try:
+        for ln in open(path):
+            parts = ln.split()
+            if len(parts) == 3 and parts[0] == "TRAFFIC_BYTES_PER_LAUNCH" and parts[1].startswith(kernel_prefix):
+                return float(parts[2])
+    except OSError:
+        pass
+    return None
 
 
 def main():
@@ -116,8 +136,9 @@ def main():
 
     C = load_native()
     dev = torch.device("cuda:0")
-    cent, bnd = O.lloyd_max_gaussian(D, 4)
-    rot = O.haar_orthogonal(D, 42)
+    # the product's own host set-up: codebook solver and seeded rotation of the library
+    cent, bnd = C.codebook.solve_lloyd_max(D, 4)
+    rot = C.haar_orthogonal(D, 42)
     book = (cent.to(dev), bnd.to(dev), rot.to(dev))
     cent_d, _, rot_d = book
     scale = 1.0 / math.sqrt(D)
@@ -145,9 +166,9 @@ def main():
         step(i)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ev_ms = time_events(step, args.steps)
-    step_ms = min(wall_ms, ev_ms) if ev_ms > 0 else wall_ms
-    warm_ms = time_events(lambda i: step(0), args.steps)
+    # the figure reported: the median over the steps of the GPU time of one step
+    step_ms, step_mean_ms = time_events(step, args.steps)
+    warm_ms, _ = time_events(lambda i: step(0), args.steps)
 
     # ---- dominant kernel alone (the split-K decode), cold ----------------------------
     parts = (torch.empty(BATCH, H_Q, n_splits, D, device=dev), torch.empty(BATCH, H_Q, n_splits, device=dev),
@@ -160,7 +181,7 @@ def main():
 
     for i in range(args.warmup):
         decode_only(i)
-    kern_ms = time_events(decode_only, args.steps)
+    _, kern_ms = time_events(decode_only, args.steps)      # average launch duration
     achieved = kv_bytes / (kern_ms * 1e-3) / 1e9
 
     extra = {
@@ -168,6 +189,7 @@ def main():
         "decode_step_us_cold": step_ms * 1e3,
         "decode_step_us_warm": warm_ms * 1e3,
         "decode_step_us_wallclock": wall_ms * 1e3,
+        "decode_step_us_cold_mean": step_mean_ms * 1e3,
         "decode_gbps_warm": kv_bytes / (warm_ms * 1e-3) / 1e9,
         "decode_pct_hbm_peak_cold": 100.0 * kv_bytes / (step_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "decode_kernel_us_cold": kern_ms * 1e3,
@@ -184,19 +206,37 @@ def main():
 
     # ---- CPU baseline: the oracle on the host cores, bounded sample ---------------------
     cpu = None
+    check = None
     if not args.skip_cpu:
         cache_h = caches[0][0].cpu()
         table_h = caches[0][1].cpu()
         q_h = q.cpu()
         lens_h = lens.cpu()
-        done, spent = 0, 0.0
+        # the GPU's result for the same cache, checked row by row against what the oracle computes
+        cache0, table0 = caches[0]
+        got = K.split_k_paged_decode(q, cache0, table0, lens, cent_d, cent_d, rot_d, H_KV, D, BS,
+                                     sm_scale=scale).float().cpu()
+        done, spent, worst = 0, 0.0, 0.0
         while spent < 10.0 and done < 40 * BATCH:      # about 10 s of CPU work, whole sequences
             s_i = done % BATCH
             t1 = time.perf_counter()
-            O.split_k_paged_decode(q_h[s_i:s_i + 1], cache_h, table_h[s_i:s_i + 1], lens_h[s_i:s_i + 1],
-                                   cent, cent, rot, H_KV, D, BS, sm_scale=scale)
+            want = O.split_k_paged_decode(q_h[s_i:s_i + 1], cache_h, table_h[s_i:s_i + 1], lens_h[s_i:s_i + 1],
+                                          cent, cent, rot, H_KV, D, BS, sm_scale=scale)
             spent += time.perf_counter() - t1
             done += 1
+            worst = max(worst, (got[s_i] - want[0].float()).abs().max().item())
+        # the reference's CPU fallback as written, a Python loop over tokens and heads, at a reduced shape
+        lb, ll = 2, 512
+        lens_l = torch.full((lb,), ll, dtype=torch.int32)
+        t1 = time.perf_counter()
+        want_l = O.paged_decode_loop(torch.matmul(q_h[:lb].float(), rot.T).to(q_h.dtype), cache_h, table_h[:lb], lens_l,
+                                     cent, cent, H_KV, D, BS, sm_scale=scale)
+        loop_s = time.perf_counter() - t1
+        # rotated-space output of a pre-rotated query: what the loop form of the reference returns
+        q_rot_d = torch.matmul(q[:lb].float(), rot_d.T).to(q.dtype)
+        got_l = C.fused_paged_tq4_decode(q_rot_d, cache0, table0[:lb].contiguous(), lens_l.to(dev), cent_d, cent_d,
+                                         None, H_KV, D, BS, sm_scale=scale).float().cpu()
+        worst_l = (got_l - want_l.float()).abs().max().item()
         cpu = {
             "value": done * CTX * ROW_BYTES / spent / 1e9,
             "unit": "GB/s",
@@ -204,6 +244,15 @@ def main():
             "kind": "port",
             "sample": f"{done} sequence decodes ({done / BATCH:.1f} batches) of the same workload with the oracle "
                       f"(vectorised-gather form of the reference's CPU fallback), {spent:.1f} s",
+            "loop_form": {
+                "value": lb * ll * ROW_BYTES / loop_s / 1e9,
+                "unit": "GB/s",
+                "sample": f"the reference's token-by-token Python loop at batch {lb} x {ll} tokens, {loop_s:.1f} s",
+            },
+        }
+        check = {
+            "max_abs_err": worst, "sequences_checked": min(done, BATCH), "tolerance": 2e-2,
+            "loop_form_max_abs_err": worst_l, "ok": bool(worst <= 2e-2 and worst_l <= 2e-2),
         }
         del cache_h
 
@@ -215,13 +264,13 @@ def main():
         x = outlier_rows(rows_tok, H_KV, D, 1001, dev)
         packed = torch.empty(rows_tok, H_KV, D // 2, dtype=torch.uint8, device=dev)
         norms = torch.empty(rows_tok, H_KV, 1, device=dev)
-        ev, od = O.split_rotation(rot)
+        ev, od = C.split_rotation(rot)
         ev, od = ev.to(dev), od.to(dev)
         bnd_d = book[1]
         for _ in range(2):
             K.tq4_compress(x, rot_d, bnd_d, rotation_T_even=ev, rotation_T_odd=od, out=(packed, norms))
-        c_ms = time_events(lambda i: K.tq4_compress(x, rot_d, bnd_d, rotation_T_even=ev, rotation_T_odd=od,
-                                                    out=(packed, norms)), 5)
+        c_ms, _ = time_events(lambda i: K.tq4_compress(x, rot_d, bnd_d, rotation_T_even=ev, rotation_T_odd=od,
+                                                       out=(packed, norms)), EXTRA_ITERS)
         nrows = rows_tok * H_KV
         extra.update({
             "compress_rows": nrows,
@@ -238,7 +287,7 @@ def main():
         y = torch.empty(rows_tok, H_KV, D, dtype=torch.bfloat16, device=dev)
         for _ in range(2):
             K.tq4_decompress(packed, norms, cent_d, torch.bfloat16, out=y)
-        d_ms = time_events(lambda i: K.tq4_decompress(packed, norms, cent_d, torch.bfloat16, out=y), 5)
+        d_ms, _ = time_events(lambda i: K.tq4_decompress(packed, norms, cent_d, torch.bfloat16, out=y), EXTRA_ITERS)
         extra.update({
             "decompress_ms": d_ms,
             "decompress_gbps": nrows * 324 / (d_ms * 1e-3) / 1e9,
@@ -272,8 +321,8 @@ def main():
         kp3, kn3, vp3, vn3 = (to_bhnd(t) for t in (kp3, kn3, vp3, vn3))
         for _ in range(2):
             K.fused_tq_attention(q3, kp3, kn3, vp3, vn3, cent_d, cent_d, rot_d, sm_scale=scale, is_causal=True)
-        p_ms = time_events(lambda i: K.fused_tq_attention(q3, kp3, kn3, vp3, vn3, cent_d, cent_d, rot_d,
-                                                          sm_scale=scale, is_causal=True), 5)
+        p_ms, _ = time_events(lambda i: K.fused_tq_attention(q3, kp3, kn3, vp3, vn3, cent_d, cent_d, rot_d,
+                                                             sm_scale=scale, is_causal=True), EXTRA_ITERS)
         p_flops = 4.0 * pn * pn * D * pb * H_Q / 2.0               # causal half of QK^T and PV
         extra.update({
             "prefill_ms": p_ms,
@@ -292,7 +341,7 @@ def main():
 
         for i in range(2):
             paged_prefill_step(i)
-        pp_ms = time_events(paged_prefill_step, 5)
+        pp_ms, _ = time_events(paged_prefill_step, EXTRA_ITERS)
         extra.update({
             "paged_prefill_ms": pp_ms,
             "paged_prefill_tflops": p_flops / (pp_ms * 1e-3) / 1e12,
@@ -304,8 +353,8 @@ def main():
         # ---- long-context decode over TurboQuantProd key / TQ4 value pages (configs[4]) ----------
         # batch 8, 64 query heads over 8, ragged contexts U{16K..128K} (seed 1004), 16-token pages
         hq4, b4 = 64, 8
-        c3, b3 = O.lloyd_max_gaussian(D, 3)
-        sk = O.qjl_matrix(D, 42)
+        c3, b3 = C.codebook.solve_lloyd_max(D, 3)
+        sk = C.qjl_matrix(D, 42)
         c3_d, b3_d, sk_d = c3.to(dev), b3.to(dev), sk.to(dev)
         g4 = torch.Generator(device="cpu").manual_seed(1004)
         lens4 = torch.randint(16384, 131072 + 1, (b4,), generator=g4)
@@ -342,7 +391,7 @@ def main():
 
         for i in range(3):
             prod_step(i)
-        pd_ms = time_events(prod_step, 10)
+        pd_ms, _ = time_events(prod_step, EXTRA_ITERS)
         prod_bytes = int(lens4.sum()) * row4
         extra.update({
             "prod_decode_ms": pd_ms,
@@ -380,12 +429,13 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a plain copy
-            # (profiles/paged_decode_hbm_traffic_pmc.txt); a measured constant, not read live
-            "traffic": 148.0e6,
-            "kernel": "paged_decode_staged_kernel<4,4,bf16,4,false,4>",
+            # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a plain copy, as the
+            # committed counter summary states them for this kernel (null when it does not cover it)
+            "traffic": committed_traffic(DOMINANT_KERNEL),
+            "kernel": DOMINANT_KERNEL,
         },
         "cpu_baseline": cpu,
+        "check": check,
         "extra": extra,
     }
     print(json.dumps(line), flush=True)

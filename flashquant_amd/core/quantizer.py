@@ -57,13 +57,13 @@ class TurboQuantMSE:
         """``(indices int64 (..., dim), norms float32 (..., 1))``."""
         require_gpu(x, "x")
         rot, bnd, _ = self._device_state(x.device)
-        return native().quantize(x, rot, bnd, self.bits)
+        return native().mse_quantize(x, rot, bnd, self.bits)
 
     def dequantize(self, indices: torch.Tensor, norms: torch.Tensor) -> torch.Tensor:
         """float32 (..., dim) in the original space."""
         require_gpu(indices, "indices")
         rot, _, cen = self._device_state(indices.device)
-        return native().dequantize(indices, norms, rot, cen)
+        return native().mse_dequantize(indices, norms, rot, cen)
 
 
 class TurboQuantProd:

@@ -44,6 +44,13 @@ RotationArg rotation_arg(const at::Tensor& rotation, const c10::Device& dev, int
     return r;
 }
 
+int option_id(const std::string& name) {
+    if (name == "decode_copy_waves") return FQ_OPT_DECODE_COPY_WAVES;
+    if (name == "decode_direct") return FQ_OPT_DECODE_DIRECT;
+    if (name == "attention_any_dim") return FQ_OPT_ATTENTION_ANY_DIM;
+    throw std::invalid_argument("unknown option '" + name + "'");
+}
+
 using OptPair = std::optional<std::tuple<at::Tensor, at::Tensor>>;
 
 std::tuple<at::Tensor, at::Tensor> tq4_compress(const at::Tensor& x, const at::Tensor& rot_T_even,
@@ -593,8 +600,9 @@ void bind_kernels(py::module_& m) {
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),
           py::arg("out") = py::none(), py::arg("num_splits") = 0,
           "Split-K paged decode over TurboQuantProd key / TQ4 value pages");
-    m.def("nibble_pack", &nibble_pack, py::arg("indices"), "Pack pairs of 4-bit indices (..., D) into bytes (..., D/2)");
-    m.def("nibble_unpack", &nibble_unpack, py::arg("packed"), "Unpack bytes (..., D/2) into int64 indices (..., D)");
+    // nibble_pack / nibble_unpack live in the sub-module only: as top-level names the reference's
+    // packing functions would call them with CPU tensors and no device test
+    // (src/flashquant/core/packing.py:37, 75, 94), and these are GPU kernels.
     {
         py::module_ pk = m.def_submodule("packing", "Index packing on the GPU");
         pk.def("nibble_pack", &nibble_pack, py::arg("indices"));
@@ -603,6 +611,19 @@ void bind_kernels(py::module_& m) {
         pk.def("unpack_2bit", &unpack_2bit, py::arg("packed"), "Inverse of pack_2bit, int64");
         pk.def("validate_indices", &validate_indices, py::arg("indices"), py::arg("bits"));
     }
+    m.def("set_option", [](const std::string& name, bool value) {
+              const int id = option_id(name);
+              const int before = fq_get_option(id);
+              fqbind::raise_on_error(fq_set_option(id, value ? 1 : 0), "set_option");
+              return before != 0;
+          }, py::arg("name"), py::arg("value"),
+          "Set a kernel-variant switch ('decode_copy_waves', 'decode_direct', 'attention_any_dim'); returns the old value");
+    m.def("get_option", [](const std::string& name) { return fq_get_option(option_id(name)) != 0; }, py::arg("name"));
+    m.def("paged_decode_fault_count", []() {
+              unsigned int n = 0;
+              fqbind::raise_on_error(fq_paged_decode_fault_count(&n), "paged_decode_fault_count");
+              return n;
+          }, "Timed-out wavefront hand-offs of the staged decode kernel on the current device (synchronises)");
     m.def("rotate_query", &rotate_query, py::arg("q"), py::arg("rotation"),
           "q_rot = (q @ rotation.T) rounded to q's dtype.");
     m.def("paged_tq4_decode_partials", &paged_tq4_decode_partials, py::arg("q_rot"), py::arg("kv_cache"),

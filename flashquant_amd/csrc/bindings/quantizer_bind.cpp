@@ -198,9 +198,12 @@ void bind_quantizer(py::module_& m) {
     m.def("qjl_matrix", &qjl_matrix, py::arg("dim"), py::arg("seed") = 42, py::arg("qjl_dim") = py::none(),
           "Seeded Gaussian sketch / sqrt(qjl_dim), float32 (qjl_dim, dim) on the CPU");
     m.def("split_rotation", &split_rotation, py::arg("rotation"), "(rotation.T[:, 0::2], rotation.T[:, 1::2]) contiguous");
-    m.def("quantize", &quantize, py::arg("x"), py::arg("rotation"), py::arg("boundaries"), py::arg("bits") = 0,
+    // Not exported as `quantize` / `dequantize`: the reference's quantizer classes call those two
+    // names with CPU tensors and no device test once they exist
+    // (src/flashquant/core/quantizer.py:140-143, 176-179), and these operators are GPU kernels.
+    m.def("mse_quantize", &quantize, py::arg("x"), py::arg("rotation"), py::arg("boundaries"), py::arg("bits") = 0,
           "TurboQuantMSE.quantize on the GPU: (indices int64 (..., D), norms float32 (..., 1))");
-    m.def("dequantize", &dequantize, py::arg("indices"), py::arg("norms"), py::arg("rotation"), py::arg("centroids"),
+    m.def("mse_dequantize", &dequantize, py::arg("indices"), py::arg("norms"), py::arg("rotation"), py::arg("centroids"),
           "TurboQuantMSE.dequantize on the GPU: float32 (..., D) in the original space");
     m.def("mse_residual", &mse_residual, py::arg("x"), py::arg("indices"), py::arg("norms"), py::arg("rotation"),
           py::arg("centroids"), "(x - dequantize(indices, norms), its row norms)");

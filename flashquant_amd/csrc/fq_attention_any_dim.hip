@@ -60,6 +60,9 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
     constexpr int CPT = D / 8;          // coordinates per thread in the dequantisation (8 threads per token)
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ _Float16 cent_k[16], cent_v[16];
+    // A row whose norm lies above 2^15 is stored divided by 2^excess (its products with a centroid
+    // then fit fp16); the power of two goes back in on the float32 score (K) or weight (V).
+    __shared__ int k_exc[32], v_exc[32];
     _Float16* ks = reinterpret_cast<_Float16*>(smem);
     _Float16* vt = reinterpret_cast<_Float16*>(smem + C::K_BYTES);
     _Float16* ps = reinterpret_cast<_Float16*>(smem + C::K_BYTES + C::V_BYTES);
@@ -178,6 +181,10 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
                 nv = p.v_norms[kv_row0 + tok];
             }
             if (!live) { nk = 0.0f; nv = 0.0f; }
+            const int ek = norm_excess(nk), ev = norm_excess(nv);
+            nk = __builtin_ldexpf(nk, -ek);
+            nv = __builtin_ldexpf(nv, -ev);
+            if (part == 0) { k_exc[tok_d] = ek; v_exc[tok_d] = ev; }
 #pragma unroll
             for (int c = 0; c < CPT / 8; ++c) {       // 4 bytes = 8 coordinates at a time
                 const int byte0 = part * (CPT / 2) + 4 * c;
@@ -210,6 +217,7 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
         }
         // lane (n16, g4): rows 4 g4 + i, tokens t0 + n16 and t0 + 16 + n16
         float pv[2][4];
+        const int kx[2] = {k_exc[n16], k_exc[16 + n16]}, vx[2] = {v_exc[n16], v_exc[16 + n16]};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int qpos = qoff + pos0 + 4 * g4 + i;
@@ -219,8 +227,9 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
             for (int tb = 0; tb < 2; ++tb) {
                 const int tok = t0 + 16 * tb + n16;
                 const bool ok = tok < NKV && (!p.causal || tok <= qpos);
-                sc[tb] = ok ? s[tb][i] * qscale : -__builtin_inff();
-                mx = __builtin_fmaxf(mx, sc[tb]);
+                sc[tb] = ok ? __builtin_ldexpf(s[tb][i] * qscale, kx[tb]) : -__builtin_inff();
+                // the reference is taken over score + value excess: weight * 2^excess then stays <= 1
+                mx = __builtin_fmaxf(mx, sc[tb] + float(vx[tb]));
             }
             mx = row16_max(mx);
             const float m_new = __builtin_fmaxf(m_run[i], mx);
@@ -241,7 +250,8 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pw[(4 * g4 + i) * C::VSTRIDE + 16 * tb + n16] = _Float16(pv[tb][i]);
+            for (int i = 0; i < 4; ++i)
+                pw[(4 * g4 + i) * C::VSTRIDE + 16 * tb + n16] = _Float16(__builtin_ldexpf(pv[tb][i], vx[tb]));
         const half8 pa = *reinterpret_cast<const half8*>(pw + n16 * C::VSTRIDE + 8 * g4);
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
@@ -316,8 +326,5 @@ int launch_attention_any_dim(const AnyDimParams& p, int D, bool paged, int max_q
 }  // namespace fq
 
 namespace fq_host {
-bool force_any_dim_attention() {
-    const char* v = getenv("FQ_ATTENTION_ANY_DIM");
-    return v && v[0] == '1';
-}
+bool force_any_dim_attention() { return option(FQ_OPT_ATTENTION_ANY_DIM) != 0; }
 }

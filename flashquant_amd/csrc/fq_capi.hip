@@ -1,18 +1,52 @@
 // Library identification, status text and per-thread HIP error text of the C ABI.
 
+#include <atomic>
+#include <cstdlib>
+#include <mutex>
 #include <string>
 
 #include "fq_common.hpp"
 
 namespace {
 thread_local std::string g_last_hip_error;
+
+// Kernel-variant switches: each takes its first value from an environment variable, read once
+// per process, and can be changed afterwards with fq_set_option.
+std::atomic<int> g_options[FQ_OPTION_COUNT];
+std::once_flag g_options_once;
+void init_options() {
+    std::call_once(g_options_once, [] {
+        const char* v = std::getenv("FQ_DECODE_COPY_WAVES");
+        g_options[FQ_OPT_DECODE_COPY_WAVES] = (v != nullptr && v[0] == '0') ? 0 : 1;
+        v = std::getenv("FQ_DECODE_DIRECT");
+        g_options[FQ_OPT_DECODE_DIRECT] = (v != nullptr && v[0] == '1') ? 1 : 0;
+        v = std::getenv("FQ_ATTENTION_ANY_DIM");
+        g_options[FQ_OPT_ATTENTION_ANY_DIM] = (v != nullptr && v[0] == '1') ? 1 : 0;
+    });
 }
+}  // namespace
 
 namespace fq_host {
 void note_hip_error(hipError_t e) {
     g_last_hip_error = std::string(hipGetErrorName(e)) + ": " + hipGetErrorString(e);
 }
+int option(int id) {
+    init_options();
+    return g_options[id].load(std::memory_order_relaxed);
+}
 }  // namespace fq_host
+
+extern "C" int fq_get_option(int option) {
+    if (option < 0 || option >= FQ_OPTION_COUNT) return -1;
+    return fq_host::option(option);
+}
+
+extern "C" int fq_set_option(int option, int value) {
+    if (option < 0 || option >= FQ_OPTION_COUNT) return FQ_ERR_BAD_SHAPE;
+    init_options();
+    g_options[option].store(value != 0 ? 1 : 0, std::memory_order_relaxed);
+    return FQ_OK;
+}
 
 extern "C" int fq_abi_version(void) { return FQ_ABI_VERSION; }
 

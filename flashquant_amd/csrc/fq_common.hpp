@@ -23,6 +23,7 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+typedef int int4v __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 
@@ -79,4 +80,7 @@ inline bool supported_dim(int d) { return d == 64 || d == 128 || d == 256; }
 // Raises the dynamic-LDS limit of a kernel function once per (function, device); later calls are a lookup.
 bool lds_limit_raised(const void* kernel, size_t bytes);
 int device_cu_count();
+// Value of a kernel-variant switch (fq_option in fq_hip.h): its environment variable, read once
+// per process, unless fq_set_option has changed it since.
+int option(int id);
 }  // namespace fq_host

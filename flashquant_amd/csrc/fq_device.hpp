@@ -11,8 +11,27 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kLutCopies = 64;                // one copy per lane: entry stride 256 bytes
 constexpr int kLutWords = 256 * kLutCopies;   // per table (64 KB)
 constexpr float kHalfMax = 65504.0f;
+constexpr float kHalfSafe = 60000.0f;         // a P operand above this makes the softmax reference move
+constexpr float kMaxLead = 16.0f;             // so does a score this many binary orders above the reference
 
 __device__ __forceinline__ uint32_t byte_of(uint32_t w, int b) { return (w >> (8 * b)) & 0xffu; }
+
+// Binary orders by which a value norm lies above 2^10 (0 for ordinary norms).  Added to a
+// token's score when the softmax reference is chosen, it keeps weight * norm below 2^11, so the
+// fp16 P operand of the second product cannot overflow whatever the norms are; numerator and
+// denominator share the reference, so the result does not depend on it.
+__device__ __forceinline__ float norm_bias(float vn) {
+    const int ex = int((float_to_bits(vn) >> 23) & 0xffu) - 127;   // floor(log2 vn); Inf / NaN: 128
+    return ex > 10 ? float(ex - 10) : 0.0f;
+}
+
+// Binary orders by which a row norm lies above 2^15 (0 for ordinary norms): a K or V tile holds
+// fp16(centroid * norm / 2^excess), which always fits, and the power of two goes back in on the
+// float32 side (the score, or the weight together with a raised softmax reference).
+__device__ __forceinline__ int norm_excess(float n) {
+    const int ex = int((float_to_bits(n) >> 23) & 0xffu) - 127;
+    return ex > 14 ? ex - 14 : 0;
+}
 
 // LDS byte address of table entry `byte K of w` in the copy of this lane: the entry
 // stride is 256 bytes and lane_off = 4 * lane < 256, so the address is the two bytes

@@ -86,6 +86,12 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     constexpr int D = 128;
     __shared__ __attribute__((aligned(256))) uint32_t lut[256 * 64];
     extern __shared__ __attribute__((aligned(16))) uint8_t bufs[];   // 2 x (K tile | V^T tile)
+    // Rows whose norm times a centroid would not fit fp16 are stored divided by a power of two.
+    // big_tile[buf] = tile + 1 marks a tile that holds such rows; scale_exp[buf] holds the exponents,
+    // K rows 0..63 then V rows 0..63, each tagged with tile + 1 in its upper bits (an entry with
+    // another tag is left over from an earlier tile and reads as 0).
+    __shared__ int big_tile[2];
+    __shared__ __attribute__((aligned(16))) int scale_exp[2][128];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -100,7 +106,9 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const int pair = lin / int(gridDim.x);
     const int b = pair / int(gridDim.y), hkv = pair % int(gridDim.y);
     const int x_in_pair = lin % int(gridDim.x);
-    const bool flip = ((lin / p.round_slots) & 1) != 0;
+    // The direction is a function of the pair alone (the round its first workgroup falls in), so
+    // inside a pair x -> wg is a bijection whatever the grid and the CU count are.
+    const bool flip = (((int64_t(pair) * int64_t(gridDim.x)) / p.round_slots) & 1) != 0;
 
     // ---- this sequence -----------------------------------------------------------------------
     int NQ = p.N_Q, NKV = p.N_KV, qoff = 0;
@@ -141,6 +149,9 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
 
     // ---- tables -----------------------------------------------------------------------------
     fill_pair_tables<8>(lut, p.centroids_k[lane & 15], p.centroids_v[lane & 15], 15, w, lane);
+    // cleared here: the barriers of the query stage order this before the first dequantisation
+    if (tid < 2) big_tile[tid] = 0;
+    if (tid < 256) (&scale_exp[0][0])[tid] = 0;
     const uint8_t* lutb = reinterpret_cast<const uint8_t*>(lut);
     const uint32_t lk = 4u * (lane & 31), lv = 128u + lk;
 
@@ -204,8 +215,21 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             nv1 = vnp[tb];
         }
     };
-    auto dequant = [&](int buf) {
+    auto dequant = [&](int buf, int tile) {
         uint8_t* dst = bufs + buf * kPfBufBytes;
+        if (__any(__builtin_fmaxf(__builtin_fabsf(nk), __builtin_fmaxf(__builtin_fabsf(nv0), __builtin_fabsf(nv1))) >= 32768.0f)) {
+            const int ek = norm_excess(nk), ev0 = norm_excess(nv0), ev1 = norm_excess(nv1);
+            nk = __builtin_ldexpf(nk, -ek);
+            nv0 = __builtin_ldexpf(nv0, -ev0);
+            nv1 = __builtin_ldexpf(nv1, -ev1);
+            const int tag = (tile + 1) << 8;
+            if (gqk == 0) scale_exp[buf][tk] = tag | ek;
+            if (jv == 0) {
+                scale_exp[buf][64 + 2 * tp] = tag | ev0;
+                scale_exp[buf][64 + 2 * tp + 1] = tag | ev1;
+            }
+            if ((ek | ev0 | ev1) != 0) big_tile[buf] = tile + 1;
+        }
         const _Float16 hk = _Float16(nk);
         const half2v nk2 = {hk, hk};
         const uint4v a0 = lookup_word(lutb, kraw.x, lk);   // coordinates 0..7 of the group
@@ -321,6 +345,25 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             }
         }
         const int t0 = tile * 64;
+        // rows stored divided by a power of two (norms beyond fp16's range): wavefront-uniform, rare
+        const bool big = __builtin_amdgcn_readfirstlane(big_tile[buf]) == tile + 1;
+        auto exps_of = [&](int first) {        // the exponents of four consecutive rows of this tile
+            const int4v raw = *reinterpret_cast<const int4v*>(&scale_exp[buf][first]);
+            int4v e;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) e[c] = (raw[c] >> 8) == tile + 1 ? (raw[c] & 0xff) : 0;
+            return e;
+        };
+        if (big) {
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int4v e = exps_of(32 * tb + 8 * q + 4 * hf);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) S[tb][4 * q + c] = __builtin_ldexpf(S[tb][4 * q + c], e[c]);
+                }
+        }
         const bool need_mask = (t0 + 63 >= NKV) || (p.causal && t0 + 63 > qoff + pos0);   // wavefront-uniform
         if (need_mask) {
             int lim = NKV - 1;
@@ -334,15 +377,31 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
                     if (off > lim) S[tb][r] = -__builtin_inff();
                 }
         }
-        float mx = S[0][0];
+        float cand;
+        if (!big) {
+            float mx = S[0][0];
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb)
+            for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, S[tb][r]);
-        mx = max_xor32(mx);
+                for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, S[tb][r]);
+            cand = mx * krow;
+        } else {
+            // a value row stored divided by 2^e gets its weight multiplied by 2^e: the reference is
+            // taken over score + e, so that these weights stay below 16 as well
+            cand = -__builtin_inff();
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int4v e = exps_of(64 + 32 * tb + 8 * q + 4 * hf);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        cand = __builtin_fmaxf(cand, __builtin_fmaf(S[tb][4 * q + c], krow, float(e[c])));
+                }
+        }
+        cand = max_xor32(cand);
         // the running maximum moves only when it would grow by more than 2^4: the weights stay
         // below 16 and the rescale of the 64 accumulator registers becomes rare
-        const float cand = mx * krow;
         const float mnew = cand > m_run + 4.0f ? cand : m_run;
         const float ms = mnew == -__builtin_inff() ? 0.0f : mnew;
         const float alpha = __builtin_amdgcn_exp2f(m_run - ms);
@@ -356,6 +415,14 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             for (int e = 0; e < 8; ++e) {
                 pe[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[s >> 1][8 * (s & 1) + e], krow, -ms));
                 ps += pe[e];
+            }
+            if (big) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int4v ev = exps_of(64 + 32 * (s >> 1) + 8 * (2 * (s & 1) + q) + 4 * hf);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) pe[4 * q + c] = __builtin_ldexpf(pe[4 * q + c], ev[c]);
+                }
             }
             pbv[s] = uint4v{pack_rtz(pe[0], pe[1]), pack_rtz(pe[2], pe[3]), pack_rtz(pe[4], pe[5]), pack_rtz(pe[6], pe[7])};
         }
@@ -377,7 +444,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     };
 
     // ---- tiles ----------------------------------------------------------------------------------------
-    dequant(0);
+    dequant(0, 0);
     issue_loads(1);
     // The dequantisation of tile i + 1 and the products of tile i sit in one basic block (no
     // conditions between them), so that the lookups and LDS writes of the one interleave with
@@ -385,13 +452,13 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     int i = 0;
     for (; i < my_tiles; ++i) {
         __syncthreads();                       // tile i is complete; the other buffer is free
-        dequant((i + 1) & 1);
+        dequant((i + 1) & 1, i + 1);
         issue_loads(i + 2);
         compute(i, i & 1);
     }
     for (; i < ntiles; ++i) {                  // tiles only the other wavefronts of the workgroup need
         __syncthreads();
-        dequant((i + 1) & 1);
+        dequant((i + 1) & 1, i + 1);
         issue_loads(i + 2);
     }
 

@@ -55,8 +55,8 @@
 #include "fq_device.hpp"
 
 namespace fq_host {
-// FQ_DECODE_DIRECT=1 in the environment routes every shape to the direct kernel
-// (both kernels are kept tested).
+// The switch FQ_OPT_DECODE_DIRECT routes every shape to the direct kernel (both kernels are kept
+// tested).
 bool force_direct_decode();
 int device_cu_count();
 }
@@ -369,7 +369,8 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
                 const bool live = tok < end;
                 rv[c][i] = live ? cur.vn[c][i] : 0.0f;
                 a_[c][i] = live ? s_[c][i] * cur.kn[c][i] * qscale : -__builtin_inff();
-                tmax = __builtin_fmaxf(tmax, a_[c][i]);
+                // the bias (0 for ordinary value norms) keeps weight * norm inside fp16
+                tmax = __builtin_fmaxf(tmax, a_[c][i] + norm_bias(rv[c][i]));
             }
         }
         tmax = max_same_head<GP>(tmax);
@@ -606,12 +607,20 @@ __device__ __forceinline__ constexpr int sign_order(int e) {
 __device__ __forceinline__ void lds_flag_signal(uint32_t* flag, int lane) {
     if (lane == 0) __hip_atomic_fetch_add(flag, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
-__device__ __forceinline__ void lds_flag_wait(uint32_t* flag, uint32_t count) {
+// Returns false when the count was not reached within the bound: the caller records the failed
+// hand-off (the workgroup then publishes NaN partials and raises the library's fault counter)
+// instead of going on silently with operands that are not there yet.
+__device__ __forceinline__ bool lds_flag_wait(uint32_t* flag, uint32_t count) {
     for (int spin = 0; spin < (1 << 20); ++spin) {
-        if (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= count) break;
+        if (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= count) return true;
         __builtin_amdgcn_s_sleep(1);
     }
+    return false;
 }
+
+// Hand-offs inside a decode workgroup that ran into their spin bound, since the library was loaded
+// (read with fq_paged_decode_fault_count).
+__device__ unsigned int g_decode_faults = 0u;
 
 template <int BSL, int GP, int DT, int PVR, bool PROD, int CW>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
@@ -632,7 +641,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // that folds into the offset field of every lookup; the tile slots are dynamic.
     __shared__ __attribute__((aligned(256))) uint32_t lut[kLutWords];
     extern __shared__ __attribute__((aligned(16))) uint8_t slots[];   // two tile slots
-    __shared__ uint32_t flags[2];   // CW > 0: rotated heads stored / sketched heads read back
+    __shared__ uint32_t flags[3];   // CW > 0: rotated heads stored / sketched heads read back / a hand-off timed out
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -847,7 +856,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         // The flags are cleared behind a barrier placed where nobody waits for anybody: every
         // wavefront has just asked for its sequence length and page ids and none has used them yet
         // (the barrier does not wait for loads from global memory).
-        if (tid == 0) { flags[0] = 0u; flags[1] = 0u; }
+        if (tid == 0) { flags[0] = 0u; flags[1] = 0u; flags[2] = 0u; }
         __syncthreads();
         load_matrix_columns();
         load_first_heads();
@@ -996,7 +1005,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             // The query exchange of the computing wavefronts goes through the second slot and, with a
             // sketch, the first: that one is free when all eight have read their sketched heads back.
             if constexpr (PROD) {
-                if (p.rotation != nullptr) lds_flag_wait(&flags[1], 8u);
+                if (p.rotation != nullptr && !lds_flag_wait(&flags[1], 8u)) flags[2] = 1u;
             }
             c_write(0, ra);
             c_issue(ra, begin + 64);
@@ -1085,7 +1094,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             }
             if constexpr (CW > 0) {
                 lds_flag_signal(&flags[0], lane);
-                lds_flag_wait(&flags[0], 8u);
+                if (!lds_flag_wait(&flags[0], 8u)) flags[2] = 1u;
             } else {
                 __syncthreads();
             }
@@ -1228,7 +1237,6 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 
         // ---- this lane's scores ------------------------------------------------------------------
         float a_[NSC], rv[NSC];
-        float tmax = -__builtin_inff();
 #pragma unroll
         for (int e = 0; e < NSC; ++e) {
             float s, s2 = 0.0f;
@@ -1253,27 +1261,42 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             float sc = s * kn[e] * qscale;
             if (PROD) sc = __builtin_fmaf(s2 * kg[e], qscale_s, sc);
             a_[e] = live ? sc : -__builtin_inff();
-            tmax = __builtin_fmaxf(tmax, a_[e]);
         }
-        tmax = max_same_head<GP>(tmax);
-        // The running maximum moves only when it would grow by more than 2^4: weights then stay
-        // below 16 (fine in fp16 next to value norms up to 4000), and the rescale of the
-        // accumulators, 32 multiplies, becomes rare.
-        const float Mnew = tmax > M + 4.0f ? tmax : M;
-        const float Ms = Mnew == -__builtin_inff() ? 0.0f : Mnew;
-        const float alpha = __builtin_amdgcn_exp2f(M - Ms);
-        M = Mnew;
+        // Weights relative to the reference M the head already has.  M is not the exact running
+        // maximum: it moves only when a score leads it by more than 2^16 or a weighted value norm
+        // w * |v| would not fit fp16 (the P operand), which one vote over the wavefront finds out.
+        // Any reference gives the same softmax as long as numerator and denominator share it.
         float wv[NSC];
         float psum = 0.0f;
+        bool redo = false;
 #pragma unroll
         for (int e = 0; e < NSC; ++e) {
-            const float w = __builtin_amdgcn_exp2f(a_[e] - Ms);
+            const float d = a_[e] - M;
+            const float w = __builtin_amdgcn_exp2f(d);
             psum += w;
-            wv[e] = __builtin_fminf(w * rv[e], kHalfMax);
+            wv[e] = w * rv[e];
+            redo = redo || d > kMaxLead || wv[e] > kHalfSafe;
         }
-        lsum = __builtin_fmaf(lsum, alpha, psum);
-
-        if (__any(alpha != 1.0f)) {
+        if (__any(redo)) {
+            // The reference moves to max(M, max over the tile of (score + bias)), where the bias of a
+            // token is the number of binary orders its value norm lies above 2^10: weights then stay
+            // below 1 / 2^bias and w * |v| below 2^11 whatever the norms are.
+            float tmax = -__builtin_inff();
+#pragma unroll
+            for (int e = 0; e < NSC; ++e) tmax = __builtin_fmaxf(tmax, a_[e] + norm_bias(rv[e]));
+            tmax = max_same_head<GP>(tmax);
+            const float Mnew = __builtin_fmaxf(M, tmax);
+            const float Ms = Mnew == -__builtin_inff() ? 0.0f : Mnew;
+            const float alpha = __builtin_amdgcn_exp2f(M - Ms);   // M = -inf (first tile): 0
+            M = Mnew;
+            psum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < NSC; ++e) {
+                const float w = __builtin_amdgcn_exp2f(a_[e] - Ms);
+                psum += w;
+                wv[e] = __builtin_fminf(w * rv[e], kHalfMax);     // only a norm of Inf still reaches the bound
+            }
+            lsum *= alpha;
             float ar[4];
             if (GP == 4) {
                 ar[0] = dpp_mov<0x00>(alpha);
@@ -1289,6 +1312,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
                 for (int i = 0; i < 4; ++i) O[db][i] *= ar[i];
         }
+        lsum += psum;
 
         // ---- weights as the A operand: slot j <-> (block j / 4, row 4g + j % 4) -------------------
         // (the weights of this lane are packed once and placed with lane-constant masks)
@@ -1353,6 +1377,14 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             for (int mask = 4 * GP; mask < 64; mask <<= 1) v = sum_xor(v, mask);
             O[db][i] = v;
         }
+    if constexpr (CW > 0) {
+        // a hand-off of the prologue that timed out (the tile barriers since then make the word
+        // visible): the result cannot be trusted, so it is made NaN and the fault is counted
+        if (__builtin_amdgcn_readfirstlane(flags[2]) != 0u) {
+            M = __builtin_nanf("");
+            if (tid == 0) atomicAdd(&g_decode_faults, 1u);
+        }
+    }
     if (g == 0 && n < p.G) {
         const int64_t o = (int64_t(seq) * p.H_Q + hq_lane) * NS + split;
         p.part_m[o] = M;
@@ -1594,12 +1626,9 @@ int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream, in
     return launch_with_lds(kernel, p, dim3(S, p.num_splits, 1), dim3(512 + 64 * copy_waves), lds, stream);
 }
 
-// The staged kernel runs with four more wavefronts that only copy; FQ_DECODE_COPY_WAVES=0
-// selects the form in which the eight wavefronts copy and compute in turn.
-inline int staged_copy_waves() {
-    const char* e = std::getenv("FQ_DECODE_COPY_WAVES");
-    return (e != nullptr && e[0] == '0') ? 0 : 4;
-}
+// The staged kernel runs with four more wavefronts that only copy; the switch
+// FQ_OPT_DECODE_COPY_WAVES = 0 selects the form in which the eight wavefronts copy and compute in turn.
+inline int staged_copy_waves() { return fq_host::option(FQ_OPT_DECODE_COPY_WAVES) != 0 ? 4 : 0; }
 
 // Staged kernel for every page size and group size; PROD selects the TurboQuantProd page format.
 template <int DT, bool PROD>
@@ -1730,10 +1759,7 @@ bool lds_limit_raised(const void* kernel, size_t bytes) {
     done[{kernel, dev}] = bytes;
     return true;
 }
-bool force_direct_decode() {
-    const char* v = getenv("FQ_DECODE_DIRECT");
-    return v && v[0] == '1';
-}
+bool force_direct_decode() { return option(FQ_OPT_DECODE_DIRECT) != 0; }
 }
 
 // A split keeps its page ids in at most 4 registers of 64 lanes: it may span at most
@@ -1837,6 +1863,16 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
 #undef FQ_DECODE_D
 }
 }  // namespace fq
+
+extern "C" int fq_paged_decode_fault_count(unsigned int* count) {
+    if (!count) return FQ_ERR_NULL_POINTER;
+    const hipError_t e = hipMemcpyFromSymbol(count, HIP_SYMBOL(fq::g_decode_faults), sizeof(unsigned int));
+    if (e != hipSuccess) {
+        fq_host::note_hip_error(e);
+        return FQ_ERR_LAUNCH;
+    }
+    return FQ_OK;
+}
 
 extern "C" int fq_paged_decode_fuses_rotation(int D, int H_KV, int shared_codebook) {
     (void)shared_codebook;   // both codebooks fit the kernel's table

@@ -13,13 +13,13 @@ def nibble_pack(indices: torch.Tensor) -> torch.Tensor:
     require_gpu(indices, "indices")
     if indices.shape[-1] % 2 != 0:
         raise ValueError(f"Last dimension must be even for nibble packing, got {indices.shape[-1]}")
-    return native().nibble_pack(indices)
+    return native().packing.nibble_pack(indices)
 
 
 def nibble_unpack(packed: torch.Tensor) -> torch.Tensor:
     """Unpack ``(..., D // 2)`` uint8 into int64 indices ``(..., D)``."""
     require_gpu(packed, "packed")
-    return native().nibble_unpack(packed)
+    return native().packing.nibble_unpack(packed)
 
 
 def pack_2bit(indices: torch.Tensor) -> torch.Tensor:

@@ -43,6 +43,23 @@ typedef enum fq_dtype {
     FQ_F32 = 2
 } fq_dtype;
 
+/*
+ * Kernel-variant switches, for tests and measurements.  Each takes its first value from an
+ * environment variable that is read once per process; fq_set_option changes it afterwards
+ * (value 0 or 1), fq_get_option reads it (-1 for an unknown option).
+ */
+typedef enum fq_option {
+    FQ_OPT_DECODE_COPY_WAVES = 0, /* FQ_DECODE_COPY_WAVES, default 1: the staged decode kernel runs with
+                                     wavefronts that only copy; 0: its computing wavefronts copy too     */
+    FQ_OPT_DECODE_DIRECT = 1,     /* FQ_DECODE_DIRECT, default 0: 1 sends every shape to the direct
+                                     decode kernel                                                      */
+    FQ_OPT_ATTENTION_ANY_DIM = 2, /* FQ_ATTENTION_ANY_DIM, default 0: 1 sends head_dim 128 to the general
+                                     attention kernel                                                   */
+    FQ_OPTION_COUNT = 3
+} fq_option;
+int fq_get_option(int option);
+int fq_set_option(int option, int value);
+
 /* Library identification and error text. */
 int fq_abi_version(void);
 const char* fq_status_string(int status);
@@ -167,7 +184,7 @@ int fq_tq4_decompress(const uint8_t* packed, const float* norms,
  *   is_causal  key j > query i (counted from the top-left corner) is hidden;
  *              ignored when N_Q == 1, as in the reference
  * D in {64, 128, 256}: 128 runs the tuned kernel, 64 and 256 a general one
- * (FQ_ATTENTION_ANY_DIM=1 in the environment sends 128 there too).  H_Q a multiple
+ * (the switch FQ_OPT_ATTENTION_ANY_DIM sends 128 there too).  H_Q a multiple
  * of H_KV; N_KV >= 1.  K and V are dequantised to fp16 with the norm folded in, so a
  * row norm times a centroid must stay below 65504.
  */
@@ -340,6 +357,16 @@ int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* 
                          int num_seqs, int H_Q, int H_KV, int D, int block_size, int max_blocks_per_seq,
                          int64_t num_blocks, float sm_scale, int dtype, int num_splits,
                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The prologue of the staged decode kernel hands the rotated query between wavefronts through
+ * LDS with bounded waits.  A wait that runs into its bound makes the workgroup publish NaN
+ * partials (the output rows of that sequence come out NaN, not silently wrong) and raises a
+ * device-side counter.  This call reads the counter of the current device since the library was
+ * loaded; it synchronises with the device (it is a diagnostic, not part of a launch path).
+ * Returns FQ_OK, or FQ_ERR_LAUNCH if the runtime refuses the copy.
+ */
+int fq_paged_decode_fault_count(unsigned int* count);
 
 /* Number of splits fq_split_k_paged_decode uses when num_splits == 0
  * (counterpart of paged_tq4_decode_num_splits, csrc/cuda/paged_decode.cu:424-426,

@@ -1,0 +1,275 @@
+"""GPU parity at the sizes the benchmark times, and on the magnitudes the reference's
+adversarial tests use (tests/test_adversarial.py:13-152: constant rows of 1e6, one
+coordinate of 1e8 among 1e-8, rows of 1e-30, zero rows), pushed through decode and prefill.
+
+The oracle is the checker.  At full size it is run on the whole problem where that takes
+seconds (paged decode) and on slices where it does not (8192-token prefill: a causal row i
+is the non-causal attention of that row over keys 0..i)."""
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+from oracle import tq_oracle as O
+from tests.conftest import outlier_rows
+from tests.gpu_util import book
+
+pytestmark = pytest.mark.gpu
+
+if torch.cuda.is_available():
+    from flashquant_amd import kernels as K
+
+DEV = "cuda:0"
+
+
+def _store_sequences(lens, kv_rows, hkv, d, bs, seed, extra_blocks=0):
+    """Paged TQ4 cache holding kv_rows(s, L) -> (k, v) float32 (L, hkv, d) for every sequence,
+    compressed by the oracle, behind a seeded random block table."""
+    c, b, r = book(d)
+    g = torch.Generator().manual_seed(seed)
+    S = len(lens)
+    max_blocks = max(1, (max(lens) + bs - 1) // bs)
+    nb = S * max_blocks + extra_blocks
+    cache = torch.zeros(nb, bs, hkv * (d + 8), dtype=torch.uint8)
+    table = torch.randperm(nb, generator=g)[: S * max_blocks].reshape(S, max_blocks).int()
+    for s, L in enumerate(lens):
+        if L == 0:
+            continue
+        k, v = kv_rows(s, L)
+        kp, kn = O.compress(k, r, b)
+        vp, vn = O.compress(v, r, b)
+        t = torch.arange(L)
+        O.store_rows(cache, table[s].long()[t // bs] * bs + t % bs, kp, kn, vp, vn)
+    return cache, table, torch.tensor(lens, dtype=torch.int32)
+
+
+def _scaled_tol(want):
+    return 2e-2 * max(1.0, want.float().abs().max().item())
+
+
+# ---- the benchmark's decode workload, exactly ---------------------------------------------------
+
+def test_paged_decode_at_the_benchmark_size():
+    """Batch 32, 4096 tokens of context each, 32 query heads over 8 KV heads, 16-token pages,
+    N(0,1) rows with four x10 outlier channels per head, block table a seeded permutation."""
+    c, b, r = book(128)
+    B, L, hq, hkv, bs = 32, 4096, 32, 8, 16
+
+    def rows(s, n):
+        return outlier_rows(n, hkv, 128, 5000 + 2 * s), outlier_rows(n, hkv, 128, 5001 + 2 * s)
+
+    cache, table, sl = _store_sequences([L] * B, rows, hkv, 128, bs, seed=2002, extra_blocks=3)
+    q = torch.randn(B, hq, 128, generator=torch.Generator().manual_seed(1002)).to(torch.bfloat16)
+    want = O.split_k_paged_decode(q, cache, table, sl, c, c, r, hkv, 128, bs)
+    cd = c.to(DEV)
+    got = K.split_k_paged_decode(q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), cd, cd, r.to(DEV), hkv, 128, bs)
+    err = (got.cpu().float() - want.float()).abs().max().item()
+    assert math.isfinite(err) and err <= 2e-2, f"max abs error {err}"
+
+
+# ---- the benchmark's prefill workload on slices -------------------------------------------------
+
+def test_fused_prefill_at_the_benchmark_size():
+    """Batch 4, 8192 tokens, 32 query heads over 8 KV heads, causal.  The GPU computes the whole
+    problem; the oracle checks (batch, head, row) samples, among them the first and last rows,
+    both sides of a 64-token tile edge and of the workgroup edges."""
+    c, bnd, r = book(128)
+    B, hq, hkv, N, d = 4, 32, 8, 8192, 128
+    g = torch.Generator().manual_seed(1003)
+    q = torch.randn(B, hq, N, d, generator=g).to(torch.bfloat16)
+    k = outlier_rows(B * hkv * N, 1, d, 6001).reshape(B, hkv, N, d)
+    v = outlier_rows(B * hkv * N, 1, d, 6002).reshape(B, hkv, N, d)
+    kp, kn = O.compress(k.reshape(-1, 1, d), r, bnd)
+    vp, vn = O.compress(v.reshape(-1, 1, d), r, bnd)
+    del k, v
+    kp, vp = kp.reshape(B, hkv, N, d // 2), vp.reshape(B, hkv, N, d // 2)
+    kn, vn = kn.reshape(B, hkv, N, 1), vn.reshape(B, hkv, N, 1)
+    got = K.fused_tq_attention(q.to(DEV), kp.to(DEV), kn.to(DEV), vp.to(DEV), vn.to(DEV), c.to(DEV), c.to(DEV),
+                               r.to(DEV), is_causal=True)
+    torch.cuda.synchronize()
+    got = got.cpu().float()
+    assert torch.isfinite(got).all()
+    rows = [0, 1, 31, 32, 63, 64, 65, 127, 128, 1000, 4095, 4096, 6000, 8127, 8128, 8190, 8191]
+    pairs = [(0, 0), (1, 13), (2, 21), (3, 31), (0, 7), (3, 16)]
+    worst = 0.0
+    for bi, h in pairs:
+        hk = h // (hq // hkv)
+        for i in rows:
+            want = O.fused_tq_attention(q[bi:bi + 1, h:h + 1, i:i + 1], kp[bi:bi + 1, hk:hk + 1, :i + 1],
+                                        kn[bi:bi + 1, hk:hk + 1, :i + 1], vp[bi:bi + 1, hk:hk + 1, :i + 1],
+                                        vn[bi:bi + 1, hk:hk + 1, :i + 1], c, c, r, is_causal=False)
+            err = (got[bi, h, i] - want[0, 0, 0].float()).abs().max().item()
+            worst = max(worst, err)
+            assert err <= _scaled_tol(want), f"batch {bi} head {h} row {i}: max abs error {err}"
+    # a full (batch, head) pair at a quarter of the length would not see the long rows; the last
+    # 64 rows of one pair are compared in full instead
+    bi, h = 2, 5
+    hk = h // (hq // hkv)
+    kd = O.decompress(kp[bi, hk].reshape(-1, 1, d // 2), kn[bi, hk].reshape(-1, 1, 1), c).reshape(N, d)
+    vd = O.decompress(vp[bi, hk].reshape(-1, 1, d // 2), vn[bi, hk].reshape(-1, 1, 1), c).reshape(N, d)
+    q_rot = torch.matmul(q[bi, h, -64:].float(), r.T).to(torch.bfloat16).float()
+    sc = (q_rot @ kd.T) / math.sqrt(d)
+    sc = sc.masked_fill(torch.arange(N)[None, :] > (N - 64 + torch.arange(64))[:, None], float("-inf"))
+    want = torch.matmul(torch.softmax(sc, -1) @ vd, r).to(torch.bfloat16).float()
+    sdpa = torch.nn.functional.scaled_dot_product_attention(
+        q_rot[None], kd[None], vd[None], attn_mask=(sc > float("-inf"))[None])[0]
+    assert (sdpa @ r - want).abs().max() < 2e-2          # the hand-written mask against the library routine
+    assert (got[bi, h, -64:] - want).abs().max().item() <= _scaled_tol(want)
+
+
+# ---- long TurboQuantProd contexts ----------------------------------------------------------------
+
+def test_prod_paged_decode_on_long_ragged_contexts():
+    """Three sequences of the long-context workload's shape (64 query heads over 8 KV heads):
+    16K, 70K and 128K tokens, the lengths at which the page ids of a split no longer fit one
+    register and the chunks are sized inside the kernel."""
+    c3, b3 = O.lloyd_max_gaussian(128, 3)
+    c4, b4 = O.lloyd_max_gaussian(128, 4)
+    r, s = O.haar_orthogonal(128, 42), O.qjl_matrix(128, 42)
+    hq, hkv, d, bs = 64, 8, 128, 16
+    lens = [16384, 70001, 131072]
+    g = torch.Generator().manual_seed(1004)
+    max_blocks = (max(lens) + bs - 1) // bs
+    nb = sum((L + bs - 1) // bs for L in lens) + 5
+    row_bytes = O.prod_page_layout(hkv, d)[4]
+    cache = torch.zeros(nb, bs, row_bytes, dtype=torch.uint8)
+    perm = torch.randperm(nb, generator=g)
+    table = torch.zeros(len(lens), max_blocks, dtype=torch.int32)
+    used = 0
+    for i, L in enumerate(lens):
+        n_pages = (L + bs - 1) // bs
+        table[i, :n_pages] = perm[used:used + n_pages].int()
+        used += n_pages
+        for t0 in range(0, L, 32768):                       # bounded memory on the CPU side
+            n = min(32768, L - t0)
+            kk = torch.randn(n, hkv, d, generator=g)
+            vv = torch.randn(n, hkv, d, generator=g)
+            idx, kn, sg, gam = O.prod_quantize(kk, r, b3, c3, s)
+            vp, vn = O.compress(vv, r, b4)
+            t = torch.arange(t0, t0 + n)
+            O.prod_store_rows(cache, table[i].long()[t // bs] * bs + t % bs, O.prod_pack_keys(idx, sg), kn, gam, vp, vn)
+    q = torch.randn(len(lens), hq, d, generator=g).to(torch.bfloat16)
+    sl = torch.tensor(lens, dtype=torch.int32)
+    want = O.prod_paged_decode(q, cache, table, sl, c3, c4, r, s, hkv, d, bs)
+    got = K.prod_paged_decode(q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), c3.to(DEV), c4.to(DEV), r.to(DEV),
+                              s.to(DEV), hkv, d, bs)
+    torch.cuda.synchronize()
+    err = (got.cpu().float() - want.float()).abs().max().item()
+    assert math.isfinite(err) and err <= 2e-2, f"max abs error {err}"
+
+
+# ---- magnitudes of the reference's adversarial tests, through decode and prefill ------------------
+
+def _adversarial_rows(kind, n, h, d, seed):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "ones_1e6":                       # tests/test_adversarial.py:16-34
+        return torch.ones(n, h, d) * 1e6
+    if kind == "outlier_1e8":                    # :57-78
+        x = torch.full((n, h, d), 1e-8)
+        x[..., 0] = 1e8
+        return x
+    if kind == "tiny_1e-30":                     # :140-152
+        return torch.randn(n, h, d, generator=g) * 1e-30
+    if kind == "zeros":                          # :81-96
+        return torch.zeros(n, h, d)
+    if kind == "scaled_1e4":                     # norms beyond what fp16(norm * centroid) holds
+        return torch.randn(n, h, d, generator=g) * 1e4
+    raise ValueError(kind)
+
+
+def _mixed_kv(n, h, d, seed):
+    """Ordinary rows, one key with a huge norm (it takes all the weight or none) and value rows
+    spread over 20 binary orders."""
+    g = torch.Generator().manual_seed(seed)
+    k = torch.randn(n, h, d, generator=g)
+    v = torch.randn(n, h, d, generator=g)
+    k[n // 3] *= 1e6
+    scale = torch.ones(n)
+    scale[::7] = 3e3
+    scale[5::11] = 1e6
+    v *= scale[:, None, None]
+    return k, v
+
+
+KINDS = ["ones_1e6", "outlier_1e8", "tiny_1e-30", "zeros", "scaled_1e4", "mixed"]
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 128), (8, 2, 64)])
+def test_paged_decode_on_adversarial_magnitudes(kind, hq, hkv, d):
+    c, b, r = book(d)
+    lens = [150, 33, 700]
+
+    def rows(s, n):
+        if kind == "mixed":
+            return _mixed_kv(n, hkv, d, 7000 + s)
+        return _adversarial_rows(kind, n, hkv, d, 7000 + s), _adversarial_rows(kind, n, hkv, d, 7100 + s)
+
+    cache, table, sl = _store_sequences(lens, rows, hkv, d, 16, seed=71, extra_blocks=2)
+    q = torch.randn(len(lens), hq, d, generator=torch.Generator().manual_seed(72)).to(torch.bfloat16)
+    want = O.split_k_paged_decode(q, cache, table, sl, c, c, r, hkv, d, 16)
+    cd = c.to(DEV)
+    for splits in (1, 3):
+        got = K.split_k_paged_decode(q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), cd, cd, r.to(DEV), hkv, d, 16,
+                                     num_splits=splits)
+        assert torch.isfinite(got).all() and torch.isfinite(want.float()).all()
+        # a row's tolerance follows that row's magnitude (value rows span 20 binary orders)
+        row_scale = want.float().abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+        rel = ((got.cpu().float() - want.float()).abs() / row_scale).max().item()
+        assert rel <= 2e-2, f"{kind} splits={splits}: max error {rel} of the row magnitude"
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (4, 2, 64)])
+def test_fused_attention_on_adversarial_magnitudes(kind, hq, hkv, d):
+    c, bnd, r = book(d)
+    B, N = 2, 200
+    if kind == "mixed":
+        _, v = _mixed_kv(B * hkv * N, 1, d, 7300)
+        k = torch.randn(B * hkv * N, 1, d, generator=torch.Generator().manual_seed(7301))
+        for bi in range(B * hkv):                 # one huge key per (batch, head)
+            k[bi * N + 40 + bi] *= 1e6
+    else:
+        k = _adversarial_rows(kind, B * hkv * N, 1, d, 7200)
+        v = _adversarial_rows(kind, B * hkv * N, 1, d, 7201)
+    kp, kn = O.compress(k, r, bnd)
+    vp, vn = O.compress(v, r, bnd)
+    shape_p, shape_n = (B, hkv, N, d // 2), (B, hkv, N, 1)
+    kp, kn, vp, vn = kp.reshape(shape_p), kn.reshape(shape_n), vp.reshape(shape_p), vn.reshape(shape_n)
+    q = torch.randn(B, hq, N, d, generator=torch.Generator().manual_seed(73)).to(torch.bfloat16)
+    for causal in (True, False):
+        want = O.fused_tq_attention(q, kp, kn, vp, vn, c, c, r, is_causal=causal)
+        got = K.fused_tq_attention(q.to(DEV), kp.to(DEV), kn.to(DEV), vp.to(DEV), vn.to(DEV), c.to(DEV), c.to(DEV),
+                                   r.to(DEV), is_causal=causal)
+        torch.cuda.synchronize()
+        assert torch.isfinite(got).all() and torch.isfinite(want.float()).all()
+        # a row's tolerance follows that row's magnitude: rows before the huge value rows stay small
+        row_scale = want.float().abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+        rel = ((got.cpu().float() - want.float()).abs() / row_scale).max().item()
+        assert rel <= 2e-2, f"{kind} causal={causal}: max error {rel} of the row magnitude"
+
+
+@pytest.mark.parametrize("kind", ["ones_1e6", "scaled_1e4", "mixed"])
+def test_paged_prefill_on_adversarial_magnitudes(kind):
+    c, b, r = book(128)
+    hq, hkv, d = 8, 2, 128
+    kv_lens, q_lens = [150, 260], [150, 31]
+
+    def rows(s, n):
+        if kind == "mixed":
+            return _mixed_kv(n, hkv, d, 7400 + s)
+        return _adversarial_rows(kind, n, hkv, d, 7400 + s), _adversarial_rows(kind, n, hkv, d, 7500 + s)
+
+    cache, table, sl = _store_sequences(kv_lens, rows, hkv, d, 16, seed=74, extra_blocks=2)
+    q = torch.randn(sum(q_lens), hq, d, generator=torch.Generator().manual_seed(75)).to(torch.bfloat16)
+    cu = torch.tensor([0, q_lens[0], sum(q_lens)], dtype=torch.int32)
+    want = O.paged_prefill(q, cu, cache, table, sl, c, c, r, hkv, d, 16)
+    got = K.paged_tq4_prefill(q.to(DEV), cu.to(DEV), max(q_lens), cache.to(DEV), table.to(DEV), sl.to(DEV), c.to(DEV),
+                              c.to(DEV), r.to(DEV), hkv, d, 16)
+    torch.cuda.synchronize()
+    assert torch.isfinite(got).all() and torch.isfinite(want.float()).all()
+    row_scale = want.float().abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+    rel = ((got.cpu().float() - want.float()).abs() / row_scale).max().item()
+    assert rel <= 2e-2, f"{kind}: max error {rel} of the row magnitude"

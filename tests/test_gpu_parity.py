@@ -25,6 +25,20 @@ if torch.cuda.is_available():
 DEV = "cuda:0"
 
 
+@pytest.fixture
+def kernel_option():
+    """Sets a kernel-variant switch of the library for one test and restores it afterwards."""
+    C = load_native()
+    changed = []
+
+    def _set(name, value):
+        changed.append((name, C.set_option(name, value)))
+
+    yield _set
+    for name, old in reversed(changed):
+        C.set_option(name, old)
+
+
 def test_native_module_is_loaded():
     C = load_native()
     for name in ("tq4_compress", "tq4_decompress", "split_k_paged_decode", "fused_paged_tq4_decode"):
@@ -173,14 +187,14 @@ def test_paged_decode_split_counts_beyond_64(num_splits):
 
 
 @pytest.mark.parametrize("hq,bs", [(32, 16), (64, 8), (128, 32)])
-def test_paged_decode_without_copy_wavefronts(hq, bs, monkeypatch):
-    """FQ_DECODE_COPY_WAVES=0: the eight wavefronts of the staged kernel copy and compute in turn."""
-    monkeypatch.setenv("FQ_DECODE_COPY_WAVES", "0")
+def test_paged_decode_without_copy_wavefronts(hq, bs, kernel_option):
+    """Switch decode_copy_waves off: the eight wavefronts of the staged kernel copy and compute in turn."""
+    kernel_option("decode_copy_waves", False)
     _decode_case([37, 0, 16, 300, 64, 65, 1, 129], hq=hq, hkv=8, bs=bs, num_splits=3)
 
 
-def test_prod_paged_decode_without_copy_wavefronts(monkeypatch):
-    monkeypatch.setenv("FQ_DECODE_COPY_WAVES", "0")
+def test_prod_paged_decode_without_copy_wavefronts(kernel_option):
+    kernel_option("decode_copy_waves", False)
     _check_prod_decode([300, 1, 77, 0, 129], 32, num_splits=5)
 
 
@@ -342,19 +356,39 @@ def test_fused_attention_other_head_dims(d, dtype, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
-def test_fused_attention_general_kernel_agrees_at_head_dim_128(causal, monkeypatch):
+def test_fused_attention_general_kernel_agrees_at_head_dim_128(causal, kernel_option):
     """The kernel that serves head_dim 64 and 256 also takes 128: against the oracle and against the
     tuned kernel on the same inputs."""
     q, kp, kn, vp, vn, c, r = _prefill_case(2, 8, 2, 200, 200, torch.bfloat16, 83)
     dev = [t.to(DEV) for t in (q, kp, kn, vp, vn, c, r)]
     tuned = K.fused_tq_attention(*dev[:5], dev[5], dev[5], dev[6], is_causal=causal)
-    monkeypatch.setenv("FQ_ATTENTION_ANY_DIM", "1")
+    kernel_option("attention_any_dim", True)
     general = K.fused_tq_attention(*dev[:5], dev[5], dev[5], dev[6], is_causal=causal)
     torch.cuda.synchronize()
     want = O.fused_tq_attention(q, kp, kn, vp, vn, c, c, r, is_causal=causal)
     tol = 2e-2 * max(1.0, want.float().abs().max().item())
     assert (general.cpu().float() - want.float()).abs().max().item() <= tol
     assert (general.float() - tuned.float()).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("b,hq,hkv,n", [(8, 32, 8, 300), (2, 32, 8, 1100), (3, 8, 8, 700)])
+def test_fused_attention_more_workgroups_than_cus(b, hq, hkv, n):
+    """Grids larger than the CU count whose x extent does not divide it: the workgroup order is
+    reversed in alternate rounds over the chip, and every (batch, head, row) must still be written
+    exactly once (every row is compared with the oracle)."""
+    q, kp, kn, vp, vn, c, r = _prefill_case(b, hq, hkv, n, n, torch.bfloat16, 75)
+    want = O.fused_tq_attention(q, kp, kn, vp, vn, c, c, r, is_causal=True)
+    got = K.fused_tq_attention(q.to(DEV), kp.to(DEV), kn.to(DEV), vp.to(DEV), vn.to(DEV), c.to(DEV), c.to(DEV),
+                               r.to(DEV), is_causal=True)
+    torch.cuda.synchronize()
+    err = (got.cpu().float() - want.float()).abs()
+    assert torch.isfinite(err).all()
+    assert err.max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
+
+
+def test_paged_prefill_more_workgroups_than_cus():
+    _check_paged_prefill([300, 17, 290, 300, 1, 250, 300, 299, 64, 300], [300, 500, 290, 333, 100, 250, 300, 299, 64, 301],
+                         hq=32, hkv=8)
 
 
 def test_fused_attention_rejects_bad_arguments():
@@ -435,8 +469,8 @@ def test_paged_prefill_other_head_dims(d, dtype):
     _check_paged_prefill([50, 3], [77, 0], hq=4, hkv=4, d=d, dtype=dtype, bs=8, causal=False)
 
 
-def test_paged_prefill_general_kernel_agrees_at_head_dim_128(monkeypatch):
-    monkeypatch.setenv("FQ_ATTENTION_ANY_DIM", "1")
+def test_paged_prefill_general_kernel_agrees_at_head_dim_128(kernel_option):
+    kernel_option("attention_any_dim", True)
     _check_paged_prefill([7, 64, 1, 130, 32], [45, 64, 300, 131, 500], hq=32, hkv=8)
 
 
@@ -451,6 +485,8 @@ def test_paged_prefill_long_sequence_equals_decode_on_last_token():
     cu = torch.tensor([0, L], dtype=torch.int32, device=DEV)
     dev = [t.to(DEV) for t in (cache, table, sl, c, r)]
     full = K.paged_tq4_prefill(q, cu, L, dev[0], dev[1], dev[2], dev[3], dev[3], dev[4], hkv, 128, bs)
+    want = O.paged_prefill(q.cpu(), cu.cpu(), cache, table, sl, c, c, r, hkv, 128, bs)     # every row, not just the tail
+    assert (full.cpu().float() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
     dec = K.split_k_paged_decode(q[-1:].contiguous(), dev[0], dev[1], dev[2], dev[3], dev[3], dev[4], hkv, 128, bs)
     assert (full[-1:].float() - dec.float()).abs().max().item() <= 2e-2
     # and a chunk of the last 100 tokens reproduces the full prefill's last 100 rows bit for bit

@@ -47,6 +47,24 @@ def test_no_cpu_fallback():
                          torch.float16, None)
 
 
+def test_names_the_reference_calls_with_cpu_tensors_are_not_exported():
+    """The reference's core modules call _C.quantize / dequantize / nibble_pack / nibble_unpack with
+    CPU tensors and no device test as soon as the names exist (src/flashquant/core/quantizer.py:43,
+    140-143, 176-179; core/packing.py:37, 75, 94).  A GPU-only module must therefore not carry them at
+    top level; the kernel operators, which the reference gates on .is_cuda, are there."""
+    C = flashquant_amd.load_native()
+    for name in ("quantize", "dequantize", "nibble_pack", "nibble_unpack"):
+        assert not hasattr(C, name), name
+    for name in ("mse_quantize", "mse_dequantize", "tq4_compress", "tq4_decompress", "fused_tq_attention",
+                 "split_k_paged_decode", "fused_paged_tq4_decode"):
+        assert hasattr(C, name), name
+    for name in ("nibble_pack", "nibble_unpack", "pack_2bit", "unpack_2bit", "validate_indices"):
+        assert hasattr(C.packing, name), name
+    # the one set-up entry the reference calls on the host works on the host
+    c, b = C.codebook.solve_lloyd_max(128, 4)
+    assert c.device.type == "cpu" and c.shape == (16,) and b.shape == (15,)
+
+
 def test_product_does_not_import_the_oracle():
     import os
     root = os.path.dirname(os.path.abspath(flashquant_amd.__file__))
