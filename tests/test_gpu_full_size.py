@@ -65,8 +65,12 @@ def test_paged_decode_at_the_benchmark_size():
     want = O.split_k_paged_decode(q, cache, table, sl, c, c, r, hkv, 128, bs)
     cd = c.to(DEV)
     got = K.split_k_paged_decode(q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), cd, cd, r.to(DEV), hkv, 128, bs)
-    err = (got.cpu().float() - want.float()).abs().max().item()
-    assert math.isfinite(err) and err <= 2e-2, f"max abs error {err}"
+    # the outlier channels make some output rows reach |x| > 4, where one bfloat16 step is 0.03:
+    # 2e-2 of the row's magnitude (never less than 2e-2 absolute)
+    assert torch.isfinite(got).all()
+    row_scale = want.float().abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+    rel = ((got.cpu().float() - want.float()).abs() / row_scale).max().item()
+    assert rel <= 2e-2, f"max error {rel} of the row magnitude"
 
 
 # ---- the benchmark's prefill workload on slices -------------------------------------------------
@@ -174,18 +178,26 @@ def _adversarial_rows(kind, n, h, d, seed):
         return torch.randn(n, h, d, generator=g) * 1e-30
     if kind == "zeros":                          # :81-96
         return torch.zeros(n, h, d)
-    if kind == "scaled_1e4":                     # norms beyond what fp16(norm * centroid) holds
-        return torch.randn(n, h, d, generator=g) * 1e4
+    if kind == "values_1e4":                     # value norms beyond what fp16(norm * centroid) holds
+        return torch.randn(n, h, d, generator=g) * (1e4 if seed % 2 else 1.0)   # odd seeds: the value rows
     raise ValueError(kind)
 
 
-def _mixed_kv(n, h, d, seed):
-    """Ordinary rows, one key with a huge norm (it takes all the weight or none) and value rows
-    spread over 20 binary orders."""
+def _biased_queries(shape, seed):
+    """N(0,1) + 0.5: every query has a clearly positive product with the all-ones direction, so a
+    key of +-1e6 * ones takes all the weight or none whatever the rounding of its 1e7-fold
+    amplified score is (a huge key nearly orthogonal to a query would make the comparison a coin
+    toss: the kernels hold the centroids in fp16)."""
+    return (torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) + 0.5).to(torch.bfloat16)
+
+
+def _mixed_kv(n, h, d, seed, huge_sign=1.0):
+    """Ordinary rows, one key with a huge norm along the all-ones direction (it takes all the
+    weight or none, see _biased_queries) and value rows spread over 20 binary orders."""
     g = torch.Generator().manual_seed(seed)
     k = torch.randn(n, h, d, generator=g)
     v = torch.randn(n, h, d, generator=g)
-    k[n // 3] *= 1e6
+    k[n // 3] = huge_sign * 1e6
     scale = torch.ones(n)
     scale[::7] = 3e3
     scale[5::11] = 1e6
@@ -193,7 +205,7 @@ def _mixed_kv(n, h, d, seed):
     return k, v
 
 
-KINDS = ["ones_1e6", "outlier_1e8", "tiny_1e-30", "zeros", "scaled_1e4", "mixed"]
+KINDS = ["ones_1e6", "outlier_1e8", "tiny_1e-30", "zeros", "values_1e4", "mixed"]
 
 
 @pytest.mark.parametrize("kind", KINDS)
@@ -204,11 +216,11 @@ def test_paged_decode_on_adversarial_magnitudes(kind, hq, hkv, d):
 
     def rows(s, n):
         if kind == "mixed":
-            return _mixed_kv(n, hkv, d, 7000 + s)
-        return _adversarial_rows(kind, n, hkv, d, 7000 + s), _adversarial_rows(kind, n, hkv, d, 7100 + s)
+            return _mixed_kv(n, hkv, d, 7000 + s, huge_sign=-1.0 if s == 1 else 1.0)
+        return _adversarial_rows(kind, n, hkv, d, 7000 + 2 * s), _adversarial_rows(kind, n, hkv, d, 7101 + 2 * s)
 
     cache, table, sl = _store_sequences(lens, rows, hkv, d, 16, seed=71, extra_blocks=2)
-    q = torch.randn(len(lens), hq, d, generator=torch.Generator().manual_seed(72)).to(torch.bfloat16)
+    q = _biased_queries((len(lens), hq, d), 72)
     want = O.split_k_paged_decode(q, cache, table, sl, c, c, r, hkv, d, 16)
     cd = c.to(DEV)
     for splits in (1, 3):
@@ -229,8 +241,8 @@ def test_fused_attention_on_adversarial_magnitudes(kind, hq, hkv, d):
     if kind == "mixed":
         _, v = _mixed_kv(B * hkv * N, 1, d, 7300)
         k = torch.randn(B * hkv * N, 1, d, generator=torch.Generator().manual_seed(7301))
-        for bi in range(B * hkv):                 # one huge key per (batch, head)
-            k[bi * N + 40 + bi] *= 1e6
+        for bi in range(B * hkv):                 # one huge key per (batch, head): it wins in batch 0, loses in batch 1
+            k[bi * N + 40 + bi] = 1e6 if bi < hkv else -1e6
     else:
         k = _adversarial_rows(kind, B * hkv * N, 1, d, 7200)
         v = _adversarial_rows(kind, B * hkv * N, 1, d, 7201)
@@ -238,7 +250,7 @@ def test_fused_attention_on_adversarial_magnitudes(kind, hq, hkv, d):
     vp, vn = O.compress(v, r, bnd)
     shape_p, shape_n = (B, hkv, N, d // 2), (B, hkv, N, 1)
     kp, kn, vp, vn = kp.reshape(shape_p), kn.reshape(shape_n), vp.reshape(shape_p), vn.reshape(shape_n)
-    q = torch.randn(B, hq, N, d, generator=torch.Generator().manual_seed(73)).to(torch.bfloat16)
+    q = _biased_queries((B, hq, N, d), 73)
     for causal in (True, False):
         want = O.fused_tq_attention(q, kp, kn, vp, vn, c, c, r, is_causal=causal)
         got = K.fused_tq_attention(q.to(DEV), kp.to(DEV), kn.to(DEV), vp.to(DEV), vn.to(DEV), c.to(DEV), c.to(DEV),
@@ -251,7 +263,7 @@ def test_fused_attention_on_adversarial_magnitudes(kind, hq, hkv, d):
         assert rel <= 2e-2, f"{kind} causal={causal}: max error {rel} of the row magnitude"
 
 
-@pytest.mark.parametrize("kind", ["ones_1e6", "scaled_1e4", "mixed"])
+@pytest.mark.parametrize("kind", ["ones_1e6", "values_1e4", "mixed"])
 def test_paged_prefill_on_adversarial_magnitudes(kind):
     c, b, r = book(128)
     hq, hkv, d = 8, 2, 128
@@ -259,11 +271,11 @@ def test_paged_prefill_on_adversarial_magnitudes(kind):
 
     def rows(s, n):
         if kind == "mixed":
-            return _mixed_kv(n, hkv, d, 7400 + s)
-        return _adversarial_rows(kind, n, hkv, d, 7400 + s), _adversarial_rows(kind, n, hkv, d, 7500 + s)
+            return _mixed_kv(n, hkv, d, 7400 + s, huge_sign=-1.0 if s == 1 else 1.0)
+        return _adversarial_rows(kind, n, hkv, d, 7400 + 2 * s), _adversarial_rows(kind, n, hkv, d, 7501 + 2 * s)
 
     cache, table, sl = _store_sequences(kv_lens, rows, hkv, d, 16, seed=74, extra_blocks=2)
-    q = torch.randn(sum(q_lens), hq, d, generator=torch.Generator().manual_seed(75)).to(torch.bfloat16)
+    q = _biased_queries((sum(q_lens), hq, d), 75)
     cu = torch.tensor([0, q_lens[0], sum(q_lens)], dtype=torch.int32)
     want = O.paged_prefill(q, cu, cache, table, sl, c, c, r, hkv, d, 16)
     got = K.paged_tq4_prefill(q.to(DEV), cu.to(DEV), max(q_lens), cache.to(DEV), table.to(DEV), sl.to(DEV), c.to(DEV),
