@@ -159,6 +159,52 @@ at::Tensor tq4_decompress(const at::Tensor& packed, const at::Tensor& norms, con
     return result;
 }
 
+// The no-allocation variant: the binding converts and allocates nothing either, so every operand
+// has to be on the GPU and contiguous already.
+at::Tensor split_k_paged_decode_static(const at::Tensor& q, const at::Tensor& kv_cache, const at::Tensor& block_table,
+                                       const at::Tensor& seq_lens, const at::Tensor& centroids_k,
+                                       const at::Tensor& centroids_v, const std::optional<at::Tensor>& rotation,
+                                       int64_t num_kv_heads, int64_t head_dim, int64_t block_size, double sm_scale,
+                                       const at::Tensor& out, int64_t num_splits) {
+    for (const at::Tensor* t : {&q, &kv_cache, &block_table, &seq_lens, &centroids_k, &centroids_v, &out}) {
+        fqbind::require_gpu(*t, "every operand");
+        require(t->is_contiguous(), "every operand must be contiguous");
+    }
+    require(q.dim() == 3 && q.size(2) == head_dim, "q must have shape (num_seqs, H_Q, D)");
+    require(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, "q must be float16 or bfloat16");
+    require(kv_cache.dim() == 3 && kv_cache.scalar_type() == at::kByte && kv_cache.size(1) == block_size &&
+                kv_cache.size(2) == num_kv_heads * (head_dim + 8),
+            "kv_cache must be uint8 of shape (num_blocks, block_size, num_kv_heads * (head_dim + 8))");
+    require(block_table.dim() == 2 && block_table.scalar_type() == at::kInt && block_table.size(0) == q.size(0),
+            "block_table must be int32 of shape (num_seqs, max_blocks)");
+    require(seq_lens.scalar_type() == at::kInt && seq_lens.numel() == q.size(0), "seq_lens must be int32 (num_seqs,)");
+    require(centroids_k.numel() == 16 && centroids_v.numel() == 16 && centroids_k.scalar_type() == at::kFloat &&
+                centroids_v.scalar_type() == at::kFloat,
+            "centroids must be 16 float32 values");
+    require(out.scalar_type() == q.scalar_type() && out.sizes() == q.sizes(), "out must have the shape and dtype of q");
+    require(num_splits >= 0, "num_splits must be >= 0");
+    const float* rot = nullptr;
+    int col_major = 0;
+    if (rotation.has_value()) {
+        const at::Tensor& r = *rotation;
+        fqbind::require_gpu(r, "rotation");
+        require(r.dim() == 2 && r.size(0) == head_dim && r.size(1) == head_dim && r.scalar_type() == at::kFloat,
+                "rotation must be float32 of shape (D, D)");
+        require(r.is_contiguous() || r.t().is_contiguous(), "rotation must be contiguous, or the transpose of a contiguous matrix");
+        col_major = r.is_contiguous() ? 0 : 1;
+        rot = r.data_ptr<float>();
+    }
+    c10::DeviceGuard guard(q.device());
+    const int st = fq_split_k_paged_decode_static(
+        q.data_ptr(), kv_cache.data_ptr<uint8_t>(), block_table.data_ptr<int32_t>(), seq_lens.data_ptr<int32_t>(),
+        centroids_k.data_ptr<float>(), centroids_v.data_ptr<float>(), rot, col_major, out.data_ptr(), int(q.size(0)),
+        int(q.size(1)), int(num_kv_heads), int(head_dim), int(block_size), int(block_table.size(1)), kv_cache.size(0),
+        float(sm_scale), fqbind::dtype_code(q.scalar_type(), "split_k_paged_decode_static"), int(num_splits),
+        fqbind::current_stream(q));
+    fqbind::raise_on_error(st, "split_k_paged_decode_static");
+    return out;
+}
+
 at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache, const at::Tensor& block_table,
                                 const at::Tensor& seq_lens, const at::Tensor& centroids_k,
                                 const at::Tensor& centroids_v, const std::optional<at::Tensor>& rotation,
@@ -577,6 +623,16 @@ void bind_kernels(py::module_& m) {
           "Split-K paged decode from the packed TQ4 cache; q un-rotated, result in the original space.");
     // Same operator under the name the vLLM attention impl looks for
     // (src/flashquant/vllm/impl.py:57-59, called with sm_scale= and out= keywords).
+    m.def("split_k_paged_decode_static", &split_k_paged_decode_static, py::arg("q"), py::arg("kv_cache"),
+          py::arg("block_table"), py::arg("seq_lens"), py::arg("centroids_k"), py::arg("centroids_v"),
+          py::arg("rotation"), py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"),
+          py::arg("sm_scale"), py::arg("out"), py::arg("num_splits") = 0,
+          "split_k_paged_decode on the library's static scratch array: allocates nothing (every tensor must "
+          "already be on the GPU, contiguous, and `out` is required).");
+    m.def("static_scratch_bytes", &fq_static_scratch_bytes);
+    m.def("paged_decode_workspace_bytes", &fq_paged_decode_workspace_bytes, py::arg("num_seqs"), py::arg("num_q_heads"),
+          py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("max_blocks_per_seq"),
+          py::arg("num_splits") = 0);
     m.def("fused_paged_tq4_decode", &split_k_paged_decode, py::arg("q"), py::arg("kv_cache"), py::arg("block_table"),
           py::arg("seq_lens"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),

@@ -1945,6 +1945,74 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_splits, stream);
 }
 
+// ---------------------------------------------------------------------------------------
+// The same decode for callers that cannot allocate (HIP graph capture, serving loops whose
+// harness forbids hipMalloc): the split partials and the rotated query live in a file-scope
+// device array instead of a caller workspace.  Every GPU the library runs on holds its own
+// copy of the array until the process ends; the host keeps each copy's address per device.
+// ---------------------------------------------------------------------------------------
+namespace fq {
+constexpr size_t kStaticScratchBytes = size_t(FQ_STATIC_SCRATCH_BYTES);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+}  // namespace fq
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device.  The array's name is a host-side handle,
+// not an address a kernel can use: the address comes from the runtime, once per device.
+int static_scratch_address(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        fq_host::note_hip_error(e);
+        return FQ_ERR_LAUNCH;
+    }
+    if (dev < 0 || dev >= kMaxDevices) return FQ_ERR_BAD_SHAPE;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(fq::scratch));
+        if (e != hipSuccess || p == nullptr) {
+            fq_host::note_hip_error(e);
+            return FQ_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return FQ_OK;
+}
+}  // namespace
+
+extern "C" size_t fq_static_scratch_bytes(void) { return fq::kStaticScratchBytes; }
+
+extern "C" int fq_split_k_paged_decode_static(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
+                                              const int32_t* seq_lens, const float* centroids_k,
+                                              const float* centroids_v, const float* rotation,
+                                              int rotation_col_major, void* out, int num_seqs, int H_Q, int H_KV,
+                                              int D, int block_size, int max_blocks_per_seq, int64_t num_blocks,
+                                              float sm_scale, int dtype, int num_splits, void* stream) {
+    using namespace fq;
+    const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
+                                       num_splits);
+    if (bad != FQ_OK) return bad;
+    if (num_seqs == 0) return FQ_OK;
+    const int ns = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
+    // the partials of this launch must fit the array: a larger problem is refused, not truncated
+    if (workspace_layout(num_seqs, H_Q, D, ns).total > kStaticScratchBytes) return FQ_ERR_WORKSPACE;
+    void* ws = nullptr;
+    const int st = static_scratch_address(&ws);
+    if (st != FQ_OK) return st;
+    // Nothing in the array has to start at zero: every (sequence, head, split) slot of the maxima
+    // and denominators is written by the decode kernel of this call (an empty split writes
+    // m = -inf), and the combine kernel ignores the accumulators of empty splits.
+    return fq_split_k_paged_decode(q, kv_cache, block_table, seq_lens, centroids_k, centroids_v, rotation,
+                                   rotation_col_major, out, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq,
+                                   num_blocks, sm_scale, dtype, ns, ws, kStaticScratchBytes, stream);
+}
+
 // TurboQuantProd pages: 3-bit keys with a sign-sketch correction of the scores, TQ4 values.
 extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
                                     const int32_t* seq_lens, const float* centroids_k3,

@@ -384,6 +384,29 @@ size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_KV, int D,
                                        int block_size, int max_blocks_per_seq,
                                        int num_splits);
 
+/*
+ * fq_split_k_paged_decode without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot call hipMalloc: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid allocation.  Arguments and results
+ * are those of fq_split_k_paged_decode; the split partials and the rotated query live in an
+ * array of FQ_STATIC_SCRATCH_BYTES bytes that the library keeps on every GPU it runs on until
+ * the process ends.  A launch whose workspace (fq_paged_decode_workspace_bytes) exceeds that
+ * size is refused with FQ_ERR_WORKSPACE.  All calls on one GPU share the array: calls that
+ * overlap on one GPU (different streams, different threads) race; calls ordered on one stream
+ * do not.  Calls no hipMalloc / hipFree; the first call on a device asks the runtime for the
+ * array's address (hipGetSymbolAddress).
+ */
+#define FQ_STATIC_SCRATCH_BYTES (16u << 20)
+size_t fq_static_scratch_bytes(void);
+int fq_split_k_paged_decode_static(const void* q, const uint8_t* kv_cache,
+                                   const int32_t* block_table, const int32_t* seq_lens,
+                                   const float* centroids_k, const float* centroids_v,
+                                   const float* rotation, int rotation_col_major, void* out,
+                                   int num_seqs, int H_Q, int H_KV, int D,
+                                   int block_size, int max_blocks_per_seq,
+                                   int64_t num_blocks, float sm_scale, int dtype,
+                                   int num_splits, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
