@@ -216,7 +216,7 @@ def main():
         cache0, table0 = caches[0]
         got = K.split_k_paged_decode(q, cache0, table0, lens, cent_d, cent_d, rot_d, H_KV, D, BS,
                                      sm_scale=scale).float().cpu()
-        done, spent, worst = 0, 0.0, 0.0
+        done, spent, worst, worst_abs = 0, 0.0, 0.0, 0.0
         while spent < 10.0 and done < 40 * BATCH:      # about 10 s of CPU work, whole sequences
             s_i = done % BATCH
             t1 = time.perf_counter()
@@ -224,7 +224,12 @@ def main():
                                           cent, cent, rot, H_KV, D, BS, sm_scale=scale)
             spent += time.perf_counter() - t1
             done += 1
-            worst = max(worst, (got[s_i] - want[0].float()).abs().max().item())
+            # 2e-2 of a row's magnitude, never less than 2e-2 absolute: the outlier channels take some
+            # output rows beyond |x| = 4, where a single bfloat16 step is 0.03
+            w_f = want[0].float()
+            row_scale = w_f.abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+            worst = max(worst, ((got[s_i] - w_f).abs() / row_scale).max().item())
+            worst_abs = max(worst_abs, (got[s_i] - w_f).abs().max().item())
         # the reference's CPU fallback as written, a Python loop over tokens and heads, at a reduced shape
         lb, ll = 2, 512
         lens_l = torch.full((lb,), ll, dtype=torch.int32)
@@ -251,7 +256,8 @@ def main():
             },
         }
         check = {
-            "max_abs_err": worst, "sequences_checked": min(done, BATCH), "tolerance": 2e-2,
+            "max_err_of_row_magnitude": worst, "max_abs_err": worst_abs, "sequences_checked": min(done, BATCH),
+            "tolerance": "2e-2 of the row's largest |x|, at least 2e-2 absolute",
             "loop_form_max_abs_err": worst_l, "ok": bool(worst <= 2e-2 and worst_l <= 2e-2),
         }
         del cache_h
