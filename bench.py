@@ -300,6 +300,14 @@ def main():
             "decompress_pct_hbm_peak": 100.0 * nrows * 324 / (d_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         })
 
+        dr_ms, _ = time_events(lambda i: K.tq4_decompress_rotated(packed, norms, cent_d, rot_d, torch.bfloat16, out=y),
+                               EXTRA_ITERS)
+        extra.update({
+            "decompress_rotated_ms": dr_ms,
+            "decompress_rotated_gbps": nrows * 324 / (dr_ms * 1e-3) / 1e9,
+            "decompress_rotated_pct_hbm_peak": 100.0 * nrows * 324 / (dr_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        })
+
         del y, packed, norms
         torch.cuda.empty_cache()
 

@@ -131,6 +131,40 @@ void tq4_compress_store(const at::Tensor& key, const at::Tensor& value, const at
     fqbind::raise_on_error(st, "tq4_compress_store");
 }
 
+// tq4_decompress followed by (x.float() @ rotation).to(dtype), one launch
+// (src/flashquant/vllm/impl.py:298-316).
+at::Tensor tq4_decompress_rotated(const at::Tensor& packed, const at::Tensor& norms, const at::Tensor& centroids,
+                                  const at::Tensor& rotation, at::ScalarType dtype,
+                                  const std::optional<at::Tensor>& out) {
+    fqbind::require_gpu(packed, "packed");
+    require(packed.dim() == 3 && packed.scalar_type() == at::kByte, "packed must be uint8 of shape (N, H, D/2)");
+    const int64_t N = packed.size(0), H = packed.size(1), D = 2 * packed.size(2);
+    require(norms.scalar_type() == at::kFloat && norms.numel() == N * H, "norms must be float32 of shape (N, H, 1)");
+    require(centroids.scalar_type() == at::kFloat && centroids.numel() == 16, "centroids must be 16 float32 values");
+    require(dtype == at::kHalf || dtype == at::kBFloat16, "tq4_decompress_rotated: dtype must be float16 or bfloat16");
+    c10::DeviceGuard guard(packed.device());
+    const at::Tensor pc = packed.contiguous();
+    const at::Tensor nc = norms.to(packed.device()).contiguous();
+    const at::Tensor cc = centroids.to(packed.device()).contiguous();
+    const RotationArg rot = rotation_arg(rotation, packed.device(), D);
+    at::Tensor result;
+    if (out.has_value()) {
+        result = *out;
+        require(result.is_cuda() && result.is_contiguous() && result.scalar_type() == dtype &&
+                    result.numel() >= N * H * D,
+                "out must be a contiguous GPU tensor of the requested dtype with room for (N, H, D)");
+        result = result.flatten().narrow(0, 0, N * H * D).view({N, H, D});
+    } else {
+        result = at::empty({N, H, D}, packed.options().dtype(dtype));
+    }
+    const int st = fq_tq4_decompress_rotated(pc.data_ptr<uint8_t>(), nc.data_ptr<float>(), cc.data_ptr<float>(), rot.ptr,
+                                             rot.col_major, result.data_ptr(),
+                                             fqbind::dtype_code(dtype, "tq4_decompress_rotated"), N * H, int(D),
+                                             fqbind::current_stream(packed));
+    fqbind::raise_on_error(st, "tq4_decompress_rotated");
+    return result;
+}
+
 at::Tensor tq4_decompress(const at::Tensor& packed, const at::Tensor& norms, const at::Tensor& centroids,
                           at::ScalarType dtype, const std::optional<at::Tensor>& out) {
     fqbind::require_gpu(packed, "packed");
@@ -667,6 +701,9 @@ void bind_kernels(py::module_& m) {
         pk.def("unpack_2bit", &unpack_2bit, py::arg("packed"), "Inverse of pack_2bit, int64");
         pk.def("validate_indices", &validate_indices, py::arg("indices"), py::arg("bits"));
     }
+    m.def("tq4_decompress_rotated", &tq4_decompress_rotated, py::arg("packed"), py::arg("norms"), py::arg("centroids"),
+          py::arg("rotation"), py::arg("dtype"), py::arg("out") = py::none(),
+          "tq4_decompress to dtype, then (x.float() @ rotation).to(dtype): original-space rows in one launch");
     m.def("set_option", [](const std::string& name, bool value) {
               const int id = option_id(name);
               const int before = fq_get_option(id);

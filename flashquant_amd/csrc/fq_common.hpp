@@ -34,10 +34,7 @@ __device__ __forceinline__ uint32_t float_to_bits(float f) { return __builtin_bi
 // torch's Tensor.to(torch.bfloat16) does; NaN stays NaN.
 __device__ __forceinline__ float bf16_to_float(uint16_t h) { return bits_to_float(uint32_t(h) << 16); }
 __device__ __forceinline__ uint16_t float_to_bf16(float f) {
-    uint32_t u = float_to_bits(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return uint16_t(u >> 16);
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));   // v_cvt_pk_bf16_f32: round to nearest even
 }
 __device__ __forceinline__ float f16_to_float(uint16_t h) {
     return float(__builtin_bit_cast(_Float16, h));

@@ -20,10 +20,10 @@
 // A lane of the accumulator holds one row and 16 consecutive output
 // coordinates (the MFMA row index is permuted on the R side to make them
 // consecutive), so a lane bucketizes and nibble-packs 8 output bytes without
-// any cross-lane traffic.  Bucketize is one LDS lookup in a 256-cell table
+// any cross-lane traffic.  Bucketize is one LDS lookup in a 64-cell table
 // built from the boundaries (base count + the single boundary that can fall in
-// the cell) plus one compare; if two boundaries share a cell the kernel falls
-// back to the 15-compare scan.
+// the cell; 32 copies of every cell, one per bank) plus one compare; if two
+// boundaries share a cell the kernel falls back to the 15-compare scan.
 
 #include "fq_common.hpp"
 
@@ -43,7 +43,6 @@ struct CompressCfg {
     static constexpr int PASSES = TT / ROWS_PER_PASS;
     static constexpr int XS_STRIDE = D * 2 + 16;       // bytes per staged row
     static constexpr int OUT_STRIDE = D / 2 + 8;       // bytes per packed row in LDS
-    static constexpr int CELLS = 256;
 };
 
 constexpr float kLoScale = 1.0f / 4096.0f;
@@ -66,8 +65,14 @@ __device__ __forceinline__ float dpp_f32(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
 
+// 64 cells over the span of the boundaries, every cell stored 32 times side by side (a cell is a
+// 256-byte row of 32 copies of 8 bytes): lane l reads copy l % 32, so the lanes of a half-wave
+// always hit different banks whatever cells their values fall in.  A single copy made the
+// data-dependent lookups collide (4-5 lanes per bank on average).
+constexpr int kBucketCells = 64;
+constexpr int kBucketCopies = 32;
 struct BucketTable {
-    uint2v cell[256];   // x = threshold bits, y = base count
+    uint2v cell[kBucketCells * kBucketCopies];   // x = threshold bits, y = base count
     float bnd[16];
     float inv_w;
     float offset;
@@ -83,11 +88,11 @@ __device__ __forceinline__ void build_bucket_table(BucketTable& t, const float* 
     __syncthreads();
     const float b0 = t.bnd[0], b14 = t.bnd[14];
     const float span = b14 - b0;
-    const float pad = span > 0.0f ? span * (1.0f / 256.0f) : 1.0f;
+    const float pad = span > 0.0f ? span * (1.0f / float(kBucketCells)) : 1.0f;
     const float lo = b0 - pad;
-    const float w = (span + 2.0f * pad) * (1.0f / 256.0f);
+    const float w = (span + 2.0f * pad) * (1.0f / float(kBucketCells));
     const float margin = 0.01f * w;
-    for (int c = tid; c < 256; c += nthreads) {
+    for (int c = tid; c < kBucketCells; c += nthreads) {
         const float lo_c = lo + w * float(c) - margin;
         const float hi_c = lo + w * float(c + 1) + margin;
         int base = 0, inside = 0;
@@ -102,7 +107,7 @@ __device__ __forceinline__ void build_bucket_table(BucketTable& t, const float* 
             }
         }
         if (inside > 1 || !(span > 0.0f)) t.slow = 1;
-        t.cell[c] = uint2v{float_to_bits(thr), uint32_t(base)};
+        for (int k = 0; k < kBucketCopies; ++k) t.cell[c * kBucketCopies + k] = uint2v{float_to_bits(thr), uint32_t(base)};
     }
     if (tid == 0) {
         t.inv_w = 1.0f / w;
@@ -111,10 +116,14 @@ __device__ __forceinline__ void build_bucket_table(BucketTable& t, const float* 
     __syncthreads();
 }
 
-__device__ __forceinline__ uint32_t bucket_fast(const BucketTable& t, float y, float inv_w, float offset) {
+// `copy` = lane % 32
+__device__ __forceinline__ uint2v bucket_cell(const BucketTable& t, float y, float inv_w, float offset, int copy) {
     const float pos = __builtin_fmaf(y, inv_w, offset);
-    const int c = int(__builtin_amdgcn_fmed3f(pos, 0.0f, 255.0f));
-    const uint2v e = t.cell[c];
+    const int c = int(__builtin_amdgcn_fmed3f(pos, 0.0f, float(kBucketCells - 1)));
+    return t.cell[c * kBucketCopies + copy];
+}
+__device__ __forceinline__ uint32_t bucket_fast(const BucketTable& t, float y, float inv_w, float offset, int copy) {
+    const uint2v e = bucket_cell(t, y, inv_w, offset, copy);
     return e.y + (bits_to_float(e.x) < y ? 1u : 0u);
 }
 
@@ -369,9 +378,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                     }
                     if (st < 16) {
                         yv[st] = acc_in[st] * inv;
-                        const float pos = __builtin_fmaf(yv[st], inv_w, offset);
-                        const int c = int(__builtin_amdgcn_fmed3f(pos, 0.0f, 255.0f));
-                        cell[st] = table.cell[c];
+                        cell[st] = bucket_cell(table, yv[st], inv_w, offset, n32);
                     }
                     if (st >= 4 && st < 20) {
                         const int e = st - 4;
@@ -461,7 +468,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             uint32_t idx[16];
             if (!slow) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) idx[i] = bucket_fast(table, yv[i], inv_w, offset);
+                for (int i = 0; i < 16; ++i) idx[i] = bucket_fast(table, yv[i], inv_w, offset, n32);
             } else {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) idx[i] = bucket_slow(table, yv[i]);

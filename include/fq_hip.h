@@ -169,6 +169,23 @@ int fq_tq4_decompress(const uint8_t* packed, const float* norms,
                       int64_t M, int D, void* stream);
 
 /*
+ * TQ4 decompress followed by the inverse rotation, one launch: what the serving path does
+ * when it materialises the cache (_decompress_cache with apply_rotation,
+ * src/flashquant/vllm/impl.py:265-318: tq4_decompress to the compute dtype, then
+ * (x.float() @ rotation).to(dtype), impl.py:309-316).
+ *
+ *   packed, norms, centroids   as for fq_tq4_decompress
+ *   rotation   (D, D) float32, layout flag as in fq_split_k_paged_decode
+ *   out        (M, D) fp16 / bf16, 16-byte aligned, original space:
+ *              out = dtype(float32(dtype(centroid[idx] * norm)) @ rotation)
+ * The contraction accumulates in float32 on the matrix cores in an order of its own, so a
+ * result may differ from a float32 matmul's by one unit in the last place of the 16-bit output.
+ */
+int fq_tq4_decompress_rotated(const uint8_t* packed, const float* norms, const float* centroids,
+                              const float* rotation, int rotation_col_major,
+                              void* out, int out_dtype, int64_t M, int D, void* stream);
+
+/*
  * Fused TQ4 attention (prefill): un-rotated query, packed keys and values,
  * original-space output.  Takes the role of the reference's fused launcher
  * (csrc/cuda/fused_tq_attention.cu:468-479); operator defined by

@@ -74,6 +74,61 @@ def test_decompress_out_argument_and_empty():
     assert empty.shape == (0, 2, 128)
 
 
+# ---- decompress + inverse rotation in one launch ----------------------------------
+
+def _ulp16(x, dtype):
+    """One unit in the last place of every element of a float32 tensor rounded to dtype."""
+    mant = 7 if dtype == torch.bfloat16 else 10
+    e = torch.floor(torch.log2(x.abs().clamp_min(1e-30)))
+    if dtype == torch.float16:
+        e = e.clamp_min(-14)
+    return torch.pow(2.0, e - mant)
+
+
+@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 1), (7, 3), (1000, 8)])
+def test_decompress_rotated_matches_decompress_then_matmul(d, dtype, shape):
+    """The serving path's two steps (src/flashquant/vllm/impl.py:298-316) in one kernel: the
+    dequantised row is rounded to the dtype, multiplied by the rotation in float32 and rounded
+    again.  The matrix cores sum in another order than a float32 matmul, so a result may sit on
+    the other side of a rounding tie: at most one unit in the last place, on few elements."""
+    c, _, r = book(d)
+    n, h = shape
+    g = torch.Generator().manual_seed(n * 17 + d)
+    packed = torch.randint(0, 256, (n, h, d // 2), dtype=torch.uint8, generator=g)
+    norms = torch.rand(n, h, 1, generator=g) * 30 + 0.01
+    want = torch.matmul(O.decompress(packed, norms, c).to(dtype).float(), r)
+    got = K.tq4_decompress_rotated(packed.to(DEV), norms.to(DEV), c.to(DEV), r.to(DEV), dtype)
+    assert got.dtype == dtype and got.shape == (n, h, d)
+    diff = (got.cpu().float() - want.to(dtype).float()).abs()
+    # (an element that nearly cancels has a tiny unit of its own; the matrix, held to 2^-17 of its
+    # entries, moves it by a few 1e-6 of the row's largest element)
+    bound = 1.001 * _ulp16(want, dtype) + 4e-5 * want.abs().amax(dim=-1, keepdim=True)
+    assert (diff <= bound).all(), f"worst {(diff / bound).max().item()} of the bound"
+    assert (diff > 0).float().mean().item() <= 0.03
+    # relative MSE of the reconstruction against the float32 result: far inside the 1e-3 bar
+    rel = ((got.cpu().float() - want) ** 2).sum().item() / (want ** 2).sum().item()
+    assert rel <= 1e-4
+    # both matrix layouts, and the out= argument
+    col = r.t().contiguous().t().to(DEV)
+    out = torch.empty(n, h, d, dtype=dtype, device=DEV)
+    again = K.tq4_decompress_rotated(packed.to(DEV), norms.to(DEV), c.to(DEV), col, dtype, out=out)
+    assert again.data_ptr() == out.data_ptr() and torch.equal(again, got)
+
+
+def test_decompress_rotated_recovers_what_compress_took():
+    c, b, r = book(128)
+    x = outlier_rows(4096, 8, 128, seed=1234)
+    packed, norms = K.tq4_compress(x.to(torch.bfloat16).to(DEV), r.to(DEV), b.to(DEV))
+    rec = K.tq4_decompress_rotated(packed, norms, c.to(DEV), r.to(DEV), torch.bfloat16).cpu().float()
+    rel = ((rec - x) ** 2).sum().item() / (x ** 2).sum().item()
+    assert 0.0085 <= rel <= 0.0105           # the 16-level Lloyd-Max distortion
+    with pytest.raises(ValueError):
+        K.tq4_decompress_rotated(packed, norms, c.to(DEV), r.to(DEV), torch.float32)
+    assert K.tq4_decompress_rotated(packed[:0], norms[:0], c.to(DEV), r.to(DEV), torch.float16).shape == (0, 8, 128)
+
+
 # ---- compress -------------------------------------------------------------------
 
 def _check_compress(x, d, dtype):
