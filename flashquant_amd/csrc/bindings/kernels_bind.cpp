@@ -295,6 +295,63 @@ at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache,
     return result;
 }
 
+// Keys or values of (B, H, N, X) taken from a buffer of larger token capacity: a view
+// buffer[:, :, :N, :] (the reference's CompressedBuffer.get(), src/flashquant/cache/buffer_pool.py:128-140)
+// keeps the row layout of a contiguous tensor with N replaced by the capacity.  Returns that
+// capacity, or 0 when the strides are anything else.
+int64_t slab_capacity(const at::Tensor& t) {
+    const int64_t B = t.size(0), H = t.size(1), N = t.size(2), X = t.size(3);
+    if (t.numel() == 0) return N;
+    if ((X > 1 && t.stride(3) != 1) || (N > 1 && t.stride(2) != X)) return 0;
+    int64_t cap = N;
+    if (H > 1) {
+        if (t.stride(1) % X != 0) return 0;
+        cap = t.stride(1) / X;
+    } else if (B > 1) {
+        if (t.stride(0) % X != 0) return 0;
+        cap = t.stride(0) / X;
+    }
+    if (cap < N) return 0;
+    if (B > 1 && t.stride(0) != H * cap * X) return 0;
+    return cap;
+}
+
+// TQ4 compress of (B, H, n, D) new tokens straight into pre-allocated buffers at `position`:
+// the compress + CompressedBuffer.append of the HF cache in one launch
+// (src/flashquant/cache/hf_cache.py:283-312, src/flashquant/cache/buffer_pool.py:86-111).
+void tq4_compress_append(const at::Tensor& x, const at::Tensor& rot_T_even, const at::Tensor& rot_T_odd,
+                         const at::Tensor& boundaries, const at::Tensor& packed_buf, const at::Tensor& norms_buf,
+                         int64_t position) {
+    fqbind::require_gpu(x, "x");
+    fqbind::require_gpu(packed_buf, "packed_buf");
+    fqbind::require_gpu(norms_buf, "norms_buf");
+    require(x.dim() == 4, "x must have shape (B, H, n, D)");
+    require(x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16, "x must be float16 or bfloat16");
+    const int64_t B = x.size(0), H = x.size(1), n = x.size(2), D = x.size(3);
+    require(packed_buf.dim() == 4 && packed_buf.scalar_type() == at::kByte && packed_buf.is_contiguous() &&
+                packed_buf.size(0) == B && packed_buf.size(1) == H && packed_buf.size(3) == D / 2,
+            "packed_buf must be a contiguous uint8 buffer of shape (B, H, capacity, D/2)");
+    const int64_t cap = packed_buf.size(2);
+    require(norms_buf.scalar_type() == at::kFloat && norms_buf.is_contiguous() && norms_buf.numel() == B * H * cap,
+            "norms_buf must be a contiguous float32 buffer of shape (B, H, capacity, 1)");
+    if (position < 0 || position + n > cap)
+        throw std::runtime_error("tq4_compress_append: appending " + std::to_string(n) + " tokens at position " +
+                                 std::to_string(position) + " would exceed the capacity " + std::to_string(cap));
+    require(rot_T_even.scalar_type() == at::kFloat && rot_T_odd.scalar_type() == at::kFloat &&
+                boundaries.scalar_type() == at::kFloat && rot_T_even.dim() == 2 && rot_T_even.size(0) == D &&
+                rot_T_even.size(1) == D / 2 && rot_T_odd.sizes() == rot_T_even.sizes() && boundaries.numel() == 15,
+            "rotation halves must be float32 (D, D/2) and boundaries 15 float32 values");
+    c10::DeviceGuard guard(x.device());
+    const at::Tensor xc = x.contiguous();
+    const at::Tensor re = rot_T_even.to(x.device()).contiguous(), ro = rot_T_odd.to(x.device()).contiguous();
+    const at::Tensor bd = boundaries.to(x.device()).contiguous();
+    const int st = fq_tq4_compress_append(xc.data_ptr(), fqbind::dtype_code(x.scalar_type(), "tq4_compress_append"),
+                                          re.data_ptr<float>(), ro.data_ptr<float>(), bd.data_ptr<float>(),
+                                          packed_buf.data_ptr<uint8_t>(), norms_buf.data_ptr<float>(), B * H, n, cap,
+                                          position, int(D), fqbind::current_stream(x));
+    fqbind::raise_on_error(st, "tq4_compress_append");
+}
+
 at::Tensor fused_tq_attention(const at::Tensor& q, const at::Tensor& k_packed, const at::Tensor& k_norms,
                               const at::Tensor& v_packed, const at::Tensor& v_norms, const at::Tensor& centroids_k,
                               const at::Tensor& centroids_v, const at::Tensor& rotation,
@@ -321,15 +378,29 @@ at::Tensor fused_tq_attention(const at::Tensor& q, const at::Tensor& k_packed, c
     c10::DeviceGuard guard(q.device());
     const double scale = sm_scale.has_value() ? *sm_scale : 1.0 / std::sqrt(double(D));
     const at::Tensor qc = q.contiguous();
-    const at::Tensor kp = k_packed.contiguous(), vp = v_packed.contiguous();
-    const at::Tensor kn = k_norms.to(q.device()).contiguous(), vn = v_norms.to(q.device()).contiguous();
+    // views of buffers with a larger token capacity are taken as they are (no copy)
+    at::Tensor kp = k_packed, vp = v_packed;
+    at::Tensor kn = k_norms.to(q.device()), vn = v_norms.to(q.device());
+    if (kn.dim() != 4) kn = kn.reshape({B, HKV, NKV, 1});
+    if (vn.dim() != 4) vn = vn.reshape({B, HKV, NKV, 1});
+    int64_t k_cap = slab_capacity(kp), v_cap = slab_capacity(vp);
+    if (k_cap == 0 || slab_capacity(kn) != k_cap) {
+        kp = kp.contiguous();
+        kn = kn.contiguous();
+        k_cap = NKV;
+    }
+    if (v_cap == 0 || slab_capacity(vn) != v_cap) {
+        vp = vp.contiguous();
+        vn = vn.contiguous();
+        v_cap = NKV;
+    }
     const at::Tensor ck = centroids_k.to(q.device()).contiguous(), cv = centroids_v.to(q.device()).contiguous();
     const RotationArg rot = rotation_arg(rotation, q.device(), D);
     at::Tensor result = at::empty_like(qc);
-    const int st = fq_fused_tq_attention(
+    const int st = fq_fused_tq_attention_strided(
         qc.data_ptr(), kp.data_ptr<uint8_t>(), kn.data_ptr<float>(), vp.data_ptr<uint8_t>(), vn.data_ptr<float>(),
         ck.data_ptr<float>(), cv.data_ptr<float>(), rot.ptr, rot.col_major, result.data_ptr(),
-        int(B), int(HQ), int(HKV), int(NQ), int(NKV), int(D), float(scale), is_causal ? 1 : 0,
+        int(B), int(HQ), int(HKV), int(NQ), int(NKV), k_cap, v_cap, int(D), float(scale), is_causal ? 1 : 0,
         fqbind::dtype_code(q.scalar_type(), "fused_tq_attention"), fqbind::current_stream(q));
     fqbind::raise_on_error(st, "fused_tq_attention");
     return result;
@@ -701,6 +772,10 @@ void bind_kernels(py::module_& m) {
         pk.def("unpack_2bit", &unpack_2bit, py::arg("packed"), "Inverse of pack_2bit, int64");
         pk.def("validate_indices", &validate_indices, py::arg("indices"), py::arg("bits"));
     }
+    m.def("tq4_compress_append", &tq4_compress_append, py::arg("x"), py::arg("rot_T_even"), py::arg("rot_T_odd"),
+          py::arg("boundaries"), py::arg("packed_buf"), py::arg("norms_buf"), py::arg("position"),
+          "TQ4 compress of x (B, H, n, D) into packed_buf (B, H, capacity, D/2) / norms_buf (B, H, capacity, 1) at "
+          "token `position`, in place");
     m.def("tq4_decompress_rotated", &tq4_decompress_rotated, py::arg("packed"), py::arg("norms"), py::arg("centroids"),
           py::arg("rotation"), py::arg("dtype"), py::arg("out") = py::none(),
           "tq4_decompress to dtype, then (x.float() @ rotation).to(dtype): original-space rows in one launch");

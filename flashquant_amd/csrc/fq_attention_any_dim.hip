@@ -153,7 +153,8 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
     for (int i = 0; i < 4; ++i) { m_run[i] = -__builtin_inff(); l_run[i] = 0.0f; }
 
     const int tok_d = tid >> 3, part = tid & 7;       // dequantisation: token of the tile, eighth of its row
-    const int64_t kv_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.N_KV;
+    const int64_t k_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.k_cap;
+    const int64_t v_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.v_cap;
     _Float16* pw = ps + w * 16 * C::VSTRIDE;
 
     for (int tile = 0; tile < ntiles; ++tile) {
@@ -175,10 +176,10 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
                 vp = row + H * (D / 2 + 4) + hkv * (D / 2);
                 nv = *reinterpret_cast<const float*>(row + H * (D + 4) + 4 * hkv);
             } else {
-                kp = p.k_packed + (kv_row0 + tok) * (D / 2);
-                vp = p.v_packed + (kv_row0 + tok) * (D / 2);
-                nk = p.k_norms[kv_row0 + tok];
-                nv = p.v_norms[kv_row0 + tok];
+                kp = p.k_packed + (k_row0 + tok) * (D / 2);
+                vp = p.v_packed + (v_row0 + tok) * (D / 2);
+                nk = p.k_norms[k_row0 + tok];
+                nv = p.v_norms[v_row0 + tok];
             }
             if (!live) { nk = 0.0f; nv = 0.0f; }
             const int ek = norm_excess(nk), ev = norm_excess(nv);

@@ -18,6 +18,7 @@ struct AnyDimParams {
     uint16_t* out;
     int rot_col_major;
     int H_Q, H_KV, G, N_Q, N_KV;
+    int64_t k_cap, v_cap;       // tokens between the slabs of consecutive (batch, KV head) pairs (>= N_KV)
     int causal;
     float scale_log2e;
     const int32_t* cu_seqlens_q;   // paged operands

@@ -154,6 +154,10 @@ struct PagedDest {
     int mapped;                 // tokens with a slot
     int H;
     int wide;                   // 16-byte stores are aligned
+    // plain (not paged) mode, append into a buffer of larger capacity: input row (o, t), t < append_n,
+    // lands in output row o * append_cap + append_pos + t; append_n == 0: output row = input row
+    uint32_t append_n;
+    int64_t append_cap, append_pos;
 };
 
 template <int D, int DT, bool PAGED>
@@ -172,6 +176,11 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
         const int64_t slot = pd.slots[tok];
         if (slot < 0 || slot >= pd.num_slots) return nullptr;
         return pd.cache + slot * (int64_t(pd.H) * (D + 8)) + (is_v ? int64_t(pd.H) * (D / 2 + 4) : 0);
+    };
+    auto out_row = [&](int64_t row) -> int64_t {
+        if (pd.append_n == 0u) return row;
+        const uint32_t o = uint32_t(row) / pd.append_n;
+        return int64_t(o) * pd.append_cap + pd.append_pos + int64_t(uint32_t(row) - o * pd.append_n);
     };
     __shared__ __attribute__((aligned(16))) uint8_t xs[2][C::TT * C::XS_STRIDE];
     // bf16 rows of head_dim 128 run a software pipeline (see below) with two packed-row buffers
@@ -312,7 +321,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                         uint8_t* dst = paged_row(row, head, is_v);
                         if (dst) *reinterpret_cast<float*>(dst + pd.H * (D / 2) + 4 * head) = nrm;
                     } else {
-                        norms[row] = nrm;
+                        norms[out_row(row)] = nrm;
                     }
                 }
             }
@@ -342,7 +351,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                         }
                     }
                 } else {
-                    __builtin_nontemporal_store(v, reinterpret_cast<uint4v*>(packed + row * (D / 2)) + q);
+                    __builtin_nontemporal_store(v, reinterpret_cast<uint4v*>(packed + out_row(row) * (D / 2)) + q);
                 }
             }
         }
@@ -490,13 +499,13 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
 
 template <int D, int DT>
 int launch_compress(const void* x, const float* re, const float* ro, const float* bnd, uint8_t* packed,
-                    float* norms, int64_t M, int num_cus, hipStream_t s) {
+                    float* norms, int64_t M, int num_cus, hipStream_t s, const PagedDest& pd = PagedDest{}) {
     using C = CompressCfg<D>;
     const int64_t tiles = (M + C::TT - 1) / C::TT;
     const int64_t cap = int64_t(num_cus) * 2;
     const unsigned grid = unsigned(tiles < cap ? tiles : cap);
     hipLaunchKernelGGL((tq4_compress_kernel<D, DT, false>), dim3(grid), dim3(C::THREADS), 0, s,
-                       reinterpret_cast<const uint4v*>(x), re, ro, bnd, packed, norms, M, tiles, PagedDest{});
+                       reinterpret_cast<const uint4v*>(x), re, ro, bnd, packed, norms, M, tiles, pd);
     return fq_host::check_launch();
 }
 
@@ -560,6 +569,39 @@ extern "C" int fq_tq4_compress(const void* x, int x_dtype, const float* rot_T_ev
 #undef FQ_COMPRESS_CASE
 }
 
+extern "C" int fq_tq4_compress_append(const void* x, int x_dtype, const float* rot_T_even, const float* rot_T_odd,
+                                      const float* boundaries, uint8_t* packed, float* norms, int64_t outer,
+                                      int64_t n_new, int64_t capacity, int64_t position, int D, void* stream) {
+    using namespace fq;
+    if (outer < 0 || n_new < 0 || capacity < 0 || position < 0 || position + n_new > capacity) return FQ_ERR_BAD_SHAPE;
+    if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
+    if (x_dtype != FQ_F16 && x_dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
+    if (outer == 0 || n_new == 0) return FQ_OK;
+    if (outer * n_new > 0x7fffffffLL || n_new > 0x7fffffffLL) return FQ_ERR_BAD_SHAPE;   // 32-bit row arithmetic in the kernel
+    if (!x || !rot_T_even || !rot_T_odd || !boundaries || !packed || !norms) return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(x, 16) || !fq_host::aligned(packed, 16) || !fq_host::aligned(norms, 4))
+        return FQ_ERR_MISALIGNED;
+    PagedDest pd{};
+    pd.append_n = uint32_t(n_new);
+    pd.append_cap = capacity;
+    pd.append_pos = position;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int cus = fq_host::device_cu_count();
+    const int64_t M = outer * n_new;
+#define FQ_APPEND_CASE(DD)                                                                                         \
+    case DD:                                                                                                       \
+        return x_dtype == FQ_F16                                                                                   \
+                   ? launch_compress<DD, FQ_F16>(x, rot_T_even, rot_T_odd, boundaries, packed, norms, M, cus, s, pd)  \
+                   : launch_compress<DD, FQ_BF16>(x, rot_T_even, rot_T_odd, boundaries, packed, norms, M, cus, s, pd);
+    switch (D) {
+        FQ_APPEND_CASE(64)
+        FQ_APPEND_CASE(128)
+        FQ_APPEND_CASE(256)
+        default: return FQ_ERR_UNSUPPORTED_DIM;
+    }
+#undef FQ_APPEND_CASE
+}
+
 extern "C" int fq_tq4_compress_store(const void* key, const void* value, int x_dtype,
                                      const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
                                      uint8_t* kv_cache, const int64_t* slot_mapping,
@@ -575,7 +617,7 @@ extern "C" int fq_tq4_compress_store(const void* key, const void* value, int x_d
         !fq_host::aligned(slot_mapping, 8))
         return FQ_ERR_MISALIGNED;
     if (num_tokens > 0x7fffffffLL || num_tokens * H_KV > (int64_t(1) << 40)) return FQ_ERR_BAD_SHAPE;
-    PagedDest pd;
+    PagedDest pd{};
     pd.x_value = static_cast<const uint4v*>(value);
     pd.cache = kv_cache;
     pd.slots = slot_mapping;

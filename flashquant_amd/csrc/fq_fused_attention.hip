@@ -56,6 +56,7 @@ struct PrefillParams {
     uint16_t* out;              // (B, H_Q, N_Q, 128)
     int rot_col_major;
     int H_Q, H_KV, G, N_Q, N_KV;
+    int64_t k_cap, v_cap;       // tokens between the slabs of consecutive (batch, KV head) pairs (>= N_KV)
     int causal;
     float scale_log2e;
     // paged mode (variable-length queries over the packed paged cache)
@@ -156,11 +157,12 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const uint32_t lk = 4u * (lane & 31), lv = 128u + lk;
 
     // ---- dequantisation plan ------------------------------------------------------------------
-    const int64_t kv_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.N_KV;
-    const uint8_t* kp = p.k_packed + kv_row0 * 64;
-    const uint8_t* vp = p.v_packed + kv_row0 * 64;
-    const float* knp = p.k_norms + kv_row0;
-    const float* vnp = p.v_norms + kv_row0;
+    const int64_t k_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.k_cap;
+    const int64_t v_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.v_cap;
+    const uint8_t* kp = p.k_packed + k_row0 * 64;
+    const uint8_t* vp = p.v_packed + v_row0 * 64;
+    const float* knp = p.k_norms + k_row0;
+    const float* vnp = p.v_norms + v_row0;
     const int tk = tid >> 3, gqk = tid & 7;        // K: token of the tile, 16-coordinate group
     const int tp = tid >> 4, jv = tid & 15;        // V: token pair of the tile, dword of the row
     const int k_wr = tk * kPfKStride + gqk * 32;
@@ -518,8 +520,21 @@ extern "C" int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, con
                                      const float* rotation, int rotation_col_major, void* out,
                                      int B, int H_Q, int H_KV, int N_Q, int N_KV, int D,
                                      float sm_scale, int is_causal, int dtype, void* stream) {
+    return fq_fused_tq_attention_strided(q, k_packed, k_norms, v_packed, v_norms, centroids_k, centroids_v, rotation,
+                                         rotation_col_major, out, B, H_Q, H_KV, N_Q, N_KV, N_KV, N_KV, D, sm_scale,
+                                         is_causal, dtype, stream);
+}
+
+extern "C" int fq_fused_tq_attention_strided(const void* q, const uint8_t* k_packed, const float* k_norms,
+                                             const uint8_t* v_packed, const float* v_norms,
+                                             const float* centroids_k, const float* centroids_v,
+                                             const float* rotation, int rotation_col_major, void* out,
+                                             int B, int H_Q, int H_KV, int N_Q, int N_KV,
+                                             int64_t k_capacity, int64_t v_capacity, int D,
+                                             float sm_scale, int is_causal, int dtype, void* stream) {
     using namespace fq;
     if (B < 0 || H_Q <= 0 || H_KV <= 0 || N_Q < 0 || N_KV < 0 || H_Q % H_KV != 0) return FQ_ERR_BAD_SHAPE;
+    if (k_capacity < N_KV || v_capacity < N_KV) return FQ_ERR_BAD_SHAPE;
     if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
     if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
     if (B == 0 || N_Q == 0) return FQ_OK;
@@ -539,6 +554,7 @@ extern "C" int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, con
         a.rotation = rotation; a.rot_col_major = rotation_col_major;
         a.out = static_cast<uint16_t*>(out);
         a.H_Q = H_Q; a.H_KV = H_KV; a.G = H_Q / H_KV; a.N_Q = N_Q; a.N_KV = N_KV;
+        a.k_cap = k_capacity; a.v_cap = v_capacity;
         a.causal = (is_causal && N_Q > 1) ? 1 : 0;
         a.scale_log2e = sm_scale * kLog2e;
         return launch_attention_any_dim(a, D, false, N_Q, B, dtype, stream);
@@ -551,6 +567,7 @@ extern "C" int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, con
     p.rotation = rotation; p.rot_col_major = rotation_col_major;
     p.out = static_cast<uint16_t*>(out);
     p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.N_Q = N_Q; p.N_KV = N_KV;
+    p.k_cap = k_capacity; p.v_cap = v_capacity;
     p.causal = (is_causal && N_Q > 1) ? 1 : 0;
     p.scale_log2e = sm_scale * kLog2e;
 
@@ -619,6 +636,7 @@ extern "C" int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, 
     p.rotation = rotation; p.rot_col_major = rotation_col_major;
     p.out = static_cast<uint16_t*>(out);
     p.H_Q = H_Q; p.H_KV = H_KV; p.G = H_Q / H_KV; p.N_Q = 0; p.N_KV = 0;
+    p.k_cap = 0; p.v_cap = 0;
     p.causal = is_causal ? 1 : 0;
     p.scale_log2e = sm_scale * kLog2e;
     p.cu_seqlens_q = cu_seqlens_q; p.seq_lens = seq_lens; p.block_table = block_table; p.cache = kv_cache;

@@ -132,6 +132,23 @@ int fq_tq4_compress(const void* x, int x_dtype,
                     int64_t M, int D, void* stream);
 
 /*
+ * TQ4 compress straight into a pre-allocated (B, H, capacity, D/2) buffer at a token position:
+ * the compress of the HF cache followed by CompressedBuffer.append
+ * (src/flashquant/cache/hf_cache.py:283-312, src/flashquant/cache/buffer_pool.py:86-111) without
+ * the intermediate tensors or the strided copy.
+ *   x          (outer, n_new, D) fp16 / bf16, contiguous: outer = B * H slabs of n_new new tokens
+ *   packed     (outer, capacity, D/2) uint8 buffer, norms (outer, capacity) float32 buffer;
+ *              row (o, t) of x lands in row (o, position + t)
+ * position >= 0 and position + n_new <= capacity, else FQ_ERR_BAD_SHAPE (the reference raises
+ * on overflow, buffer_pool.py:100-107).
+ */
+int fq_tq4_compress_append(const void* x, int x_dtype,
+                           const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
+                           uint8_t* packed, float* norms,
+                           int64_t outer, int64_t n_new, int64_t capacity, int64_t position,
+                           int D, void* stream);
+
+/*
  * Fused compress-and-store: compresses key and value rows and writes them straight
  * into the packed paged cache, one launch.  Takes the place of the two tq4_compress
  * calls, the row assembly and the advanced-index scatter of _compress_and_store
@@ -211,6 +228,23 @@ int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, const float* k
                           const float* rotation, int rotation_col_major, void* out,
                           int B, int H_Q, int H_KV, int N_Q, int N_KV, int D,
                           float sm_scale, int is_causal, int dtype, void* stream);
+
+/*
+ * The same with keys and values in pre-allocated buffers of a larger capacity: the views that
+ * the reference's ring buffer hands out, CompressedBuffer.get()
+ * (src/flashquant/cache/buffer_pool.py:128-140: indices[:, :, :len, :] of a (B, H, max_seq, D/2)
+ * buffer, norms likewise), go in without a copy (the fused mode of the HF cache,
+ * src/flashquant/cache/hf_cache.py:322-329, 387-414).
+ *   k_capacity, v_capacity   tokens between the slabs of consecutive (batch, KV head) pairs in
+ *                            the key and the value buffers (max_seq there), each >= N_KV
+ */
+int fq_fused_tq_attention_strided(const void* q, const uint8_t* k_packed, const float* k_norms,
+                                  const uint8_t* v_packed, const float* v_norms,
+                                  const float* centroids_k, const float* centroids_v,
+                                  const float* rotation, int rotation_col_major, void* out,
+                                  int B, int H_Q, int H_KV, int N_Q, int N_KV,
+                                  int64_t k_capacity, int64_t v_capacity, int D,
+                                  float sm_scale, int is_causal, int dtype, void* stream);
 
 /*
  * Prefill over the packed paged TQ4 cache: un-rotated queries of several

@@ -186,3 +186,57 @@ def test_paged_prefill_argument_errors(lib):
     assert call(S=-1) == FQ_SHAPE and call(MB=0) == FQ_SHAPE
     assert call() == FQ_NULL
     assert call(ptr=4096 + 8) == FQ_ALIGN
+
+
+def test_ring_buffer_and_rotated_decompress_argument_errors(lib):
+    ap = lib.fq_tq4_compress_append
+    ap.argtypes = ([ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 5 + [ctypes.c_int64] * 4 +
+                   [ctypes.c_int, ctypes.c_void_p])
+    assert ap(_p(), 1, _p(), _p(), _p(), _p(), _p(), 0, 5, 100, 0, 128, _p()) == FQ_OK        # no slabs: no-op
+    assert ap(_p(), 1, _p(), _p(), _p(), _p(), _p(), 4, 5, 100, 96, 128, _p()) == FQ_SHAPE    # 96 + 5 > capacity
+    assert ap(_p(), 1, _p(), _p(), _p(), _p(), _p(), 4, 5, 100, -1, 128, _p()) == FQ_SHAPE
+    assert ap(_p(), 1, _p(), _p(), _p(), _p(), _p(), 4, 5, 100, 10, 100, _p()) == FQ_DIM
+    assert ap(_p(), 2, _p(), _p(), _p(), _p(), _p(), 4, 5, 100, 10, 128, _p()) == FQ_DTYPE
+    assert ap(_p(), 1, _p(), _p(), _p(), _p(), _p(), 4, 5, 100, 10, 128, _p()) == FQ_NULL
+    at = lib.fq_fused_tq_attention_strided
+    at.argtypes = ([ctypes.c_void_p] * 8 + [ctypes.c_int, ctypes.c_void_p] + [ctypes.c_int] * 5 + [ctypes.c_int64] * 2 +
+                   [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
+
+    def att(nkv=64, kcap=64, vcap=64, d=128):
+        return at(_p(), _p(), _p(), _p(), _p(), _p(), _p(), _p(), 0, _p(), 1, 8, 2, 16, nkv, kcap, vcap, d, 0.1, 1, 1, _p())
+
+    assert att(kcap=63) == FQ_SHAPE and att(vcap=10) == FQ_SHAPE      # a capacity below the length
+    assert att(kcap=1000, vcap=2000) == FQ_NULL                       # accepted, then the NULL operands are found
+    assert att(d=96) == FQ_DIM
+    dr = lib.fq_tq4_decompress_rotated
+    dr.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                           ctypes.c_void_p]
+    assert dr(_p(), _p(), _p(), _p(), 0, _p(), 1, 0, 128, _p()) == FQ_OK
+    assert dr(_p(), _p(), _p(), _p(), 0, _p(), 2, 4, 128, _p()) == FQ_DTYPE     # float32 output: not offered
+    assert dr(_p(), _p(), _p(), _p(), 0, _p(), 1, 4, 100, _p()) == FQ_DIM
+    assert dr(_p(), _p(), _p(), _p(), 0, _p(), 1, 4, 128, _p()) == FQ_NULL
+    assert dr(_p(16), _p(16), _p(16), _p(16), 0, _p(8), 1, 4, 128, _p()) == FQ_ALIGN
+
+
+def test_static_scratch_decode_refuses_before_touching_the_gpu(lib):
+    lib.fq_static_scratch_bytes.restype = ctypes.c_size_t
+    assert lib.fq_static_scratch_bytes() == 16 << 20
+    f = lib.fq_split_k_paged_decode_static
+    f.argtypes = ([ctypes.c_void_p] * 7 + [ctypes.c_int, ctypes.c_void_p] + [ctypes.c_int] * 6 +
+                  [ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
+
+    def call(S=4, HQ=32, HKV=8, D=128, BS=16, MB=64, splits=0):
+        return f(_p(), _p(), _p(), _p(), _p(), _p(), _p(), 0, _p(), S, HQ, HKV, D, BS, MB, 100, 0.1, 1, splits, _p())
+
+    assert call(S=0) == FQ_OK
+    assert call(HQ=30) == FQ_SHAPE and call(D=100) == FQ_DIM and call(BS=12) == FQ_BLOCK
+    assert call(S=64, HQ=128, MB=4096, splits=256) == FQ_WS          # 1 GiB of partials against 16 MiB
+
+
+def test_option_switches(lib):
+    assert lib.fq_get_option(99) == -1 and lib.fq_set_option(99, 1) == FQ_SHAPE
+    for opt in range(3):
+        old = lib.fq_get_option(opt)
+        assert old in (0, 1)
+        assert lib.fq_set_option(opt, 1 - old) == FQ_OK and lib.fq_get_option(opt) == 1 - old
+        assert lib.fq_set_option(opt, old) == FQ_OK and lib.fq_get_option(opt) == old
