@@ -50,3 +50,4 @@ void* current_stream(const at::Tensor& like);
 void bind_kernels(pybind11::module_& m);
 void bind_codebook(pybind11::module_& m);
 void bind_quantizer(pybind11::module_& m);
+void bind_quantizer_classes(pybind11::module_& m);

@@ -12,4 +12,5 @@ PYBIND11_MODULE(_C, m) {
     bind_kernels(m);
     bind_codebook(m);
     bind_quantizer(m);
+    bind_quantizer_classes(m);
 }

@@ -5,6 +5,11 @@
 #include <ATen/CPUGeneratorImpl.h>
 
 #include <cmath>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include <pybind11/stl.h>
 
 #include "common.h"
 
@@ -183,13 +188,201 @@ at::Tensor project_rows(const at::Tensor& x, const at::Tensor& matrix, bool sign
     return out;
 }
 
+// ---------------------------------------------------------------------------------------
+// The class surface of the reference's C++ core (csrc/core/types.h:9-38, codebook.h:17-68,
+// quantizer.h:14-80, bound in csrc/bindings/codebook_bind.cpp:11-49 and quantizer_bind.cpp:10-64),
+// over this library's host set-up and GPU kernels: construction and the codebook live on the
+// host, the vectors on the GPU.
+// ---------------------------------------------------------------------------------------
+struct LloydMaxCodebook {
+    at::Tensor centroids;    // (2^bits,) float32
+    at::Tensor boundaries;   // (2^bits - 1,) float32
+    int dim = 0;
+    int bits = 0;
+};
+
+LloydMaxCodebook make_codebook(int dim, int bits) {
+    auto [c, b] = solve_lloyd_max(dim, bits);
+    return LloydMaxCodebook{c, b, dim, bits};
+}
+
+// torch.bucketize(x, boundaries) and centroids[indices] (csrc/core/codebook.cpp, codebook_quantize /
+// codebook_dequantize): plain tensor-library calls on whatever device the data is on.
+at::Tensor codebook_quantize(const at::Tensor& x, const at::Tensor& boundaries) {
+    return at::bucketize(x, boundaries.to(x.device()).contiguous());
+}
+at::Tensor codebook_dequantize(const at::Tensor& indices, const at::Tensor& centroids) {
+    return centroids.to(indices.device()).index({indices.to(at::kLong)});
+}
+
+class CodebookRegistry {
+public:
+    static CodebookRegistry& instance() {
+        static CodebookRegistry r;
+        return r;
+    }
+    LloydMaxCodebook get(int dim, int bits, const c10::Device& device) {
+        std::lock_guard<std::mutex> lock(mu_);
+        const std::string key = std::to_string(dim) + ":" + std::to_string(bits) + ":" + device.str();
+        auto it = cache_.find(key);
+        if (it != cache_.end()) return it->second;
+        LloydMaxCodebook cb = make_codebook(dim, bits);
+        cb.centroids = cb.centroids.to(device);
+        cb.boundaries = cb.boundaries.to(device);
+        cache_.emplace(key, cb);
+        return cb;
+    }
+    void warmup(const std::vector<int>& dims, const std::vector<int>& bits_options, const c10::Device& device) {
+        for (int d : dims)
+            for (int b : bits_options) get(d, b, device);
+    }
+    void clear() {
+        std::lock_guard<std::mutex> lock(mu_);
+        cache_.clear();
+    }
+
+private:
+    std::mutex mu_;
+    std::map<std::string, LloydMaxCodebook> cache_;
+};
+
+struct QuantizedMSE {
+    at::Tensor indices;   // (..., dim) int64
+    at::Tensor norms;     // (..., 1) float32
+};
+struct QuantizedProd {
+    at::Tensor indices;          // (..., dim) int64
+    at::Tensor norms;            // (..., 1) float32
+    at::Tensor qjl_signs;        // (..., dim) int8, +-1
+    at::Tensor residual_norms;   // (..., 1) float32
+};
+
+class TurboQuantMSE {
+public:
+    TurboQuantMSE(int dim, int bits, int64_t seed) : dim_(dim), bits_(bits) {
+        require(dim > 0, "dim must be positive");
+        require(bits >= 1 && bits <= 4, "bits must lie in 1..4");
+        rotation_ = haar_orthogonal(dim, seed);
+        codebook_ = make_codebook(dim, bits);
+    }
+    QuantizedMSE quantize(const at::Tensor& x) const {
+        require(x.dim() >= 1 && x.size(-1) == dim_, "the last dimension of x must be dim");
+        auto [idx, norms] = ::quantize(x, rotation_, codebook_.boundaries, bits_);
+        return QuantizedMSE{idx, norms};
+    }
+    at::Tensor dequantize(const at::Tensor& indices, const at::Tensor& norms) const {
+        return ::dequantize(indices, norms, rotation_, codebook_.centroids);
+    }
+    const at::Tensor& rotation() const { return rotation_; }
+    const LloydMaxCodebook& codebook() const { return codebook_; }
+    int dim() const { return dim_; }
+    int bits() const { return bits_; }
+
+private:
+    int dim_, bits_;
+    at::Tensor rotation_;        // (dim, dim) float32 on the CPU; moved to the data's device per call
+    LloydMaxCodebook codebook_;
+};
+
+class TurboQuantProd {
+public:
+    TurboQuantProd(int dim, int bits, int64_t seed)
+        : dim_(dim), bits_(bits), mse_(dim, bits >= 2 ? bits - 1 : 1, seed) {
+        require(bits >= 2, "TurboQuantProd requires bits >= 2 (1 bit for QJL), got " + std::to_string(bits));
+        sketch_ = qjl_matrix(dim, seed, std::nullopt);
+    }
+    // csrc/core/quantizer.cpp:99-139: (bits - 1)-bit indices and norms, the residual's norm, and the
+    // signs of the sketched residual as int8
+    QuantizedProd quantize(const at::Tensor& x) const {
+        const QuantizedMSE q = mse_.quantize(x);
+        auto [residual, gamma] = mse_residual(x, q.indices, q.norms, mse_.rotation(), mse_.codebook().centroids);
+        const at::Tensor signs = project_rows(residual, sketch_, true).to(at::kChar);
+        return QuantizedProd{q.indices, q.norms, signs, gamma};
+    }
+    at::Tensor dequantize(const at::Tensor& indices, const at::Tensor& norms) const {
+        return mse_.dequantize(indices, norms);
+    }
+    // <q, x_mse> + gamma sqrt(pi/2) / d <S q, signs>, one value per row (csrc/core/quantizer.cpp:148-184)
+    at::Tensor estimate_inner_product(const at::Tensor& query, const QuantizedProd& c) const {
+        require(query.dim() >= 1 && query.size(-1) == dim_, "the last dimension of query must be dim");
+        const at::Tensor q2 = query.reshape({-1, dim_});
+        const at::Tensor x_mse = mse_.dequantize(c.indices, c.norms).reshape({-1, dim_});
+        const at::Tensor mse_term = at::sum(q2.to(at::kFloat) * x_mse, {-1}, true);
+        const at::Tensor q_proj = project_rows(q2, sketch_, false);
+        const at::Tensor dot = at::sum(q_proj * c.qjl_signs.reshape({-1, dim_}).to(at::kFloat), {-1}, true);
+        const at::Tensor scale = c.residual_norms.reshape({-1, 1}) * (1.2533141373155003 / double(dim_));
+        auto shape = query.sizes().vec();
+        shape.back() = 1;
+        return (mse_term + scale * dot).reshape(shape);
+    }
+    const TurboQuantMSE& mse_quantizer() const { return mse_; }
+    const at::Tensor& sketch() const { return sketch_; }
+    int dim() const { return dim_; }
+    int bits() const { return bits_; }
+
+private:
+    int dim_, bits_;
+    TurboQuantMSE mse_;
+    at::Tensor sketch_;          // (dim, dim) float32 on the CPU
+};
+
 }  // namespace
 
 void bind_codebook(py::module_& m) {
-    py::module_ cb = m.def_submodule("codebook", "Lloyd-Max codebook solver (host)");
+    py::module_ cb = m.def_submodule("codebook", "Lloyd-Max codebook (host)");
+    // The two solvers return the (centroids, boundaries) tuple that the reference's Python layer
+    // unpacks (src/flashquant/core/codebook.py:148-149), not the struct of the reference's C++.
     cb.def("solve_lloyd_max", &solve_lloyd_max, py::arg("dim"), py::arg("bits"),
            "(centroids, boundaries) float32 CPU tensors for N(0, 1/dim) truncated to +-3.5 sigma");
     cb.def("gaussian_lloyd_max", &solve_lloyd_max, py::arg("dim"), py::arg("bits"));
+    py::class_<LloydMaxCodebook>(cb, "LloydMaxCodebook")
+        .def(py::init(&make_codebook), py::arg("dim"), py::arg("bits"))
+        .def_readwrite("centroids", &LloydMaxCodebook::centroids)
+        .def_readwrite("boundaries", &LloydMaxCodebook::boundaries)
+        .def_readonly("dim", &LloydMaxCodebook::dim)
+        .def_readonly("bits", &LloydMaxCodebook::bits);
+    cb.def("quantize", &codebook_quantize, py::arg("x"), py::arg("boundaries"),
+           "Bucket index of every value: the number of boundaries below it");
+    cb.def("dequantize", &codebook_dequantize, py::arg("indices"), py::arg("centroids"), "centroids[indices]");
+    py::class_<CodebookRegistry>(cb, "CodebookRegistry")
+        .def_static("instance", &CodebookRegistry::instance, py::return_value_policy::reference)
+        .def("get", [](CodebookRegistry& self, int dim, int bits, c10::Device device) { return self.get(dim, bits, device); },
+             py::arg("dim"), py::arg("bits"), py::arg("device"))
+        .def("warmup", [](CodebookRegistry& self, const std::vector<int>& dims, const std::vector<int>& bits_options,
+                          c10::Device device) { self.warmup(dims, bits_options, device); },
+             py::arg("dims"), py::arg("bits_options"), py::arg("device"))
+        .def("clear", &CodebookRegistry::clear);
+}
+
+void bind_quantizer_classes(py::module_& m) {
+    py::module_ q = m.def_submodule("quantizer", "TurboQuant quantizers: set-up on the host, vectors on the GPU");
+    py::class_<QuantizedMSE>(q, "QuantizedMSE")
+        .def_readwrite("indices", &QuantizedMSE::indices)
+        .def_readwrite("norms", &QuantizedMSE::norms);
+    py::class_<QuantizedProd>(q, "QuantizedProd")
+        .def_readwrite("indices", &QuantizedProd::indices)
+        .def_readwrite("norms", &QuantizedProd::norms)
+        .def_readwrite("qjl_signs", &QuantizedProd::qjl_signs)
+        .def_readwrite("residual_norms", &QuantizedProd::residual_norms);
+    py::class_<TurboQuantMSE>(q, "TurboQuantMSE")
+        .def(py::init<int, int, int64_t>(), py::arg("dim"), py::arg("bits"), py::arg("seed") = 42)
+        .def("quantize", &TurboQuantMSE::quantize, py::arg("x"), "QuantizedMSE(indices int64, norms float32) of GPU rows")
+        .def("dequantize", &TurboQuantMSE::dequantize, py::arg("indices"), py::arg("norms"),
+             "float32 rows in the original space")
+        .def_property_readonly("dim", &TurboQuantMSE::dim)
+        .def_property_readonly("bits", &TurboQuantMSE::bits)
+        .def("rotation", [](const TurboQuantMSE& self) { return self.rotation(); })
+        .def("codebook", [](const TurboQuantMSE& self) { return self.codebook(); });
+    py::class_<TurboQuantProd>(q, "TurboQuantProd")
+        .def(py::init<int, int, int64_t>(), py::arg("dim"), py::arg("bits"), py::arg("seed") = 42)
+        .def("quantize", &TurboQuantProd::quantize, py::arg("x"), "QuantizedProd with int8 signs")
+        .def("dequantize", &TurboQuantProd::dequantize, py::arg("indices"), py::arg("norms"),
+             "Reconstruction from the (bits - 1)-bit stage alone")
+        .def("estimate_inner_product", &TurboQuantProd::estimate_inner_product, py::arg("query"), py::arg("compressed"),
+             "<q, x_mse> + gamma sqrt(pi/2) / d <S q, signs>, shape (..., 1)")
+        .def_property_readonly("dim", &TurboQuantProd::dim)
+        .def_property_readonly("bits", &TurboQuantProd::bits)
+        .def("qjl_matrix", [](const TurboQuantProd& self) { return self.sketch(); });
 }
 
 void bind_quantizer(py::module_& m) {

@@ -130,3 +130,60 @@ def test_quantizer_classes_hold_reference_state_and_refuse_cpu_tensors():
         core.TurboQuantMSE(64, 2).dequantize(torch.zeros(2, 64, dtype=torch.long), torch.ones(2, 1))
     assert core.KeyCompressor(128).quantizer.mse_quantizer.bits == 3
     assert torch.equal(core.ValueCompressor(128).quantizer.rotation, O.haar_orthogonal(128, 43))
+
+
+# ---- page-size arithmetic of the serving backend (no vLLM needed) -------------------------------
+
+def test_cache_spec_arithmetic_matches_the_reference_formulas():
+    from flashquant_amd import vllm as V
+    # src/flashquant/vllm/spec.py:30-44: head_dim // 2 + 4 per K or V; twice that per token and head
+    assert V.TQ4_NORM_BYTES == 4
+    assert V.tq4_bytes_per_token(128) == 68 and V.tq4_bytes_per_token_kv(128) == 136
+    assert V.tq4_bytes_per_token(64) == 36 and V.tq4_bytes_per_token_kv(256) == 264
+    # src/flashquant/vllm/impl.py:132-138
+    assert V.tq4_row_offsets(8, 128) == (512, 544, 1056, 1088)
+    assert V.tq4_row_offsets(2, 64) == (64, 72, 136, 144)
+    # src/flashquant/vllm/backend.py:124-138, spec.py:60-66
+    assert V.get_kv_cache_shape(1000, 16, 8, 128) == (1000, 16, 1088)
+    assert V.real_page_size_bytes(16, 8, 128) == 17408
+    # the compression ratio the reference logs: fp16 K and V against the packed row (3.76x)
+    assert abs(2 * 8 * 128 * 2 / V.tq4_row_offsets(8, 128)[3] - 3.7647) < 1e-3
+    # TurboQuantProd pages of this library: 12 more bytes per head than head_dim
+    assert V.prod_bytes_per_token_kv(128) == 140 and V.prod_kv_cache_shape(10, 16, 8, 128) == (10, 16, 1120)
+    from oracle import tq_oracle as O
+    assert O.page_layout(8, 128) == V.tq4_row_offsets(8, 128)
+    assert O.prod_page_layout(8, 128)[4] == 8 * V.prod_bytes_per_token_kv(128)
+    with pytest.raises(ImportError):
+        V.get_flashquant_attention_spec()            # vLLM is not installed here
+
+
+def test_quantizer_and_codebook_class_surface_on_the_host():
+    """_C.codebook / _C.quantizer carry the classes of the reference's C++ bindings
+    (csrc/bindings/codebook_bind.cpp:11-49, quantizer_bind.cpp:10-64); construction and the
+    codebook helpers run on the host."""
+    from oracle import tq_oracle as O
+    C = flashquant_amd.load_native()
+    cb = C.codebook.LloydMaxCodebook(128, 4)
+    c, b = O.lloyd_max_gaussian(128, 4)
+    assert cb.dim == 128 and cb.bits == 4 and torch.equal(cb.centroids, c) and torch.allclose(cb.boundaries, b, atol=1e-12)
+    x = torch.tensor([-1.0, -0.01, 0.0, 0.3, 1.0])
+    # (the middle boundary is 0 up to 1e-16 on either side: compare on this codebook's own values)
+    assert torch.equal(C.codebook.quantize(x, cb.boundaries), torch.bucketize(x, cb.boundaries))
+    assert C.codebook.quantize(torch.tensor([-1.0, -0.01, 0.3, 1.0]), cb.boundaries).tolist() == [0, 7, 15, 15]
+    idx = torch.tensor([[0, 5], [15, 8]])
+    assert torch.equal(C.codebook.dequantize(idx, cb.centroids), c[idx])
+    reg = C.codebook.CodebookRegistry.instance()
+    got = reg.get(64, 3, torch.device("cpu"))
+    assert got.bits == 3 and got.centroids.shape == (8,) and torch.equal(got.centroids, O.lloyd_max_gaussian(64, 3)[0])
+    reg.warmup([128], [2, 4], torch.device("cpu"))
+    reg.clear()
+    q = C.quantizer.TurboQuantMSE(128, 4, 42)
+    assert q.dim == 128 and q.bits == 4 and torch.equal(q.rotation(), O.haar_orthogonal(128, 42))
+    p = C.quantizer.TurboQuantProd(128, 4)
+    assert p.dim == 128 and p.bits == 4 and torch.equal(p.qjl_matrix(), O.qjl_matrix(128, 42))
+    with pytest.raises(ValueError):
+        C.quantizer.TurboQuantProd(128, 1)
+    with pytest.raises(ValueError, match="GPU"):
+        q.quantize(torch.zeros(2, 128))
+    for name in ("QuantizedMSE", "QuantizedProd"):
+        assert hasattr(C.quantizer, name)
