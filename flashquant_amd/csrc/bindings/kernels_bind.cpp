@@ -48,6 +48,7 @@ int option_id(const std::string& name) {
     if (name == "decode_copy_waves") return FQ_OPT_DECODE_COPY_WAVES;
     if (name == "decode_direct") return FQ_OPT_DECODE_DIRECT;
     if (name == "attention_any_dim") return FQ_OPT_ATTENTION_ANY_DIM;
+    if (name == "decode_tiny_spin") return FQ_OPT_DECODE_TINY_SPIN;
     throw std::invalid_argument("unknown option '" + name + "'");
 }
 

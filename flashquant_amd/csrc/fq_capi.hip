@@ -22,6 +22,7 @@ void init_options() {
         g_options[FQ_OPT_DECODE_DIRECT] = (v != nullptr && v[0] == '1') ? 1 : 0;
         v = std::getenv("FQ_ATTENTION_ANY_DIM");
         g_options[FQ_OPT_ATTENTION_ANY_DIM] = (v != nullptr && v[0] == '1') ? 1 : 0;
+        g_options[FQ_OPT_DECODE_TINY_SPIN] = 0;
     });
 }
 }  // namespace

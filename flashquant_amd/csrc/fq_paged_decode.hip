@@ -83,6 +83,7 @@ struct DecodeParams {
     int num_splits;
     int two_tables;             // centroids_v differs from centroids_k
     float scale_log2e;          // sm_scale * log2(e)
+    int spin_limit;             // staged kernel: polls of a bounded wait between wavefronts before it gives up
     int balance_slots;          // staged kernel: > 0 lets the workgroups size the token chunks from the actual
                                 // sequence lengths, for this many workgroups running at a time (num_seqs <= 64)
 };
@@ -519,13 +520,15 @@ __global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p)
 // the banks; the eight rows read together by a K operand load fall in eight different
 // 16-byte bank groups; the eight chunks a quarter-wave writes together do too).
 //
-// Pipeline, one workgroup barrier per tile.  With copy wavefronts (CW = 4, the default) four
-// more wavefronts do nothing but move tiles: each keeps two tiles in flight in registers and
-// writes tile i + 1 to the LDS slot that tile i - 1 has just left, while the eight computing
-// wavefronts consume tile i and never wait for global memory.  Without them (CW = 0) the eight
-// wavefronts do both: at iteration i the registers holding tile i + 1 (loaded during
-// iteration i - 1) are written to the free slot, the loads of tile i + 2 are issued, and tile
-// i is consumed from LDS.
+// Pipeline.  With copy wavefronts (CW = 4, the default) four more wavefronts do nothing but
+// move tiles: each keeps two tiles in flight in registers and writes a tile to an LDS slot as
+// soon as the eight computing wavefronts have read the slot's previous tile into registers,
+// which they do at the very start of a tile; the computing wavefronts never wait for global
+// memory.  The two sides meet through counting flags in LDS (a bounded buffer of two slots), not
+// through workgroup barriers, so no wavefront waits for one that it does not depend on.  Without
+// copy wavefronts (CW = 0) the eight wavefronts do both, one workgroup barrier per tile: at
+// iteration i the registers holding tile i + 1 (loaded during iteration i - 1) are written to the
+// free slot, the loads of tile i + 2 are issued, and tile i is consumed from LDS.
 // A tile is 32 tokens: two 16-token blocks; with 4 query heads per KV head the 16 MFMA
 // columns carry (head, block, half of the block's rows), so that all lanes own distinct
 // (head, token) scores.
@@ -610,8 +613,8 @@ __device__ __forceinline__ void lds_flag_signal(uint32_t* flag, int lane) {
 // Returns false when the count was not reached within the bound: the caller records the failed
 // hand-off (the workgroup then publishes NaN partials and raises the library's fault counter)
 // instead of going on silently with operands that are not there yet.
-__device__ __forceinline__ bool lds_flag_wait(uint32_t* flag, uint32_t count) {
-    for (int spin = 0; spin < (1 << 20); ++spin) {
+__device__ __forceinline__ bool lds_flag_wait(uint32_t* flag, uint32_t count, int spin_limit) {
+    for (int spin = 0; spin < spin_limit; ++spin) {
         if (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= count) return true;
         __builtin_amdgcn_s_sleep(1);
     }
@@ -641,11 +644,15 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // that folds into the offset field of every lookup; the tile slots are dynamic.
     __shared__ __attribute__((aligned(256))) uint32_t lut[kLutWords];
     extern __shared__ __attribute__((aligned(16))) uint8_t slots[];   // two tile slots
-    __shared__ uint32_t flags[3];   // CW > 0: rotated heads stored / sketched heads read back / a hand-off timed out
+    // CW > 0: [0] rotated heads stored, [1] rotated (and sketched) heads read back, [2] a hand-off timed
+    // out, [3 + s] tiles written to slot s (one count per copy wavefront and tile), [5 + s] tiles read
+    // from slot s (one count per computing wavefront and tile)
+    __shared__ uint32_t flags[7];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int h = __builtin_amdgcn_readfirstlane(tid >> 6);   // wavefront = KV head
+    bool handoff_failed = false;                             // a bounded wait of this wavefront ran out
     // CW > 0: wavefronts 8 .. 8 + CW - 1 only move tiles from the cache to LDS and the first eight
     // only consume them, so that no wavefront that computes ever waits for global memory.
     const bool copier = CW > 0 && h >= 8;
@@ -856,7 +863,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         // The flags are cleared behind a barrier placed where nobody waits for anybody: every
         // wavefront has just asked for its sequence length and page ids and none has used them yet
         // (the barrier does not wait for loads from global memory).
-        if (tid == 0) { flags[0] = 0u; flags[1] = 0u; flags[2] = 0u; }
+        if (tid < 7) flags[tid] = 0u;
         __syncthreads();
         load_matrix_columns();
         load_first_heads();
@@ -1002,21 +1009,26 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             for (int k = 0; k < NR; ++k) ra[k] = rb[k] = uint4v{0u, 0u, 0u, 0u};
             c_issue(ra, begin);
             c_issue(rb, begin + 32);
-            // The query exchange of the computing wavefronts goes through the second slot and, with a
-            // sketch, the first: that one is free when all eight have read their sketched heads back.
-            if constexpr (PROD) {
-                if (p.rotation != nullptr && !lds_flag_wait(&flags[1], 8u)) flags[2] = 1u;
-            }
-            c_write(0, ra);
-            c_issue(ra, begin + 64);
-            for (int t0 = begin; t0 < end; t0 += 64) {
-                __syncthreads();                      // tile i is in LDS; the slot of tile i - 1 is free
-                c_write(1, rb);                       // tile i + 1
-                c_issue(rb, t0 + 96);                 // tile i + 3
-                if (t0 + 32 >= end) break;
-                __syncthreads();
-                c_write(0, ra);                       // tile i + 2
-                c_issue(ra, t0 + 128);                // tile i + 4
+            // Producer side of a bounded buffer of two LDS slots, synchronised with counting flags
+            // instead of workgroup barriers: the copy and the computing wavefronts are not in step
+            // with each other, nor the computing wavefronts among themselves.  Tile j goes to slot
+            // j % 2, which last held tile j - 2: it is free when all eight computing wavefronts have
+            // read j / 2 tiles from it (none can be further: tile j is not there yet).  The query
+            // exchange of the computing wavefronts goes through the second slot and, with a sketch,
+            // the first: the first write to those waits until all eight have read their heads back.
+            int j = 0;
+            for (int t0 = begin; t0 < end; t0 += 32, ++j) {
+                if (j >= 2 && !lds_flag_wait(&flags[5 + (j & 1)], 8u * uint32_t(j >> 1), p.spin_limit)) flags[2] = 1u;
+                if (p.rotation != nullptr && j == (PROD ? 0 : 1) && !lds_flag_wait(&flags[1], 8u, p.spin_limit)) flags[2] = 1u;
+                if (j & 1) {
+                    c_write(1, rb);
+                    lds_flag_signal(&flags[4], lane);
+                    c_issue(rb, t0 + 64);
+                } else {
+                    c_write(0, ra);
+                    lds_flag_signal(&flags[3], lane);
+                    c_issue(ra, t0 + 64);
+                }
             }
             return;
         }
@@ -1094,7 +1106,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             }
             if constexpr (CW > 0) {
                 lds_flag_signal(&flags[0], lane);
-                if (!lds_flag_wait(&flags[0], 8u)) flags[2] = 1u;
+                if (!lds_flag_wait(&flags[0], 8u, p.spin_limit)) { flags[2] = 1u; handoff_failed = true; }
             } else {
                 __syncthreads();
             }
@@ -1132,10 +1144,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
                     for (int e = 0; e < 8; ++e) qsh[ks][e] = _Float16(qf2[ks][e] * down2);
             }
-            if constexpr (PROD) {                  // the first slot is about to receive a tile
-                if constexpr (CW > 0) lds_flag_signal(&flags[1], lane);
-                else __syncthreads();
-            }
+            // the heads are read back: the slots they went through may receive tiles
+            if constexpr (CW > 0) lds_flag_signal(&flags[1], lane);
+            else if constexpr (PROD) __syncthreads();
         } else {
             const uint16_t* qsrc = qseq + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
@@ -1186,6 +1197,10 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageVnOff - kStageKnOff));
             kg[e] = PROD ? *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageKgOff - kStageKnOff)) : 0.0f;
         }
+        // These were all the reads of the slot (the lookups below go to the table): it is handed back
+        // to the copy wavefronts here, long before the tile's arithmetic is done (the release waits
+        // for the reads to complete).
+        if constexpr (CW > 0) lds_flag_signal(&flags[5 + slot], lane);
 
         // ---- scores: lookups of block 1 in flight during the MFMAs of block 0 ----------------
         uint4v ka[2][KS];
@@ -1357,7 +1372,11 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     } else {
         int i = 0;
         for (int t0 = begin; t0 < end; t0 += 32, ++i) {
-            __syncthreads();                      // the copy wavefronts have put tile i in LDS
+            // consumer side: tile i is complete when every copy wavefront has written its part of it
+            if (!lds_flag_wait(&flags[3 + (i & 1)], uint32_t(CW) * uint32_t((i >> 1) + 1), p.spin_limit)) {
+                flags[2] = 1u;
+                handoff_failed = true;
+            }
             compute_tile(t0, i & 1);
         }
     }
@@ -1378,11 +1397,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             O[db][i] = v;
         }
     if constexpr (CW > 0) {
-        // a hand-off of the prologue that timed out (the tile barriers since then make the word
-        // visible): the result cannot be trusted, so it is made NaN and the fault is counted
-        if (__builtin_amdgcn_readfirstlane(flags[2]) != 0u) {
+        // a hand-off that timed out, in the prologue or in the tile loop: the result cannot be
+        // trusted, so it is made NaN and the fault is counted
+        if (handoff_failed ||
+            __builtin_amdgcn_readfirstlane(__hip_atomic_load(&flags[2], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) != 0u) {
             M = __builtin_nanf("");
-            if (tid == 0) atomicAdd(&g_decode_faults, 1u);
+            if (handoff_failed && lane == 0) atomicAdd(&g_decode_faults, 1u);
         }
     }
     if (g == 0 && n < p.G) {
@@ -1470,6 +1490,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
         const int64_t row = row0 + r < rows ? row0 + r : rows - 1;
         const int64_t base = row * NS;
         float mstar = -__builtin_inff();
+        bool poisoned = false;      // a split published NaN as its maximum: its workgroup could not vouch for it
         // bit c: the chunk of eight splits c (mod 64) holds a split that wrote something.  Splits
         // beyond a sequence's length are empty (m = -inf), whole chunks of them when the split count
         // was chosen for the longest possible context: those are not read at all.
@@ -1490,6 +1511,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
                 for (int k = 0; k < 4; ++k) {
                     const int idx = s0 + t16 + 16 * k;
                     const bool wrote = idx < NS && mv[k] != -__builtin_inff();
+                    poisoned = poisoned || (idx < NS && mv[k] != mv[k]);
                     mstar = wrote ? __builtin_fmaxf(mstar, mv[k]) : mstar;
                     const int chunk = (idx >> 3) & 63;
                     live_lo |= (wrote && chunk < 32) ? 1u << chunk : 0u;
@@ -1499,6 +1521,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
 #pragma unroll
             for (int mask = 1; mask < 16; mask <<= 1) {
                 mstar = __builtin_fmaxf(mstar, xor_shuffle(mstar, mask));
+                poisoned = poisoned || __shfl_xor(int(poisoned), mask, kWave) != 0;
                 live_lo |= uint32_t(__shfl_xor(int(live_lo), mask, kWave));
                 live_hi |= uint32_t(__shfl_xor(int(live_hi), mask, kWave));
             }
@@ -1526,7 +1549,10 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
                 }
                 if (NS <= 8) {
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) mstar = __builtin_fmaxf(mstar, mv[k]);
+                    for (int k = 0; k < 8; ++k) {
+                        mstar = __builtin_fmaxf(mstar, mv[k]);
+                        poisoned = poisoned || mv[k] != mv[k];
+                    }
                 }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
@@ -1544,8 +1570,9 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
             uint32_t wds[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t a0 = live ? store_elem<DT>(num[2 * e] / den) : 0u;
-                const uint32_t a1 = live ? store_elem<DT>(num[2 * e + 1] / den) : 0u;
+                // a poisoned row comes out NaN, never as a plausible number
+                const uint32_t a0 = poisoned ? store_elem<DT>(__builtin_nanf("")) : (live ? store_elem<DT>(num[2 * e] / den) : 0u);
+                const uint32_t a1 = poisoned ? store_elem<DT>(__builtin_nanf("")) : (live ? store_elem<DT>(num[2 * e + 1] / den) : 0u);
                 wds[e] = a0 | (a1 << 16);
             }
             *reinterpret_cast<uint4v*>(&os[r * OSTRIDE + c0]) = uint4v{wds[0], wds[1], wds[2], wds[3]};
@@ -1849,6 +1876,7 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
     p.two_tables = centroids_k != centroids_v ? 1 : 0;
     p.scale_log2e = sm_scale * kLog2e;
     p.balance_slots = 0;
+    p.spin_limit = fq_host::option(FQ_OPT_DECODE_TINY_SPIN) != 0 ? 2 : (1 << 20);
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define FQ_DECODE_D(DD)                                                                 \
     case DD:                                                                            \
@@ -2052,6 +2080,7 @@ extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, cons
     p.two_tables = 1;
     p.scale_log2e = sm_scale * kLog2e;
     p.balance_slots = staged_balance_slots(num_seqs, num_splits);
+    p.spin_limit = fq_host::option(FQ_OPT_DECODE_TINY_SPIN) != 0 ? 2 : (1 << 20);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t max_ctx = int64_t(max_blocks_per_seq) * block_size;
     const int64_t chunk = (((max_ctx + num_splits - 1) / num_splits) + 63) & ~int64_t(63);

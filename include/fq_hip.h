@@ -55,7 +55,10 @@ typedef enum fq_option {
                                      decode kernel                                                      */
     FQ_OPT_ATTENTION_ANY_DIM = 2, /* FQ_ATTENTION_ANY_DIM, default 0: 1 sends head_dim 128 to the general
                                      attention kernel                                                   */
-    FQ_OPTION_COUNT = 3
+    FQ_OPT_DECODE_TINY_SPIN = 3,  /* default 0: 1 makes the bounded waits between the wavefronts of the staged
+                                     decode kernel give up after two polls, to exercise the failure path
+                                     (NaN rows, fault counter) without hanging anything                */
+    FQ_OPTION_COUNT = 4
 } fq_option;
 int fq_get_option(int option);
 int fq_set_option(int option, int value);

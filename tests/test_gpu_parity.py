@@ -284,6 +284,29 @@ def test_paged_decode_fp16_and_large_norms():
     _decode_case([100, 33], hq=8, hkv=2, kv_scale=1e-3)
 
 
+def test_paged_decode_failed_handoff_is_loud(kernel_option):
+    """The wavefronts of the staged kernel meet through bounded waits.  With the bound forced down
+    to two polls from the host the waits give up: every wavefront still runs to the end (nothing
+    hangs), the affected rows come out NaN instead of silently wrong, and the fault counter moves.
+    With the bound back to normal the same call is correct again."""
+    C = load_native()
+    c, b, r = book(128)
+    q, cache, table, sl = build_paged_case([700, 300], 32, 8, seed=51)
+    dev = [t.to(DEV) for t in (q, cache, table, sl, c, r)]
+    want = O.split_k_paged_decode(q, cache, table, sl, c, c, r, 8, 128, 16)
+    before = C.paged_decode_fault_count()
+    kernel_option("decode_tiny_spin", True)
+    bad = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], 8, 128, 16, num_splits=1)
+    torch.cuda.synchronize()
+    assert C.paged_decode_fault_count() > before
+    assert torch.isnan(bad.float()).any()
+    wrong_but_finite = (~torch.isnan(bad.float())) & ((bad.cpu().float() - want.float()).abs() > 2e-2).to(DEV)
+    assert not wrong_but_finite.any()                     # a row is either right or NaN
+    kernel_option("decode_tiny_spin", False)
+    good = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], 8, 128, 16, num_splits=1)
+    assert (good.cpu().float() - want.float()).abs().max().item() <= 2e-2
+
+
 def test_paged_decode_more_kv_heads_than_a_workgroup():
     _decode_case([50, 120], hq=24, hkv=12, num_splits=2)
 
