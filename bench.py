@@ -97,6 +97,20 @@ def time_events(fn, iters):
     return median, marks[0].elapsed_time(marks[iters]) / iters
 
 
+def time_region(fn, iters):
+    """Average time of a call in ms from two GPU events, one before the first and one after the last of
+    `iters` back-to-back calls on torch's current stream (no event between the calls: an event between
+    two launches costs the stream a barrier packet of its own, about 2 us here)."""
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    first.record()
+    for i in range(iters):
+        fn(i)
+    last.record()
+    torch.cuda.synchronize()
+    return first.elapsed_time(last) / iters
+
+
 def committed_traffic(kernel_prefix):
     """HBM bytes per launch of the dominant kernel as the committed counter summary states them
     (a line `TRAFFIC_BYTES_PER_LAUNCH <kernel> <bytes>` in profiles/paged_decode_hbm_traffic_pmc.txt,
@@ -181,7 +195,8 @@ def main():
 
     for i in range(args.warmup):
         decode_only(i)
-    _, kern_ms = time_events(decode_only, args.steps)      # average launch duration
+    kern_ms = time_region(decode_only, args.steps)         # average launch duration
+    _, kern_each_ms = time_events(decode_only, args.steps)
     achieved = kv_bytes / (kern_ms * 1e-3) / 1e9
 
     extra = {
@@ -193,6 +208,7 @@ def main():
         "decode_gbps_warm": kv_bytes / (warm_ms * 1e-3) / 1e9,
         "decode_pct_hbm_peak_cold": 100.0 * kv_bytes / (step_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "decode_kernel_us_cold": kern_ms * 1e3,
+        "decode_kernel_us_cold_event_per_launch": kern_each_ms * 1e3,
         "num_splits": n_splits,
         "kv_bytes_per_step": kv_bytes,
     }
