@@ -240,3 +240,34 @@ def test_option_switches(lib):
         assert old in (0, 1)
         assert lib.fq_set_option(opt, 1 - old) == FQ_OK and lib.fq_get_option(opt) == 1 - old
         assert lib.fq_set_option(opt, old) == FQ_OK and lib.fq_get_option(opt) == old
+
+
+def test_shape_limits_of_the_staged_and_prod_decodes(lib):
+    """What the kernels cover is a status code at the boundary, not a wrong result: TurboQuantProd pages
+    come with 8 KV heads of dimension 128 and at most 64 query heads (the kernel stages 8 heads per token
+    row); the query group is at most 16 heads; the staged TQ4 kernel (the one that rotates the query
+    itself) serves 8 KV heads of dimension 128 and every other shape runs the direct kernel."""
+    f = lib.fq_prod_paged_decode
+    f.argtypes = ([ctypes.c_void_p] * 7 + [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 6 +
+                  [ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                   ctypes.c_void_p])
+
+    def prod(S=2, HQ=32, HKV=8, D=128, BS=16, MB=4, NB=64, dtype=1, ptr=0):
+        return f(_p(ptr), _p(ptr), _p(ptr), _p(ptr), _p(ptr), _p(ptr), _p(ptr), 0, _p(ptr), _p(ptr), S, HQ, HKV, D, BS,
+                 MB, NB, 0.088, dtype, 0, _p(), 0, _p())
+
+    assert prod(S=0) == FQ_OK
+    assert prod(D=64) == FQ_DIM and prod(D=256) == FQ_DIM
+    assert prod(HKV=4, HQ=16) == FQ_SHAPE
+    assert prod(HQ=128) == FQ_SHAPE           # more than 64 query heads
+    assert prod(HQ=8 * 17) == FQ_SHAPE
+    assert prod() == FQ_NULL                  # a supported shape gets as far as the pointer check
+    lib.fq_paged_decode_fuses_rotation.argtypes = [ctypes.c_int] * 3
+    assert lib.fq_paged_decode_fuses_rotation(128, 8, 1) == 1
+    for d, hkv in ((64, 8), (256, 8), (128, 4), (128, 16), (128, 2)):
+        assert lib.fq_paged_decode_fuses_rotation(d, hkv, 1) == 0
+    # a pre-rotated query with a rotation matrix is only accepted where the kernel rotates it
+    g = lib.fq_paged_tq4_decode
+    g.argtypes = ([ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 8 + [ctypes.c_int] * 6 +
+                  [ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
+    assert g(_p(4096), _p(4096), 0, *([_p(4096)] * 8), 2, 16, 4, 128, 16, 4, 64, 0.088, 1, 1, _p()) == FQ_SHAPE
