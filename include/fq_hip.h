@@ -66,7 +66,10 @@ int fq_set_option(int option, int value);
 /* Library identification and error text. */
 int fq_abi_version(void);
 const char* fq_status_string(int status);
-/* Text of the last HIP runtime error seen by this thread ("" if none). */
+/* Text of the last HIP runtime error seen by this thread ("" if none).  An entry point that launches asks
+ * the runtime for its last error after the launch (hipGetLastError, which also clears it): an error that
+ * an earlier HIP call of the same thread left behind is therefore reported, as FQ_ERR_LAUNCH, by the next
+ * entry point called, whose own launch may have been fine; this text names the error either way. */
 const char* fq_last_hip_error(void);
 
 /*
