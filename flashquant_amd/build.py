@@ -29,6 +29,15 @@ HIP_FLAGS = [
 ]
 
 
+# Per-file additions.  The compress and decompress-with-rotation kernels consume their MFMA results in
+# the vector ALU right away: with the accumulators in ordinary vector registers (instead of the
+# accumulation registers the compiler picks under register pressure) there is no copy between the two.
+FILE_FLAGS = {
+    "fq_compress.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "fq_decompress_rotate.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     lines = [ln for ln in r.stdout.splitlines() if "is not a recognized feature for this target" not in ln]
@@ -44,7 +53,7 @@ def build_hip(verbose: bool = True) -> str:
 
     def one(pair):
         src, obj = pair
-        out = _run(["hipcc", *HIP_FLAGS, "-c", src, "-o", obj])
+        out = _run(["hipcc", *HIP_FLAGS, *FILE_FLAGS.get(os.path.basename(src), []), "-c", src, "-o", obj])
         if verbose and out.strip():
             print(out)
         return obj
