@@ -163,8 +163,17 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const uint8_t* vp = p.v_packed + v_row0 * 64;
     const float* knp = p.k_norms + k_row0;
     const float* vnp = p.v_norms + v_row0;
-    const int tk = tid >> 3, gqk = tid & 7;        // K: token of the tile, 16-coordinate group
-    const int tp = tid >> 4, jv = tid & 15;        // V: token pair of the tile, dword of the row
+    // K: token of the tile and 16-coordinate group.  Lane bits (g0 g1 t0 g2 t1 t2): eight consecutive
+    // lanes hold four groups of two consecutive tokens, so the 128 bytes they store with one 16-byte
+    // write each fall into 32 different banks (token rows are 272 bytes apart: 4 banks).
+    const int gqk = (lane & 3) | ((lane >> 1) & 4);
+    const int tk = 8 * w + ((lane >> 2) & 1) + ((lane >> 3) & 6);
+    // V: token pair of the tile and dword of the packed row.  The four pairs of a wavefront are the
+    // ones whose positions share a 16-byte group of the transposed tile (0, 2, 4, 6 within it), so
+    // that a store of half a wavefront covers all 32 banks once.
+    // Lane bits (j0 j1 j2 p0 p1 j3): each half of the wavefront holds all four pairs and eight dwords.
+    const int jv = (lane & 7) | ((lane >> 2) & 8);
+    const int tp = 8 * (w >> 1) + 2 * (w & 1) + ((lane >> 3) & 1) + 4 * ((lane >> 4) & 1);
     const int k_wr = tk * kPfKStride + gqk * 32;
     int v_wr[8];
     {
