@@ -1,5 +1,6 @@
-// Fused TQ4 FlashAttention (prefill) for gfx950: un-rotated query in, packed TQ4
-// keys and values in, original-space output out.
+// Fused TQ4 FlashAttention (prefill) for gfx950, head_dim 64 and 128: un-rotated query in,
+// packed TQ4 keys and values in, original-space output out.  (The figures in this comment are
+// those of head_dim 128.)
 //
 // Operator: fused_tq_attention_reference
 // (src/flashquant/kernels/cpu_reference.py:154-227) as dispatched by
@@ -38,11 +39,19 @@
 
 namespace fq {
 
-constexpr int kPfKStride = 272;                       // bytes per token row of the K tile (128 fp16 + pad)
-constexpr int kPfKBytes = 64 * kPfKStride;            // 17408
-constexpr int kPfVBytes = 128 * 128;                  // V^T tile: 128 coordinate rows x 64 tokens fp16
-constexpr int kPfBufBytes = kPfKBytes + kPfVBytes;    // 33792
-constexpr int kPfStageBytes = 8192;                   // per-wavefront staging area for the rotations
+// Tile geometry for head_dim D (64 or 128).
+template <int D>
+struct PrefillCfg {
+    static constexpr int KSTRIDE = 2 * D + 16;            // bytes per token row of the K tile (D fp16 + pad): 4 banks
+    static constexpr int KBYTES = 64 * KSTRIDE;           // 17408 at D = 128
+    static constexpr int VBYTES = D * 128;                // V^T tile: D coordinate rows x 64 tokens fp16
+    static constexpr int BUF = KBYTES + VBYTES;           // 33792 at D = 128
+    static constexpr int STAGE = 64 * D;                  // per-wavefront staging area for the rotations
+    static constexpr int NKS = D / 16;                    // k-steps of the score product
+    static constexpr int NOB = D / 32;                    // 32-coordinate blocks of the output
+    static constexpr int NJ = D / 32;                     // 32-wide k-steps of the head rotations
+    static constexpr int PB = D / 2;                      // packed bytes per token and head
+};
 
 struct PrefillParams {
     const uint16_t* q;          // (B, H_Q, N_Q, 128)
@@ -82,9 +91,11 @@ __device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
 // n queries and L keys sits at position L - n + j (the new tokens are the last ones), and the
 // attention result is rounded to the query dtype before the rotation back, as the attention
 // library's output is in the path this replaces (src/flashquant/vllm/impl.py:265-336, 470-512).
-template <int DT, bool PAGED>
+template <int D, int DT, bool PAGED>
 __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillParams p) {
-    constexpr int D = 128;
+    using Cfg = PrefillCfg<D>;
+    constexpr int kPfKStride = Cfg::KSTRIDE, kPfKBytes = Cfg::KBYTES, kPfBufBytes = Cfg::BUF, kPfStageBytes = Cfg::STAGE;
+    constexpr int NKS = Cfg::NKS, NOB = Cfg::NOB, NJ = Cfg::NJ, PB = Cfg::PB;
     __shared__ __attribute__((aligned(256))) uint32_t lut[256 * 64];
     extern __shared__ __attribute__((aligned(16))) uint8_t bufs[];   // 2 x (K tile | V^T tile)
     // Rows whose norm times a centroid would not fit fp16 are stored divided by a power of two.
@@ -159,21 +170,38 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     // ---- dequantisation plan ------------------------------------------------------------------
     const int64_t k_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.k_cap;
     const int64_t v_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.v_cap;
-    const uint8_t* kp = p.k_packed + k_row0 * 64;
-    const uint8_t* vp = p.v_packed + v_row0 * 64;
+    const uint8_t* kp = p.k_packed + k_row0 * PB;
+    const uint8_t* vp = p.v_packed + v_row0 * PB;
     const float* knp = p.k_norms + k_row0;
     const float* vnp = p.v_norms + v_row0;
-    // K: token of the tile and 16-coordinate group.  Lane bits (g0 g1 t0 g2 t1 t2): eight consecutive
-    // lanes hold four groups of two consecutive tokens, so the 128 bytes they store with one 16-byte
-    // write each fall into 32 different banks (token rows are 272 bytes apart: 4 banks).
-    const int gqk = (lane & 3) | ((lane >> 1) & 4);
-    const int tk = 8 * w + ((lane >> 2) & 1) + ((lane >> 3) & 6);
-    // V: token pair of the tile and dword of the packed row.  The four pairs of a wavefront are the
-    // ones whose positions share a 16-byte group of the transposed tile (0, 2, 4, 6 within it), so
-    // that a store of half a wavefront covers all 32 banks once.
-    // Lane bits (j0 j1 j2 p0 p1 j3): each half of the wavefront holds all four pairs and eight dwords.
-    const int jv = (lane & 7) | ((lane >> 2) & 8);
-    const int tp = 8 * (w >> 1) + 2 * (w & 1) + ((lane >> 3) & 1) + 4 * ((lane >> 4) & 1);
+    // Work items of the dequantisation.  K: (token of the tile, 16-coordinate group); V: (token pair, dword
+    // of the packed row).  head_dim 128: 512 of each, every thread takes one of both; head_dim 64: 256 of
+    // each, wavefronts 0..3 take the V items and wavefronts 4..7 the K items.
+    constexpr bool kSplitRoles = D == 64;
+    const bool does_k = !kSplitRoles || w >= 4;
+    const bool does_v = !kSplitRoles || w < 4;
+    int gqk, tk, jv, tp;
+    if constexpr (!kSplitRoles) {
+        // K lane bits (g0 g1 t0 g2 t1 t2): eight consecutive lanes hold four groups of two consecutive
+        // tokens, so the 128 bytes they store with one 16-byte write each fall into 32 different banks
+        // (token rows are 272 bytes apart: 4 banks).
+        gqk = (lane & 3) | ((lane >> 1) & 4);
+        tk = 8 * w + ((lane >> 2) & 1) + ((lane >> 3) & 6);
+        // V: the four pairs of a wavefront are the ones whose positions share a 16-byte group of the
+        // transposed tile (0, 2, 4, 6 within it); lane bits (j0 j1 j2 p0 p1 j3): each half of the
+        // wavefront holds all four pairs and eight dwords, so that its store covers all 32 banks once.
+        jv = (lane & 7) | ((lane >> 2) & 8);
+        tp = 8 * (w >> 1) + 2 * (w & 1) + ((lane >> 3) & 1) + 4 * ((lane >> 4) & 1);
+    } else {
+        // K (wavefronts 4..7): lane bits (g0 g1 t0 t1 t2 t3), 16 tokens per wavefront
+        gqk = lane & 3;
+        tk = 16 * (w & 3) + (lane >> 2);
+        // V (wavefronts 0..3): lane bits (j0 j1 j2 p0 p1 p2): eight pairs per wavefront, the four of
+        // each half sharing a 16-byte group of the transposed tile
+        jv = lane & 7;
+        const int i8 = lane >> 3;                       // 0..7
+        tp = 8 * (w & 3) + 2 * (i8 >> 2) + (i8 & 1) + 4 * ((i8 >> 1) & 1);
+    }
     const int k_wr = tk * kPfKStride + gqk * 32;
     int v_wr[8];
     {
@@ -187,9 +215,9 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             v_wr[k] = kPfKBytes + d * 128 + 16 * physg + 2 * within;
         }
     }
-    uint2v kraw;
-    uint32_t vra, vrb;
-    float nk, nv0, nv1;
+    uint2v kraw = {0u, 0u};
+    uint32_t vra = 0u, vrb = 0u;
+    float nk = 0.0f, nv0 = 0.0f, nv1 = 0.0f;
     auto issue_loads = [&](int tile_raw) {
         const int tile = tile_raw < ntiles ? tile_raw : ntiles - 1;   // past the end: the last tile again, never used
         const int t0 = tile > 0 ? tile * 64 : 0;
@@ -201,29 +229,37 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             // token t of the sequence: row t % BS of page block_table[t / BS]; the row holds
             // [K idx H*64 | K norm H*4 | V idx H*64 | V norm H*4]
             const int H = p.H_KV;
-            const int64_t row_bytes = int64_t(H) * 136;
+            const int64_t row_bytes = int64_t(H) * (D + 8);
             const int32_t* bt = p.block_table + int64_t(b) * p.max_blocks;
             auto row_ptr = [&](int t) {
                 int pg = bt[t >> p.bs_log2];
                 pg = pg < 0 ? 0 : (pg >= p.num_blocks ? p.num_blocks - 1 : pg);
                 return p.cache + ((int64_t(pg) << p.bs_log2) + (t & ((1 << p.bs_log2) - 1))) * row_bytes;
             };
-            const uint8_t* rk = row_ptr(tkk);
-            const uint8_t* ra = row_ptr(ta);
-            const uint8_t* rb2 = row_ptr(tb);
-            kraw = *reinterpret_cast<const uint2v*>(rk + hkv * 64 + 8 * gqk);
-            nk = *reinterpret_cast<const float*>(rk + H * 64 + 4 * hkv);
-            vra = *reinterpret_cast<const uint32_t*>(ra + H * 68 + hkv * 64 + 4 * jv);
-            vrb = *reinterpret_cast<const uint32_t*>(rb2 + H * 68 + hkv * 64 + 4 * jv);
-            nv0 = *reinterpret_cast<const float*>(ra + H * 132 + 4 * hkv);
-            nv1 = *reinterpret_cast<const float*>(rb2 + H * 132 + 4 * hkv);
+            if (does_k) {
+                const uint8_t* rk = row_ptr(tkk);
+                kraw = *reinterpret_cast<const uint2v*>(rk + hkv * PB + 8 * gqk);
+                nk = *reinterpret_cast<const float*>(rk + H * PB + 4 * hkv);
+            }
+            if (does_v) {
+                const uint8_t* ra = row_ptr(ta);
+                const uint8_t* rb2 = row_ptr(tb);
+                vra = *reinterpret_cast<const uint32_t*>(ra + H * (PB + 4) + hkv * PB + 4 * jv);
+                vrb = *reinterpret_cast<const uint32_t*>(rb2 + H * (PB + 4) + hkv * PB + 4 * jv);
+                nv0 = *reinterpret_cast<const float*>(ra + H * (D + 4) + 4 * hkv);
+                nv1 = *reinterpret_cast<const float*>(rb2 + H * (D + 4) + 4 * hkv);
+            }
         } else {
-            kraw = *reinterpret_cast<const uint2v*>(kp + int64_t(tkk) * 64 + 8 * gqk);
-            nk = knp[tkk];
-            vra = *reinterpret_cast<const uint32_t*>(vp + int64_t(ta) * 64 + 4 * jv);
-            vrb = *reinterpret_cast<const uint32_t*>(vp + int64_t(tb) * 64 + 4 * jv);
-            nv0 = vnp[ta];
-            nv1 = vnp[tb];
+            if (does_k) {
+                kraw = *reinterpret_cast<const uint2v*>(kp + int64_t(tkk) * PB + 8 * gqk);
+                nk = knp[tkk];
+            }
+            if (does_v) {
+                vra = *reinterpret_cast<const uint32_t*>(vp + int64_t(ta) * PB + 4 * jv);
+                vrb = *reinterpret_cast<const uint32_t*>(vp + int64_t(tb) * PB + 4 * jv);
+                nv0 = vnp[ta];
+                nv1 = vnp[tb];
+            }
         }
     };
     auto dequant = [&](int buf, int tile) {
@@ -234,60 +270,64 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             nv0 = __builtin_ldexpf(nv0, -ev0);
             nv1 = __builtin_ldexpf(nv1, -ev1);
             const int tag = (tile + 1) << 8;
-            if (gqk == 0) scale_exp[buf][tk] = tag | ek;
-            if (jv == 0) {
+            if (does_k && gqk == 0) scale_exp[buf][tk] = tag | ek;
+            if (does_v && jv == 0) {
                 scale_exp[buf][64 + 2 * tp] = tag | ev0;
                 scale_exp[buf][64 + 2 * tp + 1] = tag | ev1;
             }
             if ((ek | ev0 | ev1) != 0) big_tile[buf] = tile + 1;
         }
-        const _Float16 hk = _Float16(nk);
-        const half2v nk2 = {hk, hk};
-        const uint4v a0 = lookup_word(lutb, kraw.x, lk);   // coordinates 0..7 of the group
-        const uint4v a1 = lookup_word(lutb, kraw.y, lk);   // coordinates 8..15
-        // positions 0..7 = coordinates (0..3, 8..11), positions 8..15 = (4..7, 12..15)
-        const uint4v w0 = {scale_pair(a0.x, nk2), scale_pair(a0.y, nk2), scale_pair(a1.x, nk2), scale_pair(a1.y, nk2)};
-        const uint4v w1 = {scale_pair(a0.z, nk2), scale_pair(a0.w, nk2), scale_pair(a1.z, nk2), scale_pair(a1.w, nk2)};
-        *reinterpret_cast<uint4v*>(dst + k_wr) = w0;
-        *reinterpret_cast<uint4v*>(dst + k_wr + 16) = w1;
-        // V: 2x2 nibble transpose, so that a byte holds one coordinate of the two tokens
-        const uint32_t X = (vra & 0xF0F0F0F0u) | ((vrb >> 4) & 0x0F0F0F0Fu);   // even coordinates
-        const uint32_t Y = ((vra << 4) & 0xF0F0F0F0u) | (vrb & 0x0F0F0F0Fu);   // odd coordinates
-        const half2v nv2 = {_Float16(nv0), _Float16(nv1)};
-        const uint4v xe = lookup_word(lutb, X, lv);
-        const uint4v yo = lookup_word(lutb, Y, lv);
-        const uint32_t xs[4] = {xe.x, xe.y, xe.z, xe.w}, ys[4] = {yo.x, yo.y, yo.z, yo.w};
+        if (does_k) {      // uniform over the wavefront
+            const _Float16 hk = _Float16(nk);
+            const half2v nk2 = {hk, hk};
+            const uint4v a0 = lookup_word(lutb, kraw.x, lk);   // coordinates 0..7 of the group
+            const uint4v a1 = lookup_word(lutb, kraw.y, lk);   // coordinates 8..15
+            // positions 0..7 = coordinates (0..3, 8..11), positions 8..15 = (4..7, 12..15)
+            const uint4v w0 = {scale_pair(a0.x, nk2), scale_pair(a0.y, nk2), scale_pair(a1.x, nk2), scale_pair(a1.y, nk2)};
+            const uint4v w1 = {scale_pair(a0.z, nk2), scale_pair(a0.w, nk2), scale_pair(a1.z, nk2), scale_pair(a1.w, nk2)};
+            *reinterpret_cast<uint4v*>(dst + k_wr) = w0;
+            *reinterpret_cast<uint4v*>(dst + k_wr + 16) = w1;
+        }
+        if (does_v) {
+            // V: 2x2 nibble transpose, so that a byte holds one coordinate of the two tokens
+            const uint32_t X = (vra & 0xF0F0F0F0u) | ((vrb >> 4) & 0x0F0F0F0Fu);   // even coordinates
+            const uint32_t Y = ((vra << 4) & 0xF0F0F0F0u) | (vrb & 0x0F0F0F0Fu);   // odd coordinates
+            const half2v nv2 = {_Float16(nv0), _Float16(nv1)};
+            const uint4v xe = lookup_word(lutb, X, lv);
+            const uint4v yo = lookup_word(lutb, Y, lv);
+            const uint32_t xs[4] = {xe.x, xe.y, xe.z, xe.w}, ys[4] = {yo.x, yo.y, yo.z, yo.w};
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            *reinterpret_cast<uint32_t*>(dst + v_wr[2 * c]) = scale_pair(xs[c], nv2);
-            *reinterpret_cast<uint32_t*>(dst + v_wr[2 * c + 1]) = scale_pair(ys[c], nv2);
+            for (int c = 0; c < 4; ++c) {
+                *reinterpret_cast<uint32_t*>(dst + v_wr[2 * c]) = scale_pair(xs[c], nv2);
+                *reinterpret_cast<uint32_t*>(dst + v_wr[2 * c + 1]) = scale_pair(ys[c], nv2);
+            }
         }
     };
 
     issue_loads(0);
 
     // ---- query: rotate this wavefront's 32 rows, round to the query dtype, scale to fp16 ----------
-    half8 qb[8];
+    half8 qb[NKS];
     float krow;
     {
         const uint16_t* qbase = PAGED ? p.q + (q_row0 + hq) * D : p.q + (q_row0 + int64_t(hq) * NQ) * D;
-        uint16_t* st = reinterpret_cast<uint16_t*>(bufs + w * kPfStageBytes);   // (32 rows, 128) raw 16-bit
+        uint16_t* st = reinterpret_cast<uint16_t*>(bufs + w * kPfStageBytes);   // (32 rows, D) raw 16-bit
         // the rows are exact in fp16 up to a power of two: fp16-split MFMA, two terms
-        half8 a[2][4];
+        half8 a[2][NJ];
         float up[2];
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             int pos = pos0 + 16 * rb + n16;
             pos = pos < NQ ? pos : NQ - 1;
-            uint4v raw[4];
+            uint4v raw[NJ];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) raw[j] = *reinterpret_cast<const uint4v*>(qbase + int64_t(pos) * q_stride + 32 * j + 8 * g4);
+            for (int j = 0; j < NJ; ++j) raw[j] = *reinterpret_cast<const uint4v*>(qbase + int64_t(pos) * q_stride + 32 * j + 8 * g4);
             rows_as_f16<D, DT>(raw, a[rb], up[rb]);
         }
-        for (int cb = 0; cb < 8; ++cb) {
-            float rbv[4][8];
+        for (int cb = 0; cb < NKS; ++cb) {
+            float rbv[NJ][8];
             load_rotation_any<D>(p.rotation, p.rot_col_major != 0, true, 16 * cb, n16, g4, rbv);
-            half8 rhi[4], rlo[4];
+            half8 rhi[NJ], rlo[NJ];
             split_rotation_block<D>(rbv, rhi, rlo);
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb) {
@@ -297,10 +337,10 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             }
         }
         __syncthreads();
-        float qf[8][8];
+        float qf[NKS][8];
         float mx = 0.0f;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
+        for (int ks = 0; ks < NKS; ++ks) {
             const uint2v lo = *reinterpret_cast<const uint2v*>(st + m32 * D + 16 * ks + 4 * hf);
             const uint2v hi = *reinterpret_cast<const uint2v*>(st + m32 * D + 16 * ks + 8 + 4 * hf);
             const uint32_t wds[4] = {lo.x, lo.y, hi.x, hi.y};
@@ -317,7 +357,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
         const float down = bits_to_float(uint32_t(127 - ex) << 23);
         krow = p.scale_log2e * bits_to_float(uint32_t(127 + ex) << 23);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks)
+        for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
             for (int e = 0; e < 8; ++e) qb[ks][e] = _Float16(qf[ks][e] * down);
         __syncthreads();   // the staging area becomes tile buffers
@@ -333,9 +373,9 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     }
 
     // ---- running state -----------------------------------------------------------------------------
-    float16v O[4];
+    float16v O[NOB];
 #pragma unroll
-    for (int ob = 0; ob < 4; ++ob)
+    for (int ob = 0; ob < NOB; ++ob)
 #pragma unroll
         for (int r = 0; r < 16; ++r) O[ob][r] = 0.0f;
     float m_run = -__builtin_inff();
@@ -350,7 +390,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
 #pragma unroll
             for (int r = 0; r < 16; ++r) S[tb][r] = 0.0f;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
+            for (int ks = 0; ks < NKS; ++ks) {
                 const half8 a = *reinterpret_cast<const half8*>(kt + k_rd + 32 * tb * kPfKStride + 32 * ks);
                 S[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qb[ks], S[tb], 0, 0, 0);
             }
@@ -412,7 +452,7 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
         }
         cand = max_xor32(cand);
         // the running maximum moves only when it would grow by more than 2^4: the weights stay
-        // below 16 and the rescale of the 64 accumulator registers becomes rare
+        // below 16 and the rescale of the accumulator registers becomes rare
         const float mnew = cand > m_run + 4.0f ? cand : m_run;
         const float ms = mnew == -__builtin_inff() ? 0.0f : mnew;
         const float alpha = __builtin_amdgcn_exp2f(m_run - ms);
@@ -440,12 +480,12 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
         l_run = __builtin_fmaf(l_run, alpha, ps);
         if (__any(alpha != 1.0f)) {
 #pragma unroll
-            for (int ob = 0; ob < 4; ++ob)
+            for (int ob = 0; ob < NOB; ++ob)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) O[ob][r] *= alpha;
         }
 #pragma unroll
-        for (int ob = 0; ob < 4; ++ob)
+        for (int ob = 0; ob < NOB; ++ob)
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 const int c = (2 * s) ^ (4 * (ob & 1));
@@ -476,13 +516,13 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     // ---- normalise, rotate back, store -------------------------------------------------------------------
     const float l_tot = l_run + xor_shuffle(l_run, 32);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    float* stf = reinterpret_cast<float*>(bufs + w * kPfStageBytes);   // (16 rows, 128) float32
+    float* stf = reinterpret_cast<float*>(bufs + w * kPfStageBytes);   // (16 rows, D) float32
     uint16_t* obase = PAGED ? p.out + (q_row0 + hq) * D : p.out + (q_row0 + int64_t(hq) * NQ) * D;
     for (int half_rows = 0; half_rows < 2; ++half_rows) {
         __syncthreads();
         if ((m32 >> 4) == half_rows) {
 #pragma unroll
-            for (int ob = 0; ob < 4; ++ob)
+            for (int ob = 0; ob < NOB; ++ob)
 #pragma unroll
                 for (int rq = 0; rq < 4; ++rq) {
                     float4v v = {O[ob][4 * rq] * inv, O[ob][4 * rq + 1] * inv, O[ob][4 * rq + 2] * inv, O[ob][4 * rq + 3] * inv};
@@ -494,22 +534,22 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
                 }
         }
         __syncthreads();
-        float a[4][8];
+        float a[NJ][8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NJ; ++j) {
             const float4v lo = *reinterpret_cast<const float4v*>(stf + n16 * D + 32 * j + 8 * g4);
             const float4v hi = *reinterpret_cast<const float4v*>(stf + n16 * D + 32 * j + 8 * g4 + 4);
             a[j][0] = lo.x; a[j][1] = lo.y; a[j][2] = lo.z; a[j][3] = lo.w;
             a[j][4] = hi.x; a[j][5] = hi.y; a[j][6] = hi.z; a[j][7] = hi.w;
         }
         // float32 rows: both operands as two fp16 terms, three MFMA terms
-        half8 ahi[4], alo[4];
+        half8 ahi[NJ], alo[NJ];
         float up;
         rows_split_f16<D>(a, ahi, alo, up);
-        for (int cb = 0; cb < 8; ++cb) {
-            float rbv[4][8];
+        for (int cb = 0; cb < NKS; ++cb) {
+            float rbv[NJ][8];
             load_rotation_any<D>(p.rotation, p.rot_col_major != 0, false, 16 * cb, n16, g4, rbv);
-            half8 rhi[4], rlo[4];
+            half8 rhi[NJ], rlo[NJ];
             split_rotation_block<D>(rbv, rhi, rlo);
             const float4v acc = rotate_block_f16x3<D>(ahi, alo, rhi, rlo);
 #pragma unroll
@@ -519,6 +559,22 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             }
         }
     }
+}
+
+template <int D, bool PAGED>
+int launch_prefill(const PrefillParams& p, dim3 grid, int dtype, hipStream_t s) {
+    const size_t lds = 2 * size_t(PrefillCfg<D>::BUF);
+    const dim3 block(512);
+    if (dtype == FQ_F16) {
+        auto kern = fused_tq_attention_kernel<D, FQ_F16, PAGED>;
+        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
+    } else {
+        auto kern = fused_tq_attention_kernel<D, FQ_BF16, PAGED>;
+        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
+    }
+    return fq_host::check_launch();
 }
 
 }  // namespace fq
@@ -555,7 +611,7 @@ extern "C" int fq_fused_tq_attention_strided(const void* q, const uint8_t* k_pac
         return FQ_ERR_MISALIGNED;
     if (B > 65535 || H_KV > 65535) return FQ_ERR_BAD_SHAPE;
 
-    if (D != 128 || fq_host::force_any_dim_attention()) {   // the tuned tile layout is written for 128 coordinates
+    if (D == 256 || fq_host::force_any_dim_attention()) {   // the tuned tile layout serves 64 and 128 coordinates
         AnyDimParams a{};
         a.q = static_cast<const uint16_t*>(q);
         a.k_packed = k_packed; a.k_norms = k_norms; a.v_packed = v_packed; a.v_norms = v_norms;
@@ -583,22 +639,12 @@ extern "C" int fq_fused_tq_attention_strided(const void* q, const uint8_t* k_pac
     const int64_t units = int64_t((N_Q + 31) / 32) * p.G;
     const int64_t wgs = (units + 7) / 8;
     if (wgs > 0x7fffffffLL) return FQ_ERR_BAD_SHAPE;
-    const dim3 grid(static_cast<unsigned>(wgs), H_KV, B), block(512);
-    const size_t lds = 2 * size_t(kPfBufBytes);
+    const dim3 grid(static_cast<unsigned>(wgs), H_KV, B);
     hipStream_t s = static_cast<hipStream_t>(stream);
     p.cu_seqlens_q = nullptr; p.seq_lens = nullptr; p.block_table = nullptr; p.cache = nullptr;
     p.max_blocks = 0; p.num_blocks = 0; p.bs_log2 = 0;
     p.round_slots = fq_host::device_cu_count();
-    if (dtype == FQ_F16) {
-        auto kern = fused_tq_attention_kernel<FQ_F16, false>;
-        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
-        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
-    } else {
-        auto kern = fused_tq_attention_kernel<FQ_BF16, false>;
-        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
-        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
-    }
-    return fq_host::check_launch();
+    return D == 64 ? launch_prefill<64, false>(p, grid, dtype, s) : launch_prefill<128, false>(p, grid, dtype, s);
 }
 
 extern "C" int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, const uint8_t* kv_cache,
@@ -623,7 +669,7 @@ extern "C" int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, 
         return FQ_ERR_MISALIGNED;
     if (num_seqs > 65535 || H_KV > 65535) return FQ_ERR_BAD_SHAPE;
 
-    if (D != 128 || fq_host::force_any_dim_attention()) {
+    if (D == 256 || fq_host::force_any_dim_attention()) {
         AnyDimParams a{};
         a.q = static_cast<const uint16_t*>(q);
         a.centroids_k = centroids_k; a.centroids_v = centroids_v;
@@ -656,17 +702,7 @@ extern "C" int fq_paged_tq4_prefill(const void* q, const int32_t* cu_seqlens_q, 
     const int64_t units = int64_t((max_q_len + 31) / 32) * p.G;
     const int64_t wgs = (units + 7) / 8;
     if (wgs > 0x7fffffffLL) return FQ_ERR_BAD_SHAPE;
-    const dim3 grid(static_cast<unsigned>(wgs), H_KV, num_seqs), block(512);
-    const size_t lds = 2 * size_t(kPfBufBytes);
+    const dim3 grid(static_cast<unsigned>(wgs), H_KV, num_seqs);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == FQ_F16) {
-        auto kern = fused_tq_attention_kernel<FQ_F16, true>;
-        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
-        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
-    } else {
-        auto kern = fused_tq_attention_kernel<FQ_BF16, true>;
-        if (!fq_host::lds_limit_raised(reinterpret_cast<const void*>(kern), lds)) return FQ_ERR_LAUNCH;
-        hipLaunchKernelGGL(kern, grid, block, lds, s, p);
-    }
-    return fq_host::check_launch();
+    return D == 64 ? launch_prefill<64, true>(p, grid, dtype, s) : launch_prefill<128, true>(p, grid, dtype, s);
 }

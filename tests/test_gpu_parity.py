@@ -433,6 +433,32 @@ def test_fused_attention_other_head_dims(d, dtype, causal):
     _check_prefill(1, 4, 4, 37, 99, dtype, False, d=d, seed=82, cv=(book(d)[0] * 1.25).contiguous())
 
 
+@pytest.mark.parametrize("b,hq,hkv,nq,nkv,causal,dtype", [
+    (2, 32, 8, 300, 300, True, torch.bfloat16),     # 4 query heads per KV head, ragged last tile
+    (1, 8, 8, 129, 700, False, torch.float16),      # one head per KV head, N_Q != N_KV
+    (3, 16, 2, 1100, 1100, True, torch.bfloat16),   # 8 heads per KV head, more workgroups than fit one round
+    (1, 12, 4, 64, 64, True, torch.float16),        # 3 heads per KV head
+])
+def test_fused_attention_head_dim_64_on_the_tuned_kernel(b, hq, hkv, nq, nkv, causal, dtype):
+    """head_dim 64 runs the same tile layout as 128 (half the dequantisation items: the wavefronts
+    split into a K group and a V group): every row against the oracle."""
+    _check_prefill(b, hq, hkv, nq, nkv, dtype, causal, d=64, seed=91)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_fused_attention_head_dim_64_kernels_agree(causal, kernel_option):
+    q, kp, kn, vp, vn, c, r = _prefill_case(2, 8, 2, 200, 200, torch.bfloat16, 93, d=64)
+    dev = [t.to(DEV) for t in (q, kp, kn, vp, vn, c, r)]
+    tuned = K.fused_tq_attention(*dev[:5], dev[5], dev[5], dev[6], is_causal=causal)
+    kernel_option("attention_any_dim", True)
+    general = K.fused_tq_attention(*dev[:5], dev[5], dev[5], dev[6], is_causal=causal)
+    torch.cuda.synchronize()
+    want = O.fused_tq_attention(q, kp, kn, vp, vn, c, c, r, is_causal=causal)
+    tol = 2e-2 * max(1.0, want.float().abs().max().item())
+    assert (tuned.cpu().float() - want.float()).abs().max().item() <= tol
+    assert (general.float() - tuned.float()).abs().max().item() <= tol
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_fused_attention_general_kernel_agrees_at_head_dim_128(causal, kernel_option):
     """The kernel that serves head_dim 64 and 256 also takes 128: against the oracle and against the
