@@ -108,6 +108,10 @@ def test_split_count_rules(lib):
     auto = lib.fq_paged_decode_auto_splits(8, 8, 16, 8192)
     assert auto >= 32
     assert lib.fq_paged_decode_auto_splits(1, 1, 16, 1) == 1
+    # fewer than 8 KV heads (the direct kernel): chunks of at least 256 tokens
+    assert lib.fq_paged_decode_auto_splits(32, 1, 16, 256) <= 16
+    assert lib.fq_paged_decode_auto_splits(32, 2, 16, 256) <= 16
+    assert lib.fq_paged_decode_auto_splits(4, 4, 16, 2048) >= 32      # long contexts still fill the chip
     f = lib.fq_paged_tq4_decode
     f.argtypes = ([ctypes.c_void_p] * 2 + [ctypes.c_int] + [ctypes.c_void_p] * 8 + [ctypes.c_int] * 6 +
                   [ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
