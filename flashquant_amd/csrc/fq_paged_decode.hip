@@ -89,8 +89,10 @@ struct DecodeParams {
 };
 
 
+// head_dim 256 keeps 64 accumulator registers per lane and runs with at most four wavefronts per workgroup,
+// so that a wavefront may use up to 512 registers (with eight it spilled 150-220 of them).
 template <int D, int BSL, int GP, int DT, int PVR>
-__global__ __launch_bounds__(512) void paged_decode_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(D == 256 ? 256 : 512) void paged_decode_kernel(const DecodeParams p) {
     constexpr int BS = 1 << BSL;
     constexpr int KS = D / 32;            // k-steps of the score product
     constexpr int KW = D / 32;            // K dwords per lane per block
@@ -1702,7 +1704,8 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
                                             stream);
     }
 
-    const int waves = p.H_KV < 8 ? p.H_KV : 8;
+    const int max_waves = D == 256 ? 4 : 8;
+    const int waves = p.H_KV < max_waves ? p.H_KV : max_waves;
     const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
     const size_t lds = p.two_tables ? size_t(kLutWords) * sizeof(uint32_t) : 0;   // the K table is static
 #define FQ_DECODE_GP(BSL, GPV)                                                                  \
