@@ -57,9 +57,11 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
     using C = AnyDimCfg<D>;
     constexpr int NJ = D / 32;          // k-steps of the score product
     constexpr int NCB = D / 16;         // 16-coordinate output blocks
-    constexpr int CPT = D / 8;          // coordinates per thread in the dequantisation (8 threads per token)
+    constexpr int BPT = D / 32;         // packed bytes per thread and token in the dequantisation (16 threads per token pair)
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ _Float16 cent_k[16], cent_v[16];
+    // byte -> (fp16 centroid[high nibble], fp16 centroid[low nibble]); for V the two nibbles of the byte
+    // come from two consecutive tokens (see the dequantisation)
+    __shared__ uint32_t pair_k[256], pair_v[256];
     // A row whose norm lies above 2^15 is stored divided by 2^excess (its products with a centroid
     // then fit fp16); the power of two goes back in on the float32 score (K) or weight (V).
     __shared__ int k_exc[32], v_exc[32];
@@ -91,8 +93,12 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
     if (pos_wg >= NQ) return;                         // uniform: the grid is sized for the longest sequence
     const int pos0 = pos_wg + 16 * w;                 // first row of this wavefront
 
-    if (tid < 16) cent_k[tid] = _Float16(p.centroids_k[tid]);
-    else if (tid < 32) cent_v[tid - 16] = _Float16(p.centroids_v[tid - 16]);
+    {
+        const half2v ck = {_Float16(p.centroids_k[tid >> 4]), _Float16(p.centroids_k[tid & 15])};
+        const half2v cv = {_Float16(p.centroids_v[tid >> 4]), _Float16(p.centroids_v[tid & 15])};
+        pair_k[tid] = __builtin_bit_cast(uint32_t, ck);
+        pair_v[tid] = __builtin_bit_cast(uint32_t, cv);
+    }
 
     // ---- rotate the 16 query rows of this wavefront, round to the query dtype, stage as fp16 ------
     float up = 1.0f;
@@ -152,58 +158,100 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
 #pragma unroll
     for (int i = 0; i < 4; ++i) { m_run[i] = -__builtin_inff(); l_run[i] = 0.0f; }
 
-    const int tok_d = tid >> 3, part = tid & 7;       // dequantisation: token of the tile, eighth of its row
+    const int tp = tid >> 4, part = tid & 15;         // dequantisation: token pair of the tile, sixteenth of its rows
     const int64_t k_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.k_cap;
     const int64_t v_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.v_cap;
     _Float16* pw = ps + w * 16 * C::VSTRIDE;
 
-    for (int tile = 0; tile < ntiles; ++tile) {
+    // The packed bytes and norms of a tile are asked for one tile ahead (into registers), so that the
+    // memory latency runs under the products of the tile before.
+    uint32_t kw[2][2] = {{0u, 0u}, {0u, 0u}}, vw[2][2] = {{0u, 0u}, {0u, 0u}};
+    float nk[2] = {0.0f, 0.0f}, nv[2] = {0.0f, 0.0f};
+    auto load_tile = [&](int tile) {
         const int t0 = tile * 32;
-        // ---- dequantise: thread = (token, D/8 coordinates) -----------------------------------------
-        {
-            int tok = t0 + tok_d;
+        const uint8_t *kp[2], *vp[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            int tok = t0 + 2 * tp + u;
             const bool live = tok < NKV;
             tok = live ? tok : (NKV > 0 ? NKV - 1 : 0);
-            const uint8_t *kp, *vp;
-            float nk, nv;
             if (PAGED) {
                 const int H = p.H_KV;
                 int pg = p.block_table[int64_t(b) * p.max_blocks + (tok >> p.bs_log2)];
                 pg = pg < 0 ? 0 : (pg >= p.num_blocks ? p.num_blocks - 1 : pg);
                 const uint8_t* row = p.cache + ((int64_t(pg) << p.bs_log2) + (tok & ((1 << p.bs_log2) - 1))) * (int64_t(H) * (D + 8));
-                kp = row + hkv * (D / 2);
-                nk = *reinterpret_cast<const float*>(row + H * (D / 2) + 4 * hkv);
-                vp = row + H * (D / 2 + 4) + hkv * (D / 2);
-                nv = *reinterpret_cast<const float*>(row + H * (D + 4) + 4 * hkv);
+                kp[u] = row + hkv * (D / 2);
+                nk[u] = *reinterpret_cast<const float*>(row + H * (D / 2) + 4 * hkv);
+                vp[u] = row + H * (D / 2 + 4) + hkv * (D / 2);
+                nv[u] = *reinterpret_cast<const float*>(row + H * (D + 4) + 4 * hkv);
             } else {
-                kp = p.k_packed + (k_row0 + tok) * (D / 2);
-                vp = p.v_packed + (v_row0 + tok) * (D / 2);
-                nk = p.k_norms[k_row0 + tok];
-                nv = p.v_norms[v_row0 + tok];
+                kp[u] = p.k_packed + (k_row0 + tok) * (D / 2);
+                vp[u] = p.v_packed + (v_row0 + tok) * (D / 2);
+                nk[u] = p.k_norms[k_row0 + tok];
+                nv[u] = p.v_norms[v_row0 + tok];
             }
-            if (!live) { nk = 0.0f; nv = 0.0f; }
-            const int ek = norm_excess(nk), ev = norm_excess(nv);
-            nk = __builtin_ldexpf(nk, -ek);
-            nv = __builtin_ldexpf(nv, -ev);
-            if (part == 0) { k_exc[tok_d] = ek; v_exc[tok_d] = ev; }
+            if (!live) { nk[u] = 0.0f; nv[u] = 0.0f; }
+            // packed bytes part * BPT .. of the token (BPT = 2, 4 or 8)
+            if (BPT == 2) {
+                kw[u][0] = *reinterpret_cast<const uint16_t*>(kp[u] + 2 * part);
+                vw[u][0] = *reinterpret_cast<const uint16_t*>(vp[u] + 2 * part);
+            } else {
 #pragma unroll
-            for (int c = 0; c < CPT / 8; ++c) {       // 4 bytes = 8 coordinates at a time
-                const int byte0 = part * (CPT / 2) + 4 * c;
-                const uint32_t kw = *reinterpret_cast<const uint32_t*>(kp + byte0);
-                const uint32_t vw = *reinterpret_cast<const uint32_t*>(vp + byte0);
+                for (int c = 0; c < BPT / 4; ++c) {
+                    kw[u][c] = *reinterpret_cast<const uint32_t*>(kp[u] + BPT * part + 4 * c);
+                    vw[u][c] = *reinterpret_cast<const uint32_t*>(vp[u] + BPT * part + 4 * c);
+                }
+            }
+        }
+    };
+    if (ntiles > 0) load_tile(0);
+
+    for (int tile = 0; tile < ntiles; ++tile) {
+        const int t0 = tile * 32;
+        // ---- dequantise: thread = (two consecutive tokens, D/16 coordinates of each) ---------------------
+        {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const uint32_t kb = (kw >> (8 * e)) & 0xffu, vb = (vw >> (8 * e)) & 0xffu;
-                    const int d = 2 * (byte0 + e);
-                    // fp16(centroid) * norm, rounded to fp16: the same values as the tuned kernel's tiles
-                    ks[tok_d * C::KSTRIDE + d] = _Float16(float(cent_k[kb >> 4]) * nk);
-                    ks[tok_d * C::KSTRIDE + d + 1] = _Float16(float(cent_k[kb & 15]) * nk);
-                    vt[d * C::VSTRIDE + tok_d] = _Float16(float(cent_v[vb >> 4]) * nv);
-                    vt[(d + 1) * C::VSTRIDE + tok_d] = _Float16(float(cent_v[vb & 15]) * nv);
+            for (int u = 0; u < 2; ++u) {
+                const int ek = norm_excess(nk[u]), ev = norm_excess(nv[u]);
+                nk[u] = __builtin_ldexpf(nk[u], -ek);
+                nv[u] = __builtin_ldexpf(nv[u], -ev);
+                if (part == 0) { k_exc[2 * tp + u] = ek; v_exc[2 * tp + u] = ev; }
+            }
+            // K, row-major: byte j of the thread's run -> coordinates 2 (part BPT + j), + 1 of its token:
+            // fp16(centroid) * norm, rounded to fp16 (the same values as the tuned kernel's tiles)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const _Float16 hn = _Float16(nk[u]);
+                const half2v n2 = {hn, hn};
+                uint32_t* dst = reinterpret_cast<uint32_t*>(ks + (2 * tp + u) * C::KSTRIDE + 2 * BPT * part);
+#pragma unroll
+                for (int j = 0; j < BPT; ++j) {
+                    const uint32_t byte = (kw[u][j >> 2] >> (8 * (j & 3))) & 0xffu;
+                    const half2v c2 = __builtin_bit_cast(half2v, pair_k[byte]) * n2;
+                    dst[j] = __builtin_bit_cast(uint32_t, c2);
+                }
+            }
+            // V, transposed: a 2 x 2 nibble transpose makes a byte hold one coordinate of the two tokens,
+            // so one lookup yields the dword (token 2 tp, token 2 tp + 1) of a coordinate row
+            {
+                const half2v n2 = {_Float16(nv[0]), _Float16(nv[1])};
+#pragma unroll
+                for (int c = 0; c < (BPT + 3) / 4; ++c) {
+                    const uint32_t X = (vw[0][c] & 0xF0F0F0F0u) | ((vw[1][c] >> 4) & 0x0F0F0F0Fu);   // even coordinates
+                    const uint32_t Y = ((vw[0][c] << 4) & 0xF0F0F0F0u) | (vw[1][c] & 0x0F0F0F0Fu);   // odd coordinates
+#pragma unroll
+                    for (int j = 0; j < (BPT < 4 ? BPT : 4); ++j) {
+                        const int d = 2 * (BPT * part + 4 * c + j);
+                        const half2v xe = __builtin_bit_cast(half2v, pair_v[(X >> (8 * j)) & 0xffu]) * n2;
+                        const half2v yo = __builtin_bit_cast(half2v, pair_v[(Y >> (8 * j)) & 0xffu]) * n2;
+                        *reinterpret_cast<uint32_t*>(vt + d * C::VSTRIDE + 2 * tp) = __builtin_bit_cast(uint32_t, xe);
+                        *reinterpret_cast<uint32_t*>(vt + (d + 1) * C::VSTRIDE + 2 * tp) = __builtin_bit_cast(uint32_t, yo);
+                    }
                 }
             }
         }
         __syncthreads();
+        if (tile + 1 < ntiles) load_tile(tile + 1);
 
         // ---- scores: two blocks of 16 tokens ----------------------------------------------------------
         float4v s[2];
