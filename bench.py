@@ -432,7 +432,85 @@ def main():
             "prod_bytes_per_token_per_kv_head": row4 // H_KV,
             "prod_cache_bytes": prod_bytes,
         })
-        del cache4
+        del cache4, q4, out4, table4
+        torch.cuda.empty_cache()
+
+        # ---- the same operators on other shapes (not BASELINE configs; shapes the reference's launchers
+        # also take: csrc/cuda/paged_decode.cu:401-415, fused_tq_attention.cu:497-506) -----------------
+        def decode_shape(n_seq, ctx, hq, hkv, d, n_caches=2):
+            cent_s, bnd_s = C.codebook.solve_lloyd_max(d, 4)
+            rot_s = C.haar_orthogonal(d, 42).to(dev)
+            cent_s, bnd_s = cent_s.to(dev), bnd_s.to(dev)
+            row = hkv * (d + 8)
+            pages = n_seq * ctx // BS
+            made = []
+            for i in range(n_caches):
+                kx = torch.randn(n_seq * ctx, hkv, d, device=dev).to(torch.bfloat16)
+                vx = torch.randn(n_seq * ctx, hkv, d, device=dev).to(torch.bfloat16)
+                cache_s = torch.zeros(pages, BS, row, dtype=torch.uint8, device=dev)
+                tab = torch.randperm(pages, generator=torch.Generator().manual_seed(70 + i)).reshape(n_seq, ctx // BS)
+                tab = tab.to(torch.int32).to(dev)
+                t = torch.arange(ctx, device=dev)
+                slots = (tab.long()[:, t // BS] * BS + (t % BS)).reshape(-1)
+                K.tq4_compress_and_store(kx, vx, rot_s, bnd_s, cache_s, slots)
+                made.append((cache_s, tab))
+                del kx, vx
+            qs = torch.randn(n_seq, hq, d, device=dev).to(torch.bfloat16)
+            ls = torch.full((n_seq,), ctx, dtype=torch.int32, device=dev)
+            os_ = torch.empty_like(qs)
+
+            def f(i):
+                c_, t_ = made[i % n_caches]
+                K.split_k_paged_decode(qs, c_, t_, ls, cent_s, cent_s, rot_s, hkv, d, BS, sm_scale=1.0 / math.sqrt(d), out=os_)
+
+            for i in range(30):
+                f(i)
+            ms, _ = time_events(f, 40)
+            return ms, n_seq * ctx * row
+
+        def prefill_shape(b, n, hq, hkv, d):
+            cent_s, bnd_s = C.codebook.solve_lloyd_max(d, 4)
+            rot_s = C.haar_orthogonal(d, 42).to(dev)
+            cent_s, bnd_s = cent_s.to(dev), bnd_s.to(dev)
+            qx = torch.randn(b, hq, n, d, device=dev).to(torch.bfloat16)
+            kx = torch.randn(b * n, hkv, d, device=dev).to(torch.bfloat16)
+            vx = torch.randn(b * n, hkv, d, device=dev).to(torch.bfloat16)
+            kp_, kn_ = K.tq4_compress(kx, rot_s, bnd_s)
+            vp_, vn_ = K.tq4_compress(vx, rot_s, bnd_s)
+
+            def bhnd(t_):
+                return t_.reshape(b, n, hkv, -1).permute(0, 2, 1, 3).contiguous()
+
+            kp_, kn_, vp_, vn_ = (bhnd(t_) for t_ in (kp_, kn_, vp_, vn_))
+
+            def f(i):
+                K.fused_tq_attention(qx, kp_, kn_, vp_, vn_, cent_s, cent_s, rot_s, sm_scale=1.0 / math.sqrt(d), is_causal=True)
+
+            for i in range(2):
+                f(i)
+            ms, _ = time_events(f, 5)
+            return ms, 4.0 * n * n * d * b * hq / 2
+
+        shapes = {}
+        for name, (n_seq, ctx, hq, hkv, d) in {
+            "decode_32x16384_32q_8kv_d128": (32, 16384, 32, 8, 128),
+            "decode_32x4096_32q_4kv_d128": (32, 4096, 32, 4, 128),
+            "decode_32x4096_32q_8kv_d64": (32, 4096, 32, 8, 64),
+            "decode_32x4096_32q_8kv_d256": (32, 4096, 32, 8, 256),
+        }.items():
+            ms, nbytes = decode_shape(n_seq, ctx, hq, hkv, d)
+            shapes[name] = {"step_us": ms * 1e3, "gbps": nbytes / (ms * 1e-3) / 1e9,
+                            "pct_hbm_peak": 100.0 * nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+            torch.cuda.empty_cache()
+        for name, (b, n, hq, hkv, d) in {
+            "prefill_2x8192_32q_8kv_d64": (2, 8192, 32, 8, 64),
+            "prefill_2x8192_16q_4kv_d256": (2, 8192, 16, 4, 256),
+        }.items():
+            ms, flops = prefill_shape(b, n, hq, hkv, d)
+            shapes[name] = {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12,
+                            "pct_fp16_mfma_peak": 100.0 * flops / (ms * 1e-3) / 2.5e15}
+            torch.cuda.empty_cache()
+        extra["other_shapes"] = shapes
 
     value = kv_bytes / (step_ms * 1e-3) / 1e9
     line = {
