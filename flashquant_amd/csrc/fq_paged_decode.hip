@@ -33,9 +33,12 @@
 //            A lane's K operand is the 16 bytes it loaded (token n, quarter g of
 //            the row): the contraction index is permuted (k-step ks, group g,
 //            element e) <-> d = g*D/4 + 8*ks + e, and Q is loaded the same way.
-//   softmax  base 2, float32; the weight handed to the second product is
-//            min(w * |v|, 65504) in fp16 (the V norm rides on the weight), the
-//            denominator accumulates w.
+//   softmax  base 2, float32; the weight handed to the second product is w * |v| in
+//            fp16 (the V norm rides on the weight), the denominator accumulates w.  The
+//            running reference moves only when a score leads it by more than 2^16 or a
+//            product w * |v| would pass 60000; it then becomes the maximum over the tile
+//            of score + (binary orders of |v| above 2^10), so the product stays below
+//            2^11 whatever the norms are and accumulator rescales are rare.
 //   output   O (16 rows x D) += P (16 x tokens) . V (tokens x D), where row n of P
 //            holds the weights of head n % GP for the tokens of block class n / GP
 //            only (zero elsewhere), so the lane that computed a weight is the lane
