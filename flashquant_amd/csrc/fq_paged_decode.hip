@@ -630,6 +630,22 @@ __device__ __forceinline__ bool lds_flag_wait(uint32_t* flag, uint32_t count, in
 // (read with fq_paged_decode_fault_count).
 __device__ unsigned int g_decode_faults = 0u;
 
+// Byte offset, inside a page of `H` KV heads, of chunk `cc` of the 8-head rows that head group `hgrp`
+// (heads 8 hgrp .. 8 hgrp + 7) sees: the group's slices of the four sections of a token row laid end
+// to end, kChunksPerRow chunks per token.  With 8 heads the slices are the row itself (16 cc).
+template <bool PROD>
+__device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
+    constexpr int CPR = StagedCfg<PROD>::CHUNKS_PER_ROW;
+    if constexpr (PROD) return uint32_t(16 * cc);          // TurboQuantProd pages come with 8 KV heads
+    const int r = cc / CPR, ci = cc - r * CPR;
+    int off;
+    if (ci < 32) off = 512 * hgrp + 16 * ci;                               // K indices
+    else if (ci < 34) off = H * 64 + 32 * hgrp + 16 * (ci - 32);           // K norms
+    else if (ci < 66) off = H * 68 + 512 * hgrp + 16 * (ci - 34);          // V indices
+    else off = H * 132 + 32 * hgrp + 16 * (ci - 66);                       // V norms
+    return uint32_t(r * (H * 136) + off);
+}
+
 template <int BSL, int GP, int DT, int PVR, bool PROD, int CW>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     using Cfg = StagedCfg<PROD>;
@@ -671,6 +687,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // come last instead of alternating with the live ones.
     int seq = blockIdx.x;
     int split = blockIdx.y;
+    // More than 8 KV heads: a workgroup serves the group of 8 heads blockIdx.z, i.e. the query heads
+    // hq0 .. hq0 + 8 G - 1, and copies that group's slices of the token rows.
+    const int hgrp = blockIdx.z;
+    const int HQG = 8 * p.G;                   // query heads of a group
+    const int hq0 = hgrp * HQG;
+    const int row_bytes = p.H_KV * (PROD ? 140 : 136);   // a token row of the cache (ROWB with 8 heads)
 
     // Every load that depends on nothing is asked for first, so that the memory
     // latencies of the prologue overlap instead of adding up: the centroids, the
@@ -723,7 +745,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
         src_page[k] = pg;
         const int sub = (kSpreadTail && k == 4) ? 4 * (tid & 3) : 0;
-        src_off[k] = uint32_t(16 * (c - pg * PC) + sub);
+        src_off[k] = staged_src_offset<PROD>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
         dst_off[k] = kChunkDst<PROD>.off[c] + sub;
     }
     const bool has_round4 = kSpreadTail || tid < kChunksPerTile - 4 * 512;   // else whole wavefronts
@@ -833,13 +855,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         L_known = __builtin_amdgcn_readlane(l_mine, seq);
     }
 
-    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + int64_t(seq) * p.H_Q * 128;
+    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + (int64_t(seq) * p.H_Q + hq0) * 128;
     uint4v q_pre[2][4];
     auto load_first_heads = [&]() {
         if (p.rotation != nullptr && !copier) {
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb) {
-                const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
+                const int row = 16 * rb + n < HQG ? 16 * rb + n : HQG - 1;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) q_pre[rb][j] = *reinterpret_cast<const uint4v*>(qseq + row * 128 + 32 * j + 8 * g);
             }
@@ -880,7 +902,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     const int hq_lane = h * p.G + n;
     if (begin >= end) {   // uniform over the workgroup
         if (g == 0 && n < p.G && !copier) {
-            const int64_t o = (int64_t(seq) * p.H_Q + hq_lane) * NS + split;
+            const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS + split;
             p.part_m[o] = -__builtin_inff();
             p.part_l[o] = 0.0f;
         }
@@ -889,7 +911,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     const int last_page_idx = (L - 1) >> BSL;
     const int max_page = p.num_blocks - 1;
     const uint8_t* cache = p.cache;
-    constexpr int64_t page_bytes = int64_t(BS) * ROWB;
+    const int64_t page_bytes = int64_t(BS) * row_bytes;
 
     // ---- page ids of the split in registers (see the direct kernel) ---------------------
     const int split_p0 = rowwide ? 0 : begin >> BSL;   // page index held by lane 0 of pv[0]
@@ -920,7 +942,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         const int p0 = (t0 >> BSL) - split_p0;
 #pragma unroll
         for (int i = 0; i < PPT; ++i) base[i] = cache + int64_t(page_id(p0 + i)) * page_bytes;
-        const uint32_t in_page = BS >= 32 ? uint32_t((t0 & (BS - 1)) * ROWB) : 0u;
+        const uint32_t in_page = BS >= 32 ? uint32_t((t0 & (BS - 1)) * row_bytes) : 0u;
 #pragma unroll
         for (int k = 0; k < ROUNDS; ++k) {
             // where a page is a whole number of wavefront rounds (16 rows of 68 chunks = 17 x 64), a
@@ -971,7 +993,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
                 c_page[k] = pg;
                 const int sub = (k < FULL || !kHalfTail) ? 0 : 8 * (ct & 1);
-                c_src[k] = uint32_t(16 * (c - pg * PC) + sub);
+                c_src[k] = staged_src_offset<PROD>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
                 c_dst[k] = kChunkDst<PROD>.off[c] + sub;
             }
             const bool has_rest = kHalfTail || ct < REST;
@@ -981,7 +1003,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 const int p0 = (t0 >> BSL) - split_p0;
 #pragma unroll
                 for (int i = 0; i < PPT; ++i) base[i] = cache + int64_t(page_id(p0 + i)) * page_bytes;
-                const uint32_t in_page = BS >= 32 ? uint32_t((t0 & (BS - 1)) * ROWB) : 0u;
+                const uint32_t in_page = BS >= 32 ? uint32_t((t0 & (BS - 1)) * row_bytes) : 0u;
 #pragma unroll
                 for (int k = 0; k < NR; ++k) {
                     constexpr bool kUniformPage = (BS * kChunksPerRow) % 64 == 0;
@@ -1075,8 +1097,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 split_rotation_block<D>(rot_b, rot_hi, rot_lo);
                 if constexpr (PROD) split_rotation_block<D>(rot_s, sk_hi, sk_lo);
             }
-            for (int rb = 0; 16 * rb < p.H_Q; ++rb) {
-                const int row = 16 * rb + n < p.H_Q ? 16 * rb + n : p.H_Q - 1;
+            for (int rb = 0; 16 * rb < HQG; ++rb) {
+                const int row = 16 * rb + n < HQG ? 16 * rb + n : HQG - 1;
                 uint4v raw[KS];
 #pragma unroll
                 for (int j = 0; j < KS; ++j)
@@ -1099,13 +1121,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int head = 16 * rb + 4 * g + i;
-                    if (head < p.H_Q) qs[head * D + 16 * h + n] = store_elem<DT>(acc[i] * up);
+                    if (head < HQG) qs[head * D + 16 * h + n] = store_elem<DT>(acc[i] * up);
                 }
                 if constexpr (PROD) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int head = 16 * rb + 4 * g + i;
-                        if (head < p.H_Q) qs2[head * D + 16 * h + n] = acc2[i] * up;
+                        if (head < HQG) qs2[head * D + 16 * h + n] = acc2[i] * up;
                     }
                 }
             }
@@ -1411,7 +1433,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         }
     }
     if (g == 0 && n < p.G) {
-        const int64_t o = (int64_t(seq) * p.H_Q + hq_lane) * NS + split;
+        const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS + split;
         p.part_m[o] = M;
         p.part_l[o] = lsum;
     }
@@ -1420,7 +1442,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         for (int i = 0; i < 4; ++i) {
             const int head = 4 * g + i;
             if (head < p.G) {
-                float* dst = p.part_acc + ((int64_t(seq) * p.H_Q + h * p.G + head) * NS + split) * D + n * DPL;
+                float* dst = p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + h * p.G + head) * NS + split) * D + n * DPL;
 #pragma unroll
                 for (int q4 = 0; q4 < DPL / 4; ++q4) {
                     const float4v v = {O[4 * q4][i], O[4 * q4 + 1][i], O[4 * q4 + 2][i], O[4 * q4 + 3][i]};
@@ -1646,16 +1668,16 @@ inline int staged_balance_slots(int num_seqs, int num_splits) {
     return (num_seqs <= 64 && int64_t(num_seqs) * num_splits > cus) ? cus : 0;
 }
 
-// The staged kernel covers 8 KV heads of dimension 128.
+// The staged kernel covers KV heads of dimension 128 in groups of 8.
 inline bool staged_applies(int D, int H_KV) {
-    return D == 128 && H_KV == 8 && !fq_host::force_direct_decode();
+    return D == 128 && H_KV >= 8 && H_KV % 8 == 0 && !fq_host::force_direct_decode();
 }
 
 template <bool PROD, typename K>
 int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream, int copy_waves = 0) {
     // dynamic part only; the 64 KB table is static
     const size_t lds = 2 * size_t(StagedCfg<PROD>::TILE_BYTES);
-    return launch_with_lds(kernel, p, dim3(S, p.num_splits, 1), dim3(512 + 64 * copy_waves), lds, stream);
+    return launch_with_lds(kernel, p, dim3(S, p.num_splits, PROD ? 1 : p.H_KV / 8), dim3(512 + 64 * copy_waves), lds, stream);
 }
 
 // The staged kernel runs with four more wavefronts that only copy; the switch
@@ -1701,7 +1723,10 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
     // four page-id registers also when they can hold the whole block-table row
     if (staged_applies(D, p.H_KV)) {
         DecodeParams ps = p;
-        ps.balance_slots = staged_balance_slots(S, p.num_splits);
+        // every group of 8 heads is a slice of the grid with the same (sequence, split) pairs
+        const int groups = p.H_KV / 8;
+        ps.balance_slots = staged_balance_slots(S, p.num_splits * groups);
+        if (ps.balance_slots > 0) ps.balance_slots = ps.balance_slots / groups > 0 ? ps.balance_slots / groups : 1;
         // a chosen chunk may span up to 256 pages: four page-id registers
         return launch_staged_any<DT, false>(ps, S, BS, wide || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256),
                                             stream);

@@ -250,7 +250,7 @@ def test_shape_limits_of_the_staged_and_prod_decodes(lib):
     """What the kernels cover is a status code at the boundary, not a wrong result: TurboQuantProd pages
     come with 8 KV heads of dimension 128 and at most 64 query heads (the kernel stages 8 heads per token
     row); the query group is at most 16 heads; the staged TQ4 kernel (the one that rotates the query
-    itself) serves 8 KV heads of dimension 128 and every other shape runs the direct kernel."""
+    itself) serves KV heads of dimension 128 in groups of 8 and every other shape runs the direct kernel."""
     f = lib.fq_prod_paged_decode
     f.argtypes = ([ctypes.c_void_p] * 7 + [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 6 +
                   [ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
@@ -268,7 +268,8 @@ def test_shape_limits_of_the_staged_and_prod_decodes(lib):
     assert prod() == FQ_NULL                  # a supported shape gets as far as the pointer check
     lib.fq_paged_decode_fuses_rotation.argtypes = [ctypes.c_int] * 3
     assert lib.fq_paged_decode_fuses_rotation(128, 8, 1) == 1
-    for d, hkv in ((64, 8), (256, 8), (128, 4), (128, 16), (128, 2)):
+    assert lib.fq_paged_decode_fuses_rotation(128, 16, 1) == 1 and lib.fq_paged_decode_fuses_rotation(128, 40, 1) == 1
+    for d, hkv in ((64, 8), (256, 8), (128, 4), (128, 12), (128, 2)):
         assert lib.fq_paged_decode_fuses_rotation(d, hkv, 1) == 0
     # a pre-rotated query with a rotation matrix is only accepted where the kernel rotates it
     g = lib.fq_paged_tq4_decode

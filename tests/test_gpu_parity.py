@@ -311,6 +311,16 @@ def test_paged_decode_more_kv_heads_than_a_workgroup():
     _decode_case([50, 120], hq=24, hkv=12, num_splits=2)
 
 
+@pytest.mark.parametrize("hq,hkv,bs,splits", [(16, 16, 16, 0), (32, 16, 8, 3), (64, 32, 32, 2), (40, 40, 16, 5), (96, 24, 16, 1)])
+def test_paged_decode_kv_heads_in_groups_of_eight(hq, hkv, bs, splits, kernel_option):
+    """A multiple of 8 KV heads runs the staged kernel once per group of 8 (each workgroup copies its
+    group's slices of the token rows): against the oracle, and the direct kernel agrees."""
+    lens = [70, 0, 333, 16, 129]
+    _decode_case(lens, hq=hq, hkv=hkv, bs=bs, num_splits=splits, seed=41)
+    kernel_option("decode_direct", True)
+    _decode_case(lens, hq=hq, hkv=hkv, bs=bs, num_splits=splits, seed=41)
+
+
 def test_paged_decode_rotated_space_and_out_argument():
     c, b, r = book(128)
     q, cache, table, sl = build_paged_case([90, 10], 8, 2)
