@@ -633,11 +633,23 @@ __device__ unsigned int g_decode_faults = 0u;
 // Byte offset, inside a page of `H` KV heads, of chunk `cc` of the 8-head rows that head group `hgrp`
 // (heads 8 hgrp .. 8 hgrp + 7) sees: the group's slices of the four sections of a token row laid end
 // to end, kChunksPerRow chunks per token.  With 8 heads the slices are the row itself (16 cc).
-template <bool PROD>
+//
+// HALF (4 KV heads): the kernel works on rows of 8 "heads" made of two consecutive tokens, head h of
+// the even token as head h and of the odd token as head 4 + h, so row r is the real rows 2 r and
+// 2 r + 1 (544 bytes each) with their sections interleaved; a page then holds half as many rows.
+template <bool PROD, bool HALF>
 __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     constexpr int CPR = StagedCfg<PROD>::CHUNKS_PER_ROW;
     if constexpr (PROD) return uint32_t(16 * cc);          // TurboQuantProd pages come with 8 KV heads
     const int r = cc / CPR, ci = cc - r * CPR;
+    if constexpr (HALF) {
+        int tok, off;                                      // which of the two tokens, offset in its 544-byte row
+        if (ci < 32) { tok = ci >> 4; off = 16 * (ci & 15); }                      // K indices, 256 bytes per token
+        else if (ci < 34) { tok = ci - 32; off = 256; }                            // K norms, 16 bytes
+        else if (ci < 66) { tok = (ci - 34) >> 4; off = 272 + 16 * ((ci - 34) & 15); }   // V indices
+        else { tok = ci - 66; off = 528; }                                         // V norms
+        return uint32_t((2 * r + tok) * 544 + off);
+    }
     int off;
     if (ci < 32) off = 512 * hgrp + 16 * ci;                               // K indices
     else if (ci < 34) off = H * 64 + 32 * hgrp + 16 * (ci - 32);           // K norms
@@ -646,8 +658,9 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     return uint32_t(r * (H * 136) + off);
 }
 
-template <int BSL, int GP, int DT, int PVR, bool PROD, int CW>
+template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
+    static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
     using Cfg = StagedCfg<PROD>;
     constexpr int kStageBytes = Cfg::STAGE_BYTES;
     constexpr int kTileBytes = Cfg::TILE_BYTES;
@@ -658,7 +671,6 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     constexpr int KS = 4;                 // k-steps of the score product
     constexpr int DPL = 8;                // V coordinates per lane
     constexpr int NSC = GP / 2;           // scores per lane per tile
-    constexpr int ROWB = Cfg::ROWB;       // 1088, or 1120 with residual norms
     constexpr int PPT = BS >= 32 ? 1 : 32 / BS;   // pages per tile
 
     // The table is a static array so that its LDS address is a compile-time constant
@@ -690,9 +702,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // More than 8 KV heads: a workgroup serves the group of 8 heads blockIdx.z, i.e. the query heads
     // hq0 .. hq0 + 8 G - 1, and copies that group's slices of the token rows.
     const int hgrp = blockIdx.z;
-    const int HQG = 8 * p.G;                   // query heads of a group
+    const int HQG = (HALF ? 4 : 8) * p.G;      // query heads of a group
     const int hq0 = hgrp * HQG;
-    const int row_bytes = p.H_KV * (PROD ? 140 : 136);   // a token row of the cache (ROWB with 8 heads)
+    const int row_bytes = HALF ? 1088 : p.H_KV * (PROD ? 140 : 136);   // a row of the cache as the kernel sees it
+    // HALF: wavefront h works on real head h % 4 and on the tokens of parity h / 4 (rows are token pairs)
+    const int hr = HALF ? (h & 3) : h;
+    const int tsel = HALF ? (h >> 2) & 1 : 0;
 
     // Every load that depends on nothing is asked for first, so that the memory
     // latencies of the prologue overlap instead of adding up: the centroids, the
@@ -745,7 +760,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
         src_page[k] = pg;
         const int sub = (kSpreadTail && k == 4) ? 4 * (tid & 3) : 0;
-        src_off[k] = staged_src_offset<PROD>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+        src_off[k] = staged_src_offset<PROD, HALF>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
         dst_off[k] = kChunkDst<PROD>.off[c] + sub;
     }
     const bool has_round4 = kSpreadTail || tid < kChunksPerTile - 4 * 512;   // else whole wavefronts
@@ -806,8 +821,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         cand = cand > chunk ? cand : chunk;
         const float rc = __builtin_amdgcn_rcpf(float(cand));
         const int nseq = int(gridDim.x);
-        int l_mine = lane < nseq ? p.seq_lens[lane] : 0;
-        l_mine = l_mine < 0 ? 0 : (l_mine > p.max_blocks * BS ? p.max_blocks * BS : l_mine);
+        int l_real = lane < nseq ? p.seq_lens[lane] : 0;
+        l_real = l_real < 0 ? 0 : (l_real > p.max_blocks * BS * (HALF ? 2 : 1) ? p.max_blocks * BS * (HALF ? 2 : 1) : l_real);
+        const int l_mine = HALF ? (l_real + 1) >> 1 : l_real;      // in rows
         float groups = 0.0f;
         for (int sq = 0; sq < nseq; ++sq)
             groups += __builtin_ceilf(float(__builtin_amdgcn_readlane(l_mine, sq)) * rc - 0.0009765625f);
@@ -852,7 +868,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             split = __builtin_amdgcn_readlane(n_mine, s_idx) + (e - __builtin_amdgcn_readlane(dead_incl - dead_mine, s_idx));
             split = split < NS ? split : NS - 1;
         }
-        L_known = __builtin_amdgcn_readlane(l_mine, seq);
+        L_known = __builtin_amdgcn_readlane(l_real, seq);
     }
 
     const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + (int64_t(seq) * p.H_Q + hq0) * 128;
@@ -896,13 +912,21 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         load_first_heads();
     }
     L = L < 0 ? 0 : L;
-    L = L > p.max_blocks * BS ? p.max_blocks * BS : L;
+    L = L > p.max_blocks * BS * (HALF ? 2 : 1) ? p.max_blocks * BS * (HALF ? 2 : 1) : L;
+    // HALF: from here on L counts rows (token pairs); a wavefront's last row may hold a token of the
+    // other parity only
+    const int rows_mine = HALF ? (L + 1 - tsel) >> 1 : L;
+    L = HALF ? (L + 1) >> 1 : L;
     const int begin = split * chunk;
     const int end = L < begin + chunk ? L : begin + chunk;
-    const int hq_lane = h * p.G + n;
+    const int end_mine = rows_mine < end ? rows_mine : end;      // rows < end_mine hold a token of this wavefront
+    const int hq_lane = hr * p.G + n;
+    // HALF: the two parities of a head are two partials, 2 split + parity of 2 NS
+    const int NS_out = HALF ? 2 * NS : NS;
+    const int split_out = HALF ? 2 * split + tsel : split;
     if (begin >= end) {   // uniform over the workgroup
         if (g == 0 && n < p.G && !copier) {
-            const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS + split;
+            const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS_out + split_out;
             p.part_m[o] = -__builtin_inff();
             p.part_l[o] = 0.0f;
         }
@@ -993,7 +1017,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
                 c_page[k] = pg;
                 const int sub = (k < FULL || !kHalfTail) ? 0 : 8 * (ct & 1);
-                c_src[k] = staged_src_offset<PROD>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+                c_src[k] = staged_src_offset<PROD, HALF>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
                 c_dst[k] = kChunkDst<PROD>.off[c] + sub;
             }
             const bool has_rest = kHalfTail || ct < REST;
@@ -1137,7 +1161,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             } else {
                 __syncthreads();
             }
-            const uint16_t* src = qs + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
+            const uint16_t* src = qs + (hr * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const uint4v raw = *reinterpret_cast<const uint4v*>(src + 8 * ks);
@@ -1151,7 +1175,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             }
             if constexpr (PROD) {
                 // <S q, signs> * sqrt(pi/2) / D: the constant rides on the query side
-                const float* src2 = qs2 + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
+                const float* src2 = qs2 + (hr * p.G + (live ? hd : 0)) * D + g * (D / 4);
                 float qf2[KS][8];
                 float mx2 = 0.0f;
 #pragma unroll
@@ -1175,7 +1199,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             if constexpr (CW > 0) lds_flag_signal(&flags[1], lane);
             else if constexpr (PROD) __syncthreads();
         } else {
-            const uint16_t* qsrc = qseq + (h * p.G + (live ? hd : 0)) * D + g * (D / 4);
+            const uint16_t* qsrc = qseq + (hr * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const uint4v raw = *reinterpret_cast<const uint4v*>(qsrc + 8 * ks);
@@ -1298,7 +1322,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 s = acc[e >> 2][e & 3];
                 if (PROD) s2 = acc_s[e >> 2][e & 3];
             }
-            const bool live = t0 + sc_tok[e] < end;
+            const bool live = t0 + sc_tok[e] < end_mine;
             rv[e] = live ? vn[e] : 0.0f;
             float sc = s * kn[e] * qscale;
             if (PROD) sc = __builtin_fmaf(s2 * kg[e], qscale_s, sc);
@@ -1317,7 +1341,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             const float w = __builtin_amdgcn_exp2f(d);
             psum += w;
             wv[e] = w * rv[e];
-            redo = redo || d > kMaxLead || wv[e] > kHalfSafe;
+            // (HALF: the first tile of a split may hold no token of this wavefront's parity; -inf - -inf
+            // is then NaN in every lane, and the vote must still send the tile through the safe path)
+            redo = redo || (HALF ? !(d <= kMaxLead) : d > kMaxLead) || wv[e] > kHalfSafe;
         }
         if (__any(redo)) {
             // The reference moves to max(M, max over the tile of (score + bias)), where the bias of a
@@ -1433,7 +1459,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         }
     }
     if (g == 0 && n < p.G) {
-        const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS + split;
+        const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS_out + split_out;
         p.part_m[o] = M;
         p.part_l[o] = lsum;
     }
@@ -1442,7 +1468,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         for (int i = 0; i < 4; ++i) {
             const int head = 4 * g + i;
             if (head < p.G) {
-                float* dst = p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + h * p.G + head) * NS + split) * D + n * DPL;
+                float* dst = p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS_out + split_out) * D + n * DPL;
 #pragma unroll
                 for (int q4 = 0; q4 < DPL / 4; ++q4) {
                     const float4v v = {O[4 * q4][i], O[4 * q4 + 1][i], O[4 * q4 + 2][i], O[4 * q4 + 3][i]};
@@ -1713,8 +1739,42 @@ int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream
     return FQ_ERR_UNSUPPORTED_BLOCK;
 }
 
+// 4 KV heads of dimension 128 on pages of 16 or 32 tokens: the staged kernel on rows of two tokens
+// (`rows_per_page` = block_size / 2), with its copy wavefronts.
+inline bool staged_half_applies(int D, int H_KV, int block_size) {
+    return D == 128 && H_KV == 4 && block_size >= 16 && !fq_host::force_direct_decode() && staged_copy_waves() == 4;
+}
+template <int DT>
+int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wide, hipStream_t stream) {
+    const size_t lds = 2 * size_t(StagedCfg<false>::TILE_BYTES);
+    const dim3 grid(S, p.num_splits, 1), block(512 + 64 * 4);
+#define FQ_HALF_GP(BSL, GPV)                                                                                      \
+    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, true>, p, grid, block, lds, stream) \
+                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, true>, p, grid, block, lds, stream)
+#define FQ_HALF_BS(BSL)                          \
+    do {                                         \
+        if (p.G <= 4) { FQ_HALF_GP(BSL, 4); }    \
+        else if (p.G <= 8) { FQ_HALF_GP(BSL, 8); } \
+        else { FQ_HALF_GP(BSL, 16); }            \
+    } while (0)
+    if (rows_per_page == 8) FQ_HALF_BS(3);
+    else FQ_HALF_BS(4);
+#undef FQ_HALF_BS
+#undef FQ_HALF_GP
+}
+
 template <int D, int DT>
-int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream) {
+int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bool allow_half) {
+    if (allow_half && staged_half_applies(D, p.H_KV, BS)) {
+        // the kernel counts rows of two tokens: half the page size, chunks of rows
+        const int rows_per_page = BS / 2;
+        const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
+        const int64_t chunk_rows = (((max_rows + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
+        DecodeParams ps = p;
+        ps.balance_slots = staged_balance_slots(S, p.num_splits);
+        const bool wide_rows = chunk_rows / rows_per_page > 64 || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256);
+        return launch_staged_half<DT>(ps, S, rows_per_page, wide_rows, stream);
+    }
     // pages a split can span: its tokens are ceil(max_ctx / splits) rounded up to a tile
     const int64_t max_ctx = int64_t(p.max_blocks) * BS;
     const int64_t chunk = (((max_ctx + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
@@ -1837,7 +1897,9 @@ extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_siz
     // one round of workgroups over the chip (8 wavefronts per CU, one wavefront per sequence,
     // KV head and split) ...
     const int64_t target_waves = int64_t(fq_host::device_cu_count()) * 8;
-    const int64_t one_round = (target_waves + int64_t(num_seqs) * H_KV - 1) / (int64_t(num_seqs) * H_KV);
+    // (4 KV heads run as 8: the staged kernel reads their tokens in pairs)
+    const int64_t heads = H_KV == 4 ? 8 : H_KV;
+    const int64_t one_round = (target_waves + int64_t(num_seqs) * heads - 1) / (int64_t(num_seqs) * heads);
     // ... and twice that when the contexts are long enough for splits of 1024 tokens: the lengths
     // of the sequences are not known here, a ragged batch leaves many splits empty, and the
     // kernel can merge splits (it sizes its chunks from the actual lengths) but not divide them
@@ -1865,6 +1927,8 @@ extern "C" size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_K
                                                   int max_blocks_per_seq, int num_splits) {
     if (num_seqs <= 0 || H_Q <= 0 || H_KV <= 0 || D <= 0) return 0;
     num_splits = fq::effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
+    // room for the two partials per split of the 4-KV-head staged decode, whatever the switches say
+    if (D == 128 && H_KV == 4 && block_size >= 16) num_splits *= 2;
     return fq::workspace_layout(num_seqs, H_Q, D, num_splits).total;
 }
 
@@ -1890,7 +1954,7 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
                     const int32_t* seq_lens, const float* centroids_k, const float* centroids_v, float* partial_acc,
                     float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D, int block_size,
                     int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype, int num_splits,
-                    void* stream) {
+                    void* stream, bool allow_half = false) {
     const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
                                        num_splits);
     if (bad != FQ_OK) return bad;
@@ -1915,8 +1979,8 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define FQ_DECODE_D(DD)                                                                 \
     case DD:                                                                            \
-        return dtype == FQ_F16 ? launch_partials<DD, FQ_F16>(p, num_seqs, block_size, s) \
-                               : launch_partials<DD, FQ_BF16>(p, num_seqs, block_size, s);
+        return dtype == FQ_F16 ? launch_partials<DD, FQ_F16>(p, num_seqs, block_size, s, allow_half) \
+                               : launch_partials<DD, FQ_BF16>(p, num_seqs, block_size, s, allow_half);
     switch (D) {
         FQ_DECODE_D(64)
         FQ_DECODE_D(128)
@@ -1983,7 +2047,10 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     if (!q || !out) return FQ_ERR_NULL_POINTER;
     if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16)) return FQ_ERR_MISALIGNED;
     num_splits = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
-    const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_splits);
+    // 4 KV heads: the staged kernel reads rows of two tokens and writes one partial per token parity
+    const bool half = staged_half_applies(D, H_KV, block_size);
+    const int num_partials = half ? 2 * num_splits : num_splits;
+    const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_partials);
     if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
     if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
@@ -1993,7 +2060,7 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     const void* q_in = q;
     const float* fused_rotation = nullptr;
     if (rotation) {
-        if (centroids_k && staged_applies(D, H_KV)) {
+        if (centroids_k && (half || staged_applies(D, H_KV))) {
             fused_rotation = rotation;       // the staged kernel rotates the query in its prologue
         } else {
             const int st = fq_rotate_query(q, rotation, rotation_col_major, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
@@ -2003,9 +2070,9 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     }
     int st = decode_partials(q_in, fused_rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m,
                              l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
-                             num_splits, stream);
+                             num_splits, stream, half);
     if (st != FQ_OK) return st;
-    return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_splits, stream);
+    return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_partials, stream);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -2064,7 +2131,8 @@ extern "C" int fq_split_k_paged_decode_static(const void* q, const uint8_t* kv_c
     if (num_seqs == 0) return FQ_OK;
     const int ns = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
     // the partials of this launch must fit the array: a larger problem is refused, not truncated
-    if (workspace_layout(num_seqs, H_Q, D, ns).total > kStaticScratchBytes) return FQ_ERR_WORKSPACE;
+    const int num_partials = staged_half_applies(D, H_KV, block_size) ? 2 * ns : ns;
+    if (workspace_layout(num_seqs, H_Q, D, num_partials).total > kStaticScratchBytes) return FQ_ERR_WORKSPACE;
     void* ws = nullptr;
     const int st = static_scratch_address(&ws);
     if (st != FQ_OK) return st;

@@ -321,6 +321,29 @@ def test_paged_decode_kv_heads_in_groups_of_eight(hq, hkv, bs, splits, kernel_op
     _decode_case(lens, hq=hq, hkv=hkv, bs=bs, num_splits=splits, seed=41)
 
 
+@pytest.mark.parametrize("hq,bs,splits,dtype", [(16, 16, 0, torch.bfloat16), (4, 16, 3, torch.bfloat16),
+                                                (32, 32, 2, torch.float16), (64, 16, 1, torch.bfloat16),
+                                                (8, 32, 5, torch.float16), (16, 16, 40, torch.bfloat16)])
+def test_paged_decode_four_kv_heads_on_token_pairs(hq, bs, splits, dtype, kernel_option):
+    """4 KV heads of dimension 128 on pages of 16 or 32 tokens run the staged kernel on rows of two
+    tokens (the even and the odd tokens of a head are combined as two partials).  Odd and even
+    lengths, lengths one past a chunk of 64 token pairs, empty sequences; against the oracle, and the
+    direct kernel (also the one that serves pages of 8 tokens) agrees."""
+    lens = [70, 0, 333, 16, 129, 1, 2, 257, 127, 128]
+    _decode_case(lens, hq=hq, hkv=4, bs=bs, num_splits=splits, seed=43, dtype=dtype)
+    kernel_option("decode_direct", True)
+    _decode_case(lens, hq=hq, hkv=4, bs=bs, num_splits=splits, seed=43, dtype=dtype)
+
+
+def test_paged_decode_four_kv_heads_ragged_long_contexts():
+    """More (sequence, split) workgroups than CUs with 4 KV heads: chunks sized from the actual lengths,
+    counted in token pairs."""
+    lens = [1500, 0, 37, 6001, 64, 2049, 1, 3333]
+    _decode_case(lens, hq=16, hkv=4, num_splits=40)
+    _decode_case(lens, hq=32, hkv=4, num_splits=64, bs=32, dtype=torch.float16)
+    _decode_case(lens, hq=16, hkv=4, num_splits=0, bs=8)          # pages of 8 tokens: the direct kernel
+
+
 def test_paged_decode_rotated_space_and_out_argument():
     c, b, r = book(128)
     q, cache, table, sl = build_paged_case([90, 10], 8, 2)
