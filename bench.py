@@ -294,6 +294,17 @@ def main():
         c_ms, _ = time_events(lambda i: K.tq4_compress(x, rot_d, bnd_d, rotation_T_even=ev, rotation_T_odd=od,
                                                        out=(packed, norms)), EXTRA_ITERS)
         nrows = rows_tok * H_KV
+        if check is not None:
+            # the indices and norms of a sample of the rows just compressed, against the oracle
+            ns = 2048
+            idx_want, norms_want, _ = O.compress_indices(x[:ns].cpu(), rot, book[1].cpu())
+            idx_got = O.nibble_unpack(packed[:ns].cpu())
+            rate = (idx_got != idx_want).float().mean().item()
+            nrel = ((norms[:ns].cpu() - norms_want).abs() / norms_want.clamp_min(1e-30)).max().item()
+            check.update({"compress_index_mismatch_rate": rate, "compress_rows_checked": ns * H_KV,
+                          "compress_norm_max_rel_err": nrel,
+                          "compress_tolerance": "index mismatches on at most 1e-4 of the entries"})
+            check["ok"] = bool(check["ok"] and rate <= 1e-4 and nrel <= 1e-5)
         extra.update({
             "compress_rows": nrows,
             "compress_ms": c_ms,
@@ -301,8 +312,9 @@ def main():
             "compress_mtok_per_s": rows_tok / (c_ms * 1e-3) / 1e6,
             "compress_gbps": nrows * 324 / (c_ms * 1e-3) / 1e9,
             "compress_pct_hbm_peak": 100.0 * nrows * 324 / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-            # bf16 rows against the 3-term bf16 split of the rotation: 3 x 2 D^2 flops per row on the MFMA
-            "compress_tflops_bf16_mfma": nrows * 3 * 2 * D * D / (c_ms * 1e-3) / 1e12,
+            # bf16 rows against the 2-term bf16 split of the rotation: 2 x 2 D^2 flops per row on the MFMA
+            "compress_matrix_terms": 2,
+            "compress_tflops_bf16_mfma": nrows * 2 * 2 * D * D / (c_ms * 1e-3) / 1e12,
         })
         del x
         torch.cuda.empty_cache()

@@ -49,6 +49,7 @@ int option_id(const std::string& name) {
     if (name == "decode_direct") return FQ_OPT_DECODE_DIRECT;
     if (name == "attention_any_dim") return FQ_OPT_ATTENTION_ANY_DIM;
     if (name == "decode_tiny_spin") return FQ_OPT_DECODE_TINY_SPIN;
+    if (name == "compress_three_terms") return FQ_OPT_COMPRESS_THREE_TERMS;
     throw std::invalid_argument("unknown option '" + name + "'");
 }
 
@@ -786,7 +787,7 @@ void bind_kernels(py::module_& m) {
               fqbind::raise_on_error(fq_set_option(id, value ? 1 : 0), "set_option");
               return before != 0;
           }, py::arg("name"), py::arg("value"),
-          "Set a kernel-variant switch ('decode_copy_waves', 'decode_direct', 'attention_any_dim'); returns the old value");
+          "Set a kernel-variant switch ('decode_copy_waves', 'decode_direct', 'attention_any_dim', 'compress_three_terms'); returns the old value");
     m.def("get_option", [](const std::string& name) { return fq_get_option(option_id(name)) != 0; }, py::arg("name"));
     m.def("paged_decode_fault_count", []() {
               unsigned int n = 0;

@@ -23,6 +23,8 @@ void init_options() {
         v = std::getenv("FQ_ATTENTION_ANY_DIM");
         g_options[FQ_OPT_ATTENTION_ANY_DIM] = (v != nullptr && v[0] == '1') ? 1 : 0;
         g_options[FQ_OPT_DECODE_TINY_SPIN] = 0;
+        v = std::getenv("FQ_COMPRESS_THREE_TERMS");
+        g_options[FQ_OPT_COMPRESS_THREE_TERMS] = (v != nullptr && v[0] == '1') ? 1 : 0;
     });
 }
 }  // namespace

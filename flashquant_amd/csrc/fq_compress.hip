@@ -54,6 +54,11 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ __bf16 bf16_trunc(float f) {
     return __builtin_bit_cast(__bf16, uint16_t(float_to_bits(f) >> 16));
 }
+// nearest bf16, ties to even (finite inputs)
+__device__ __forceinline__ __bf16 bf16_nearest(float f) {
+    const uint32_t b = float_to_bits(f);
+    return __builtin_bit_cast(__bf16, uint16_t((b + 0x7fffu + ((b >> 16) & 1u)) >> 16));
+}
 __device__ __forceinline__ float bf16_value(__bf16 h) {
     return bits_to_float(uint32_t(__builtin_bit_cast(uint16_t, h)) << 16);
 }
@@ -65,11 +70,19 @@ __device__ __forceinline__ float dpp_f32(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
 
-// 64 cells over the span of the boundaries, every cell stored 32 times side by side (a cell is a
+// 128 cells over the span of the boundaries, every cell stored 32 times side by side (a cell is a
 // 256-byte row of 32 copies of 8 bytes): lane l reads copy l % 32, so the lanes of a half-wave
 // always hit different banks whatever cells their values fall in.  A single copy made the
 // data-dependent lookups collide (4-5 lanes per bank on average).
-constexpr int kBucketCells = 64;
+//
+// The table is the first object of the kernel's LDS block, at LDS address 0: the address of a lane's
+// copy of cell c is then (c << 8) | (8 * copy), which v_cvt_pk_u8_f32 builds in one instruction from
+// the cell coordinate (float -> integer saturated to 0..255, written into byte 1 of the lane's
+// constant 8 * copy).  A value y is looked up by its cell coordinate pos = y / w + offset and compared
+// with the cell's boundary as it is (in the cell coordinate values within 3e-8 of the boundary 0 would
+// lose their sign, which is all that rows of negligible norm have).  The conversion's rounding is left
+// open: a cell answers for the coordinates one cell to either side of its own as well.
+constexpr int kBucketCells = 128;
 constexpr int kBucketCopies = 32;
 struct BucketTable {
     uint2v cell[kBucketCells * kBucketCopies];   // x = threshold bits, y = base count
@@ -78,52 +91,64 @@ struct BucketTable {
     float offset;
     int slow;
 };
+typedef __attribute__((address_space(3))) const uint2v lds_cell_t;
+
+// LDS address of an object
+template <typename T>
+__device__ __forceinline__ uint32_t lds_address(const T* p) {
+    return uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)p));
+}
 
 // Builds the cell table from the 15 boundaries (block-wide, ends with a barrier).
 __device__ __forceinline__ void build_bucket_table(BucketTable& t, const float* __restrict__ boundaries,
                                                    int tid, int nthreads) {
     if (tid < 15) t.bnd[tid] = boundaries[tid];
     if (tid == 15) t.bnd[15] = __builtin_inff();
-    if (tid == 0) t.slow = 0;
+    // the one-instruction address needs the table at LDS address 0
+    if (tid == 0) t.slow = lds_address(&t.cell[0]) != 0u ? 1 : 0;
     __syncthreads();
     const float b0 = t.bnd[0], b14 = t.bnd[14];
     const float span = b14 - b0;
-    const float pad = span > 0.0f ? span * (1.0f / float(kBucketCells)) : 1.0f;
-    const float lo = b0 - pad;
-    const float w = (span + 2.0f * pad) * (1.0f / float(kBucketCells));
-    const float margin = 0.01f * w;
+    // two cells of padding on either side of the outer boundaries
+    const float w = span > 0.0f ? span * (1.0f / float(kBucketCells - 4)) : 1.0f;
+    const float lo = b0 - 2.0f * w;
+    const float inv_w = 1.0f / w, offset = -lo / w;
     for (int c = tid; c < kBucketCells; c += nthreads) {
-        const float lo_c = lo + w * float(c) - margin;
-        const float hi_c = lo + w * float(c + 1) + margin;
+        // coordinates that may be converted to cell c: [c - 1, c + 2), with a margin for rounding
+        const float lo_c = float(c) - 1.01f;
+        const float hi_c = float(c) + 2.01f;
         int base = 0, inside = 0;
         float thr = __builtin_inff();
         for (int b = 0; b < 15; ++b) {
-            const float v = t.bnd[b];
+            const float v = __builtin_fmaf(t.bnd[b], inv_w, offset);
             if (v < lo_c) {
                 ++base;
             } else if (v <= hi_c) {
                 ++inside;
-                thr = v;
+                thr = t.bnd[b];
             }
         }
         if (inside > 1 || !(span > 0.0f)) t.slow = 1;
         for (int k = 0; k < kBucketCopies; ++k) t.cell[c * kBucketCopies + k] = uint2v{float_to_bits(thr), uint32_t(base)};
     }
     if (tid == 0) {
-        t.inv_w = 1.0f / w;
-        t.offset = -lo / w;
+        t.inv_w = inv_w;
+        t.offset = offset;
     }
     __syncthreads();
 }
 
-// `copy` = lane % 32
-__device__ __forceinline__ uint2v bucket_cell(const BucketTable& t, float y, float inv_w, float offset, int copy) {
+// `copy8` = 8 * (lane % 32)
+__device__ __forceinline__ uint2v bucket_cell(float y, float inv_w, float offset, uint32_t copy8) {
     const float pos = __builtin_fmaf(y, inv_w, offset);
-    const int c = int(__builtin_amdgcn_fmed3f(pos, 0.0f, float(kBucketCells - 1)));
-    return t.cell[c * kBucketCopies + copy];
+    // the conversion saturates at 0 and 255, the table ends at cell 127; the median also sends a NaN
+    // to cell 0 (no boundary lies below a NaN: index 0, as the reference's count gives)
+    const float top = __builtin_amdgcn_fmed3f(pos, 0.0f, float(kBucketCells - 1));
+    const uint32_t addr = __builtin_amdgcn_cvt_pk_u8_f32(top, 1u, copy8);
+    return *reinterpret_cast<lds_cell_t*>(addr);
 }
-__device__ __forceinline__ uint32_t bucket_fast(const BucketTable& t, float y, float inv_w, float offset, int copy) {
-    const uint2v e = bucket_cell(t, y, inv_w, offset, copy);
+__device__ __forceinline__ uint32_t bucket_fast(float y, float inv_w, float offset, uint32_t copy8) {
+    const uint2v e = bucket_cell(y, inv_w, offset, copy8);
     return e.y + (bits_to_float(e.x) < y ? 1u : 0u);
 }
 
@@ -150,6 +175,7 @@ struct PagedDest {
     uint8_t* cache;             // (num_slots, H*(D+8))
     const int64_t* slots;       // (mapped,) flat slot of each token; negative: not stored
     int64_t rows_k;             // tokens * H
+    uint32_t tokens;
     int64_t num_slots;
     int mapped;                 // tokens with a slot
     int H;
@@ -160,35 +186,79 @@ struct PagedDest {
     int64_t append_cap, append_pos;
 };
 
-template <int D, int DT, bool PAGED>
+// NT: bf16 terms of the rotation matrix for bf16 rows of head_dim <= 128 (ignored otherwise).
+// 3: R = t0 + t1 + t2 exactly.  2: t0, t1 rounded to nearest, |R - t0 - t1| <= 2^-18 |R|: the rotated
+// coordinates move by about 2e-7 (standard deviation, unit rows of 128 coordinates), which puts about 6
+// indices in a million on the other side of a bucket boundary, for two thirds of the matrix instructions.
+template <int D, int DT, bool PAGED, int NT>
 __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     const uint4v* __restrict__ x, const float* __restrict__ rot_T_even,
     const float* __restrict__ rot_T_odd, const float* __restrict__ boundaries,
     uint8_t* __restrict__ packed, float* __restrict__ norms, int64_t M, int64_t num_tiles, const PagedDest pd) {
     using C = CompressCfg<D>;
-    // paged mode: cache row of a (tensor, token, head) row, or nullptr when the token has no slot
-    auto paged_row = [&](int64_t row, int& head, int& is_v) -> uint8_t* {
-        is_v = row >= pd.rows_k ? 1 : 0;
-        const int64_t r = row - (is_v ? pd.rows_k : 0);
-        const int64_t tok = r / pd.H;
-        head = int(r - tok * pd.H);
-        if (tok >= pd.mapped) return nullptr;
+    // Rows are grouped by a divisor: in paged mode the H heads of a token, in append mode the append_n
+    // new tokens of a (batch, head) pair.  The first row of a tile is row0 = q * divisor + r (Origin,
+    // wave-uniform, carried from tile to tile by additions); row0 + i then belongs to group
+    // q + (r + i) / divisor, at place (r + i) % divisor.  In paged mode rows_k is a multiple of H, so
+    // the same pair serves the rows of both tensors (token counted over keys, then values).
+    struct Origin { uint32_t q, r; };
+    const uint32_t divisor = PAGED ? uint32_t(pd.H) : (pd.append_n != 0u ? pd.append_n : 1u);
+    const float rcp_div = 1.0f / float(divisor);
+    auto origin_of = [&](uint32_t first_tile) {
+        const uint32_t row0 = first_tile * uint32_t(C::TT);      // the first tiles: below 2^32 rows
+        return Origin{row0 / divisor, row0 % divisor};
+    };
+    const Origin tile_step = origin_of(gridDim.x);
+    auto advance = [&](Origin o) {
+        o.q += tile_step.q;
+        o.r += tile_step.r;
+        if (o.r >= divisor) { o.r -= divisor; o.q += 1u; }
+        return o;
+    };
+    // group and place of row i of the tile
+    auto locate = [&](Origin o, int i, uint32_t& group, uint32_t& place) {
+        const uint32_t t = o.r + uint32_t(i);                       // < divisor + TT
+        // t / divisor: (t + 1/2) / divisor lies at least 1 / (2 divisor) away from an integer, far more
+        // than the rounding of the float32 product while the divisor is below 2^20; a larger divisor
+        // exceeds t at most once
+        uint32_t dq = uint32_t(__builtin_fmaf(float(t), rcp_div, 0.5f * rcp_div));
+        if (!PAGED && divisor >= (1u << 20)) dq = t >= divisor ? 1u : 0u;
+        group = o.q + dq;
+        place = t - dq * divisor;
+    };
+    // paged mode: cache row of row i of the tile, or nullptr when the token has no slot
+    auto paged_row = [&](Origin o, int i, int& head, int& is_v) -> uint8_t* {
+        uint32_t tok, hd;
+        locate(o, i, tok, hd);
+        head = int(hd);
+        is_v = tok >= pd.tokens ? 1 : 0;
+        tok -= is_v ? pd.tokens : 0u;
+        if (tok >= uint32_t(pd.mapped)) return nullptr;
         const int64_t slot = pd.slots[tok];
         if (slot < 0 || slot >= pd.num_slots) return nullptr;
         return pd.cache + slot * (int64_t(pd.H) * (D + 8)) + (is_v ? int64_t(pd.H) * (D / 2 + 4) : 0);
     };
-    auto out_row = [&](int64_t row) -> int64_t {
-        if (pd.append_n == 0u) return row;
-        const uint32_t o = uint32_t(row) / pd.append_n;
-        return int64_t(o) * pd.append_cap + pd.append_pos + int64_t(uint32_t(row) - o * pd.append_n);
+    // plain mode appending into a buffer of larger capacity: output row of row i of the tile
+    auto appended_row = [&](Origin o, int i) -> int64_t {
+        uint32_t outer, t;
+        locate(o, i, outer, t);
+        return int64_t(outer) * pd.append_cap + pd.append_pos + int64_t(t);
     };
-    __shared__ __attribute__((aligned(16))) uint8_t xs[2][C::TT * C::XS_STRIDE];
     // bf16 rows of head_dim 128 run a software pipeline (see below) with two packed-row buffers
     constexpr bool kPipe = DT == FQ_BF16 && D == 128;
     constexpr int kOutBytes = C::TT * C::OUT_STRIDE;
-    __shared__ __attribute__((aligned(16))) uint8_t outs[(kPipe ? 2 : 1) * kOutBytes];
-    __shared__ float inv_s[2][C::TT];
-    __shared__ BucketTable table;
+    // one LDS block, the bucket table first (its lookups address it from LDS address 0)
+    struct Lds {
+        BucketTable table;
+        __attribute__((aligned(16))) uint8_t xs[2][C::TT * C::XS_STRIDE];
+        __attribute__((aligned(16))) uint8_t outs[(kPipe ? 2 : 1) * kOutBytes];
+        float inv_s[2][C::TT];
+    };
+    __shared__ __attribute__((aligned(256))) Lds lds;
+    BucketTable& table = lds.table;
+    auto& xs = lds.xs;
+    auto& outs = lds.outs;
+    auto& inv_s = lds.inv_s;
 
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
@@ -200,12 +270,13 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
 
     // ---- the rotation rows of this wave, split into two fp16 terms ----------
     // fp16 rows: R = hi + lo / 4096 in fp16.  bf16 rows go to the bf16 MFMA as they are, against
-    // R = t0 + t1 + t2 in bf16 (3 x 8 bits: the float32 value exactly); bf16 terms keep the
-    // float32 exponent range, so the three products share one accumulator.
-    // (head_dim 256 would need 192 registers for the three terms: it keeps the fp16 route)
+    // R = t0 + t1 (+ t2) in bf16 (3 x 8 bits: the float32 value exactly); bf16 terms keep the
+    // float32 exponent range, so the products share one accumulator.
+    // (head_dim 256 would need 192 registers for three terms: it keeps the fp16 route)
     constexpr bool kBf16 = DT == FQ_BF16 && D <= 128;
+    static_assert(NT == 2 || NT == 3, "two or three bf16 terms");
     half8 a_hi[kBf16 ? 1 : C::NK], a_lo[kBf16 ? 1 : C::NK];
-    bf16x8 a_t[kBf16 ? 3 : 1][kBf16 ? C::NK : 1];
+    bf16x8 a_t[kBf16 ? NT : 1][kBf16 ? C::NK : 1];
     {
         const int j = 32 * cb + mfma_row_to_coord(n32);
         const float* src = (j & 1) ? rot_T_odd : rot_T_even;
@@ -216,12 +287,15 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             for (int e = 0; e < 8; ++e) {
                 const int k = 16 * ks + 8 * kg + e;
                 const float r = src[k * (D / 2) + col];
-                if constexpr (kBf16) {
+                if constexpr (kBf16 && NT == 3) {
                     const __bf16 t0 = bf16_trunc(r);
                     const float r1 = r - bf16_value(t0);
                     const __bf16 t1 = bf16_trunc(r1);
                     const __bf16 t2 = bf16_trunc(r1 - bf16_value(t1));
                     a_t[0][ks][e] = t0; a_t[1][ks][e] = t1; a_t[2][ks][e] = t2;
+                } else if constexpr (kBf16) {
+                    const __bf16 t0 = bf16_nearest(r);
+                    a_t[0][ks][e] = t0; a_t[1][ks][e] = bf16_nearest(r - bf16_value(t0));
                 } else {
                     const _Float16 hi = _Float16(r);
                     a_hi[ks][e] = hi;
@@ -233,30 +307,46 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     build_bucket_table(table, boundaries, tid, C::THREADS);
     const float inv_w = table.inv_w, offset = table.offset;
     const bool slow = table.slow != 0;
+    const uint32_t copy8 = 8u * uint32_t(n32);
 
     // ---- staging helpers -----------------------------------------------------
     const int chunk = tid % C::CPR;
     const int row_in_pass = tid / C::CPR;
     uint4v pre[C::PASSES];
 
-    auto issue_loads = [&](int64_t tile) {
-#pragma unroll
-        for (int p = 0; p < C::PASSES; ++p) {
-            const int64_t row = tile * C::TT + p * C::ROWS_PER_PASS + row_in_pass;
-            if (PAGED) {
-                const bool second = row >= pd.rows_k;
-                const uint4v* src = second ? pd.x_value + (row - pd.rows_k) * C::CPR : x + row * C::CPR;
-                pre[p] = row < M ? __builtin_nontemporal_load(src + chunk) : uint4v{0, 0, 0, 0};
-            } else {
-                pre[p] = row < M ? __builtin_nontemporal_load(x + row * C::CPR + chunk) : uint4v{0, 0, 0, 0};
-            }
-        }
+    // Everything that depends on the tile alone is wave-uniform (scalar registers); a thread adds
+    // 32-bit offsets to it.  rows_in(tile): rows of the tile that exist (0..TT).
+    auto rows_in = [&](int64_t tile) -> int {
+        const int64_t left = M - tile * C::TT;
+        return left >= C::TT ? C::TT : (left > 0 ? int(left) : 0);
     };
-    auto stage = [&](int64_t tile, int buf) {
+    auto issue_loads = [&](int64_t tile) {
+        const int64_t row0 = tile * C::TT;
+        const int live = rows_in(tile);
+        const uint4v* base = x + row0 * C::CPR;
+        // paged mode: rows [rows_k, 2 rows_k) come from the value tensor; a tile may hold rows of both
+        int first_v = C::TT;
+        const uint4v* base_v = base;
+        if (PAGED) {
+            const int64_t k_left = pd.rows_k - row0;
+            first_v = k_left >= C::TT ? C::TT : (k_left > 0 ? int(k_left) : 0);
+            base_v = reinterpret_cast<const uint4v*>(reinterpret_cast<uintptr_t>(pd.x_value) +
+                                                     uintptr_t((row0 - pd.rows_k) * C::CPR * int64_t(sizeof(uint4v))));
+        }
 #pragma unroll
         for (int p = 0; p < C::PASSES; ++p) {
             const int r = p * C::ROWS_PER_PASS + row_in_pass;
-            const int64_t row = tile * C::TT + r;
+            const int off = p * C::ROWS_PER_PASS * C::CPR + tid;           // r * CPR + chunk
+            const uint4v* src = (PAGED && r >= first_v) ? base_v : base;
+            pre[p] = r < live ? __builtin_nontemporal_load(src + off) : uint4v{0, 0, 0, 0};
+        }
+    };
+    auto stage = [&](int64_t tile, Origin org, int buf) {
+        const int live = rows_in(tile);
+        const int64_t row0 = tile * C::TT;
+#pragma unroll
+        for (int p = 0; p < C::PASSES; ++p) {
+            const int r = p * C::ROWS_PER_PASS + row_in_pass;
             float e[8];
             const uint32_t w[4] = {pre[p].x, pre[p].y, pre[p].z, pre[p].w};
             float ss = 0.0f, mx = 0.0f;
@@ -315,13 +405,15 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             *reinterpret_cast<uint4v*>(&xs[buf][r * C::XS_STRIDE + chunk * 16]) = h;
             if (chunk == 0) {
                 inv_s[buf][r] = up * __builtin_amdgcn_rcpf(nrm + 1e-10f);
-                if (row < M) {
+                if (r < live) {
                     if (PAGED) {
                         int head, is_v;
-                        uint8_t* dst = paged_row(row, head, is_v);
+                        uint8_t* dst = paged_row(org, r, head, is_v);
                         if (dst) *reinterpret_cast<float*>(dst + pd.H * (D / 2) + 4 * head) = nrm;
+                    } else if (pd.append_n == 0u) {      // uniform
+                        (norms + row0)[r] = nrm;
                     } else {
-                        norms[out_row(row)] = nrm;
+                        norms[appended_row(org, r)] = nrm;
                     }
                 }
             }
@@ -329,18 +421,19 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     };
 
     // packed rows of a tile: LDS -> global, 16 bytes per lane
-    auto store_tile = [&](int64_t tile, const uint8_t* ob) {
+    auto store_tile = [&](int64_t tile, Origin org, const uint8_t* ob) {
         constexpr int OC = D / 32;   // 16-byte chunks per packed row
+        const int live = rows_in(tile);
+        const int64_t row0 = tile * C::TT;
         for (int c = tid; c < C::TT * OC; c += C::THREADS) {
             const int r = c / OC, q = c % OC;
-            const int64_t row = tile * C::TT + r;
-            if (row < M) {
+            if (r < live) {
                 const uint2v lo = *reinterpret_cast<const uint2v*>(&ob[r * C::OUT_STRIDE + q * 16]);
                 const uint2v hi = *reinterpret_cast<const uint2v*>(&ob[r * C::OUT_STRIDE + q * 16 + 8]);
                 uint4v v = {lo.x, lo.y, hi.x, hi.y};
                 if (PAGED) {
                     int head, is_v;
-                    uint8_t* dst = paged_row(row, head, is_v);
+                    uint8_t* dst = paged_row(org, r, head, is_v);
                     if (dst) {
                         dst += head * (D / 2) + 16 * q;
                         if (pd.wide) {
@@ -350,8 +443,10 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                             d4[0] = v.x; d4[1] = v.y; d4[2] = v.z; d4[3] = v.w;
                         }
                     }
+                } else if (pd.append_n == 0u) {          // uniform: chunk c of the tile is chunk c of its rows
+                    __builtin_nontemporal_store(v, reinterpret_cast<uint4v*>(packed + row0 * (D / 2)) + c);
                 } else {
-                    __builtin_nontemporal_store(v, reinterpret_cast<uint4v*>(packed + out_row(row) * (D / 2)) + q);
+                    __builtin_nontemporal_store(v, reinterpret_cast<uint4v*>(packed + appended_row(org, r) * (D / 2)) + q);
                 }
             }
         }
@@ -373,46 +468,50 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                             const float16v& acc_in, uint8_t* ob) {
                 const uint8_t* brow = &xs[mbuf][(32 * mtb + n32) * C::XS_STRIDE + kg * 16];
                 const float inv = inv_s[fbuf][32 * ftb + n32];
-                float16v acc = {};
-                uint32_t idx[16];
+                float16v acc;
                 uint2v cell[16];
                 float yv[16];
-                // element e: address and lookup at step e, compare at step e + 4
+                uint32_t word[2] = {0u, 0u};
+                // Step st looks up element ord(st) and compares the element of step st - 4.  The order
+                // is that of the nibbles of the two output words from the top down (byte j = idx[2j] <<
+                // 4 | idx[2j+1]), so that a word is built as word = (word << 4) + base + (thr < y):
+                // two instructions per element for index and packing.
+                auto ord = [](int st) { return 8 * (st >> 3) + (6 - 2 * ((st & 7) >> 1)) + (st & 1); };
+                constexpr int kSteps = 8 * NT > 20 ? 8 * NT : 20;
 #pragma unroll
-                for (int st = 0; st < 24; ++st) {
-                    {
-                        const int ks = st / 3, t = 2 - st % 3;
+                for (int st = 0; st < kSteps; ++st) {
+                    if (st < 8 * NT) {
+                        const int ks = st / NT, t = NT - 1 - st % NT;
                         const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
-                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc, 0, 0, 0);
+                        // (the first product starts from the constant 0, not from cleared registers)
+                        if (st == 0) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, float16v{}, 0, 0, 0);
+                        else acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc, 0, 0, 0);
                     }
                     if (st < 16) {
-                        yv[st] = acc_in[st] * inv;
-                        cell[st] = bucket_cell(table, yv[st], inv_w, offset, n32);
+                        yv[st] = acc_in[ord(st)] * inv;
+                        cell[st] = bucket_cell(yv[st], inv_w, offset, copy8);
                     }
                     if (st >= 4 && st < 20) {
                         const int e = st - 4;
-                        idx[e] = cell[e].y + (bits_to_float(cell[e].x) < yv[e] ? 1u : 0u);
+                        word[e >> 3] = (word[e >> 3] << 4) + cell[e].y + (bits_to_float(cell[e].x) < yv[e] ? 1u : 0u);
                     }
                 }
-                uint2v o;
-                o.x = (idx[0] << 4 | idx[1]) | (idx[2] << 4 | idx[3]) << 8 | (idx[4] << 4 | idx[5]) << 16 |
-                      (idx[6] << 4 | idx[7]) << 24;
-                o.y = (idx[8] << 4 | idx[9]) | (idx[10] << 4 | idx[11]) << 8 | (idx[12] << 4 | idx[13]) << 16 |
-                      (idx[14] << 4 | idx[15]) << 24;
+                const uint2v o = {word[0], word[1]};
                 *reinterpret_cast<uint2v*>(&ob[(32 * ftb + n32) * C::OUT_STRIDE + 16 * cb + 8 * kg]) = o;
                 acc_out = acc;
             };
 
+            Origin org = origin_of(blockIdx.x);
             issue_loads(tile);
-            stage(tile, 0);
+            stage(tile, org, 0);
             if (tile + G < num_tiles) issue_loads(tile + G);
             __syncthreads();
             float16v acc_a = {}, acc_b = {};
             {   // block (tile, 0): nothing to overlap with yet
                 const uint8_t* brow = &xs[0][n32 * C::XS_STRIDE + kg * 16];
 #pragma unroll
-                for (int st = 0; st < 24; ++st) {
-                    const int ks = st / 3, t = 2 - st % 3;
+                for (int st = 0; st < 8 * NT; ++st) {
+                    const int ks = st / NT, t = NT - 1 - st % NT;
                     const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
                     acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc_a, 0, 0, 0);
                 }
@@ -423,23 +522,26 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                 const bool has_next = next < num_tiles;
                 uint8_t* ob = outs + cur * kOutBytes;
                 pipe(cur, 1, acc_b, cur, 0, acc_a, ob);
+                const Origin next_org = advance(org);
                 if (has_next) {
-                    stage(next, cur ^ 1);
+                    stage(next, next_org, cur ^ 1);
                     if (next + G < num_tiles) issue_loads(next + G);
                 }
                 __syncthreads();                      // tile + 1 is staged
                 // past the last tile the matrix instructions run on stale rows and their result is dropped
                 pipe(cur ^ 1, 0, acc_a, cur, 1, acc_b, ob);
                 __syncthreads();                      // the packed rows of this tile are complete
-                store_tile(tile, ob);
+                store_tile(tile, org, ob);
+                org = next_org;
             }
             return;
         }
     }
 
+    Origin org = origin_of(blockIdx.x);
     if (tile < num_tiles) {
         issue_loads(tile);
-        stage(tile, 0);
+        stage(tile, org, 0);
     }
     __syncthreads();
 
@@ -455,7 +557,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             if constexpr (kBf16) {
                 // the small terms first, so that they are not rounded away against the large one
 #pragma unroll
-                for (int t = 2; t >= 0; --t)
+                for (int t = NT - 1; t >= 0; --t)
 #pragma unroll
                     for (int ks = 0; ks < C::NK; ++ks) {
                         const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
@@ -477,7 +579,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             uint32_t idx[16];
             if (!slow) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) idx[i] = bucket_fast(table, yv[i], inv_w, offset, n32);
+                for (int i = 0; i < 16; ++i) idx[i] = bucket_fast(yv[i], inv_w, offset, copy8);
             } else {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) idx[i] = bucket_slow(table, yv[i]);
@@ -491,10 +593,19 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
         }
         __syncthreads();
 
-        store_tile(tile, outs);
-        if (next < num_tiles) stage(next, cur ^ 1);
+        store_tile(tile, org, outs);
+        org = advance(org);
+        if (next < num_tiles) stage(next, org, cur ^ 1);
         __syncthreads();
     }
+}
+
+// bf16 terms of the matrix: three (exact) on request, and where the count does not matter (the
+// fp16 route: one instantiation)
+template <int D, int DT>
+int bf16_terms() {
+    if (DT != FQ_BF16 || D > 128) return 3;
+    return fq_host::option(FQ_OPT_COMPRESS_THREE_TERMS) != 0 ? 3 : 2;
 }
 
 template <int D, int DT>
@@ -504,8 +615,12 @@ int launch_compress(const void* x, const float* re, const float* ro, const float
     const int64_t tiles = (M + C::TT - 1) / C::TT;
     const int64_t cap = int64_t(num_cus) * 2;
     const unsigned grid = unsigned(tiles < cap ? tiles : cap);
-    hipLaunchKernelGGL((tq4_compress_kernel<D, DT, false>), dim3(grid), dim3(C::THREADS), 0, s,
-                       reinterpret_cast<const uint4v*>(x), re, ro, bnd, packed, norms, M, tiles, pd);
+    if (bf16_terms<D, DT>() == 3)
+        hipLaunchKernelGGL((tq4_compress_kernel<D, DT, false, 3>), dim3(grid), dim3(C::THREADS), 0, s,
+                           reinterpret_cast<const uint4v*>(x), re, ro, bnd, packed, norms, M, tiles, pd);
+    else
+        hipLaunchKernelGGL((tq4_compress_kernel<D, DT, false, 2>), dim3(grid), dim3(C::THREADS), 0, s,
+                           reinterpret_cast<const uint4v*>(x), re, ro, bnd, packed, norms, M, tiles, pd);
     return fq_host::check_launch();
 }
 
@@ -517,9 +632,14 @@ int launch_compress_store(const void* key, const float* re, const float* ro, con
     const int64_t tiles = (M + C::TT - 1) / C::TT;
     const int64_t cap = int64_t(num_cus) * 2;
     const unsigned grid = unsigned(tiles < cap ? tiles : cap);
-    hipLaunchKernelGGL((tq4_compress_kernel<D, DT, true>), dim3(grid), dim3(C::THREADS), 0, s,
-                       reinterpret_cast<const uint4v*>(key), re, ro, bnd, static_cast<uint8_t*>(nullptr),
-                       static_cast<float*>(nullptr), M, tiles, pd);
+    if (bf16_terms<D, DT>() == 3)
+        hipLaunchKernelGGL((tq4_compress_kernel<D, DT, true, 3>), dim3(grid), dim3(C::THREADS), 0, s,
+                           reinterpret_cast<const uint4v*>(key), re, ro, bnd, static_cast<uint8_t*>(nullptr),
+                           static_cast<float*>(nullptr), M, tiles, pd);
+    else
+        hipLaunchKernelGGL((tq4_compress_kernel<D, DT, true, 2>), dim3(grid), dim3(C::THREADS), 0, s,
+                           reinterpret_cast<const uint4v*>(key), re, ro, bnd, static_cast<uint8_t*>(nullptr),
+                           static_cast<float*>(nullptr), M, tiles, pd);
     return fq_host::check_launch();
 }
 
@@ -616,12 +736,14 @@ extern "C" int fq_tq4_compress_store(const void* key, const void* value, int x_d
     if (!fq_host::aligned(key, 16) || !fq_host::aligned(value, 16) || !fq_host::aligned(kv_cache, 16) ||
         !fq_host::aligned(slot_mapping, 8))
         return FQ_ERR_MISALIGNED;
-    if (num_tokens > 0x7fffffffLL || num_tokens * H_KV > (int64_t(1) << 40)) return FQ_ERR_BAD_SHAPE;
+    // the kernel counts tokens in 32 bits and divides by the head count in float32
+    if (num_tokens > 0x7fffffffLL || H_KV > 65536 || num_tokens * H_KV > (int64_t(1) << 40)) return FQ_ERR_BAD_SHAPE;
     PagedDest pd{};
     pd.x_value = static_cast<const uint4v*>(value);
     pd.cache = kv_cache;
     pd.slots = slot_mapping;
     pd.rows_k = num_tokens * H_KV;
+    pd.tokens = uint32_t(num_tokens);
     pd.num_slots = num_slots;
     pd.mapped = int(num_mapped);
     pd.H = H_KV;

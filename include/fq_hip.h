@@ -58,7 +58,11 @@ typedef enum fq_option {
     FQ_OPT_DECODE_TINY_SPIN = 3,  /* default 0: 1 makes the bounded waits between the wavefronts of the staged
                                      decode kernel give up after two polls, to exercise the failure path
                                      (NaN rows, fault counter) without hanging anything                */
-    FQ_OPTION_COUNT = 4
+    FQ_OPT_COMPRESS_THREE_TERMS = 4, /* FQ_COMPRESS_THREE_TERMS, default 0: bf16 rows of head_dim 64 / 128 are
+                                     rotated against the matrix as two bf16 terms (|error| <= 2^-18 per
+                                     element: about 6 indices in a million differ from the float32 result);
+                                     1: three terms, the float32 matrix exactly, at 3/2 of the matrix work */
+    FQ_OPTION_COUNT = 5
 } fq_option;
 int fq_get_option(int option);
 int fq_set_option(int option, int value);

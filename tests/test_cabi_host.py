@@ -239,7 +239,7 @@ def test_static_scratch_decode_refuses_before_touching_the_gpu(lib):
 
 def test_option_switches(lib):
     assert lib.fq_get_option(99) == -1 and lib.fq_set_option(99, 1) == FQ_SHAPE
-    for opt in range(4):
+    for opt in range(5):
         old = lib.fq_get_option(opt)
         assert old in (0, 1)
         assert lib.fq_set_option(opt, 1 - old) == FQ_OK and lib.fq_get_option(opt) == 1 - old

@@ -189,6 +189,31 @@ def test_compress_scales_and_adversarial_rows():
     assert torch.equal(packed.cpu(), want_p) and torch.equal(norms.cpu(), want_n)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+def test_compress_bf16_two_and_three_matrix_terms(d, kernel_option):
+    """bf16 rows are rotated against the matrix as two bf16 terms (default) or three (the float32
+    matrix exactly).  Measured on 2 M coordinates against the oracle: the two-term mode may move a few
+    indices in a million across a boundary (|y| error below 1e-6), the three-term mode is as close as
+    float32 summation order allows; both stay far inside the 1e-4 that is allowed."""
+    c, b, r = book(d)
+    x = outlier_rows(2048, 8, d, seed=77, dtype=torch.bfloat16)
+    idx_want, norms_want, y = O.compress_indices(x, r, b)
+    rates = {}
+    for three in (False, True):
+        kernel_option("compress_three_terms", three)
+        packed, norms = K.tq4_compress(x.to(DEV), r.to(DEV), b.to(DEV))
+        idx_got = O.nibble_unpack(packed.cpu())
+        bad = idx_got != idx_want
+        rates[three] = bad.float().mean().item()
+        if bad.any():
+            dist = (y[bad].unsqueeze(-1) - b).abs().min(dim=-1).values
+            assert dist.max() < 2e-6
+            assert (idx_got[bad].int() - idx_want[bad].int()).abs().max() == 1
+        assert torch.equal(norms.cpu(), norms_want) or ((norms.cpu() - norms_want).abs() / norms_want).max() < 2e-6
+    assert rates[False] <= 3e-5, rates
+    assert rates[True] <= 5e-6, rates
+
+
 def test_compress_out_buffers_and_presplit_rotation():
     c, b, r = book(128)
     x = outlier_rows(33, 8, 128, seed=9, dtype=torch.bfloat16)
