@@ -35,7 +35,7 @@ H_Q, H_KV, D, BS = 32, 8, 128, 16
 BATCH, CTX = 32, 4096
 EXTRA_ITERS = 20              # timed calls of every leg other than the headline
 ROW_BYTES = H_KV * (D + 8)
-DOMINANT_KERNEL = "paged_decode_staged_kernel<4,4,bf16,4,false,4>"
+DOMINANT_KERNEL = "paged_decode_staged_kernel<4,4,bf16,4,false,4,false>"
 
 
 def log(*a):
@@ -133,6 +133,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="omit the compress / decompress legs")
+    ap.add_argument("--skip-other-shapes", action="store_true",
+                    help="omit the legs on shapes that are not BASELINE configs (profiles of the configs alone)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain device copy of one cache (142.6 MB read + 142.6 MB written): the "
                          "reference point for scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run")
@@ -504,25 +506,26 @@ def main():
             return ms, 4.0 * n * n * d * b * hq / 2
 
         shapes = {}
-        for name, (n_seq, ctx, hq, hkv, d) in {
+        for name, (n_seq, ctx, hq, hkv, d) in ({} if args.skip_other_shapes else {
             "decode_32x16384_32q_8kv_d128": (32, 16384, 32, 8, 128),
             "decode_32x4096_32q_4kv_d128": (32, 4096, 32, 4, 128),
             "decode_32x4096_32q_8kv_d64": (32, 4096, 32, 8, 64),
             "decode_32x4096_32q_8kv_d256": (32, 4096, 32, 8, 256),
-        }.items():
+        }).items():
             ms, nbytes = decode_shape(n_seq, ctx, hq, hkv, d)
             shapes[name] = {"step_us": ms * 1e3, "gbps": nbytes / (ms * 1e-3) / 1e9,
                             "pct_hbm_peak": 100.0 * nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
             torch.cuda.empty_cache()
-        for name, (b, n, hq, hkv, d) in {
+        for name, (b, n, hq, hkv, d) in ({} if args.skip_other_shapes else {
             "prefill_2x8192_32q_8kv_d64": (2, 8192, 32, 8, 64),
             "prefill_2x8192_16q_4kv_d256": (2, 8192, 16, 4, 256),
-        }.items():
+        }).items():
             ms, flops = prefill_shape(b, n, hq, hkv, d)
             shapes[name] = {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12,
                             "pct_fp16_mfma_peak": 100.0 * flops / (ms * 1e-3) / 2.5e15}
             torch.cuda.empty_cache()
-        extra["other_shapes"] = shapes
+        if shapes:
+            extra["other_shapes"] = shapes
 
     value = kv_bytes / (step_ms * 1e-3) / 1e9
     line = {
