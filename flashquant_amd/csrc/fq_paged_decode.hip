@@ -86,6 +86,7 @@ struct DecodeParams {
     int num_splits;
     int two_tables;             // centroids_v differs from centroids_k
     float scale_log2e;          // sm_scale * log2(e)
+    int heads_per_wg;           // direct kernel: KV heads a workgroup serves; its other wavefronts take further splits
     int spin_limit;             // staged kernel: polls of a bounded wait between wavefronts before it gives up
     int balance_slots;          // staged kernel: > 0 lets the workgroups size the token chunks from the actual
                                 // sequence lengths, for this many workgroups running at a time (num_seqs <= 64)
@@ -115,15 +116,18 @@ __global__ __launch_bounds__(D == 256 ? 256 : 512) void paged_decode_kernel(cons
     const int g = lane >> 4;
     const int hd = n % GP;                // query head inside the group
     const int bc_lane = n / GP;           // block class kept by this lane
-    const int split = blockIdx.x;
+    // Fewer KV heads than wavefronts: the workgroup serves all heads of waves / heads_per_wg consecutive
+    // splits (a workgroup of one or two wavefronts would leave the CU, which holds two such workgroups
+    // beside their 64 KB tables, almost empty).
+    const int split = int(blockIdx.x) * (waves / p.heads_per_wg) + wave / p.heads_per_wg;
     const int seq = blockIdx.y;
-    const int h = blockIdx.z * waves + wave;
+    const int h = blockIdx.z * p.heads_per_wg + wave % p.heads_per_wg;
 
     // ---- byte -> (fp16, fp16) tables, one copy per LDS bank ----------------------
     build_byte_table(lut, p.centroids_k, wave, waves, lane);
     if (p.two_tables) build_byte_table(lut2, p.centroids_v, wave, waves, lane);
     __syncthreads();
-    if (h >= p.H_KV) return;
+    if (h >= p.H_KV || split >= p.num_splits) return;
     const uint8_t* lut_k = reinterpret_cast<const uint8_t*>(lut);
     const uint8_t* lut_v = p.two_tables ? reinterpret_cast<const uint8_t*>(lut2) : lut_k;
     const uint32_t lane_off = 4u * lane;
@@ -1793,12 +1797,20 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
     }
 
     const int max_waves = D == 256 ? 4 : 8;
-    const int waves = p.H_KV < max_waves ? p.H_KV : max_waves;
-    const dim3 grid(p.num_splits, S, (p.H_KV + waves - 1) / waves), block(64 * waves);
+    // 1 or 2 KV heads: a full workgroup, its wavefronts beyond the heads on the next splits (measured on 8 x 32768
+    // tokens with 2 KV heads: 71 -> 57 us; with 4 heads on 8-token pages, the one case that reaches this kernel, it
+    // was slower)
+    const bool pack_splits = p.H_KV <= 2 && p.num_splits > 1;
+    const int waves = pack_splits ? max_waves : (p.H_KV < max_waves ? p.H_KV : max_waves);
+    DecodeParams pk = p;
+    pk.heads_per_wg = pack_splits ? p.H_KV : waves;
+    const int splits_per_wg = waves / pk.heads_per_wg;
+    const dim3 grid((p.num_splits + splits_per_wg - 1) / splits_per_wg, S, (p.H_KV + pk.heads_per_wg - 1) / pk.heads_per_wg),
+        block(64 * waves);
     const size_t lds = p.two_tables ? size_t(kLutWords) * sizeof(uint32_t) : 0;   // the K table is static
 #define FQ_DECODE_GP(BSL, GPV)                                                                  \
-    return wide ? launch_with_lds(paged_decode_kernel<D, BSL, GPV, DT, 4>, p, grid, block, lds, stream) \
-                : launch_with_lds(paged_decode_kernel<D, BSL, GPV, DT, 1>, p, grid, block, lds, stream)
+    return wide ? launch_with_lds(paged_decode_kernel<D, BSL, GPV, DT, 4>, pk, grid, block, lds, stream) \
+                : launch_with_lds(paged_decode_kernel<D, BSL, GPV, DT, 1>, pk, grid, block, lds, stream)
 #define FQ_DECODE_BS(BSL)                             \
     do {                                              \
         if (p.G <= 4) { FQ_DECODE_GP(BSL, 4); }       \
@@ -1975,6 +1987,7 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
     p.two_tables = centroids_k != centroids_v ? 1 : 0;
     p.scale_log2e = sm_scale * kLog2e;
     p.balance_slots = 0;
+    p.heads_per_wg = 0;
     p.spin_limit = fq_host::option(FQ_OPT_DECODE_TINY_SPIN) != 0 ? 2 : (1 << 20);
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define FQ_DECODE_D(DD)                                                                 \

@@ -369,6 +369,16 @@ def test_paged_decode_four_kv_heads_ragged_long_contexts():
     _decode_case(lens, hq=16, hkv=4, num_splits=0, bs=8)          # pages of 8 tokens: the direct kernel
 
 
+@pytest.mark.parametrize("hkv,d,splits", [(1, 128, 0), (1, 128, 5), (2, 128, 3), (2, 64, 8), (1, 256, 6), (2, 256, 4),
+                                          (1, 128, 40)])
+def test_paged_decode_one_or_two_kv_heads_share_a_workgroup_over_splits(hkv, d, splits):
+    """With 1 or 2 KV heads the wavefronts of a workgroup beyond the heads take the following splits (odd
+    split counts leave some of them without work, ragged lengths leave others with an empty split)."""
+    lens = [70, 0, 700, 16, 129, 1, 333, 64]
+    _decode_case(lens, hq=4 * hkv, hkv=hkv, d=d, bs=16, num_splits=splits, seed=47)
+    _decode_case(lens, hq=hkv, hkv=hkv, d=d, bs=32, num_splits=splits, seed=48, dtype=torch.float16)
+
+
 def test_paged_decode_rotated_space_and_out_argument():
     c, b, r = book(128)
     q, cache, table, sl = build_paged_case([90, 10], 8, 2)
