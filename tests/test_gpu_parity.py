@@ -687,7 +687,8 @@ def test_paged_prefill_rejects_bad_arguments():
 # ---- fused compress-and-store into the paged cache -----------------------------------
 
 @pytest.mark.parametrize("h,d,dtype", [(8, 128, torch.bfloat16), (8, 128, torch.float16), (1, 64, torch.bfloat16),
-                                       (3, 256, torch.float16), (2, 128, torch.bfloat16)])
+                                       (3, 256, torch.float16), (2, 128, torch.bfloat16), (7, 128, torch.bfloat16),
+                                       (40, 64, torch.float16), (5, 128, torch.float16)])
 def test_compress_and_store_matches_compress_then_scatter(h, d, dtype):
     c, bnd, r = book(d)
     n, bs, nb = 203, 16, 20

@@ -74,6 +74,33 @@ def test_append_in_place_equals_compress_then_append(d, dtype):
     assert idx.shape == (B, H, 169, d // 2) and nrm.shape == (B, H, 169, 1)
 
 
+def test_append_of_more_than_a_million_tokens_at_once():
+    """A long prompt appended in one call: with 2^20 tokens or more per (batch, head) pair the kernel
+    finds the pair of a row by comparison instead of by the float32 quotient.  Bit-equal to the plain
+    compress of the same rows, in place at the position, everything else untouched."""
+    d, dtype = 64, torch.bfloat16
+    c, bnd, r = book(d)
+    B, H, n = 1, 2, (1 << 20) + 37
+    cap = n + 5
+    C = load_native()
+    ev, od = C.split_rotation(r)
+    ev, od, bd = ev.to(DEV), od.to(DEV), bnd.to(DEV)
+    buf = CompressedBuffer(cap, B, H, d // 2, device=torch.device(DEV))
+    buf._indices.fill_(0xAB)
+    buf._norms.fill_(-7.0)
+    first = outlier_rows(B * H * 3, 1, d, 400, dtype=dtype).reshape(B, H, 3, d).to(DEV)
+    buf.append_from(first, ev, od, bd)
+    g = torch.Generator(device=DEV).manual_seed(401)
+    x = torch.randn(B, H, n, d, generator=g, device=DEV).to(dtype)
+    buf.append_from(x, ev, od, bd)
+    p, nrm = K.tq4_compress(x.reshape(B * H * n, 1, d), r.to(DEV), bd)
+    assert torch.equal(buf._indices[:, :, 3:3 + n], p.reshape(B, H, n, d // 2))
+    assert torch.equal(buf._norms[:, :, 3:3 + n], nrm.reshape(B, H, n, 1))
+    assert (buf._indices[:, :, 3 + n:] == 0xAB).all() and (buf._norms[:, :, 3 + n:] == -7.0).all()
+    p0, n0 = K.tq4_compress(first.reshape(B * H * 3, 1, d), r.to(DEV), bd)
+    assert torch.equal(buf._indices[:, :, :3], p0.reshape(B, H, 3, d // 2))
+
+
 def test_append_then_attend_matches_the_oracle():
     """A cache step of the fused mode: prefill 150 tokens, then three decode steps of one token
     each, attention over the growing buffers read in place."""
