@@ -186,7 +186,7 @@ struct PagedDest {
     int64_t append_cap, append_pos;
 };
 
-// NT: bf16 terms of the rotation matrix for bf16 rows of head_dim <= 128 (ignored otherwise).
+// NT: bf16 terms of the rotation matrix for bf16 rows (ignored for fp16 rows; three at head_dim 256 means the fp16 route).
 // 3: R = t0 + t1 + t2 exactly.  2: t0, t1 rounded to nearest, |R - t0 - t1| <= 2^-18 |R|: the rotated
 // coordinates move by about 2e-7 (standard deviation, unit rows of 128 coordinates), which puts about 6
 // indices in a million on the other side of a bucket boundary, for two thirds of the matrix instructions.
@@ -244,8 +244,8 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
         locate(o, i, outer, t);
         return int64_t(outer) * pd.append_cap + pd.append_pos + int64_t(t);
     };
-    // bf16 rows of head_dim 128 run a software pipeline (see below) with two packed-row buffers
-    constexpr bool kPipe = DT == FQ_BF16 && D == 128;
+    // head_dim 128 runs a software pipeline (see below) with two packed-row buffers
+    constexpr bool kPipe = D == 128;
     constexpr int kOutBytes = C::TT * C::OUT_STRIDE;
     // one LDS block, the bucket table first (its lookups address it from LDS address 0)
     struct Lds {
@@ -272,8 +272,8 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     // fp16 rows: R = hi + lo / 4096 in fp16.  bf16 rows go to the bf16 MFMA as they are, against
     // R = t0 + t1 (+ t2) in bf16 (3 x 8 bits: the float32 value exactly); bf16 terms keep the
     // float32 exponent range, so the products share one accumulator.
-    // (head_dim 256 would need 192 registers for three terms: it keeps the fp16 route)
-    constexpr bool kBf16 = DT == FQ_BF16 && D <= 128;
+    // (head_dim 256 would need 192 registers for three terms: with three it takes the fp16 route)
+    constexpr bool kBf16 = DT == FQ_BF16 && (D <= 128 || NT == 2);
     static_assert(NT == 2 || NT == 3, "two or three bf16 terms");
     half8 a_hi[kBf16 ? 1 : C::NK], a_lo[kBf16 ? 1 : C::NK];
     bf16x8 a_t[kBf16 ? NT : 1][kBf16 ? C::NK : 1];
@@ -454,7 +454,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
 
     int64_t tile = blockIdx.x;
 
-    // ---- software pipeline (bf16, head_dim 128) ------------------------------------------------
+    // ---- software pipeline (head_dim 128) -------------------------------------------------------
     // The unit of work is a block of 32 rows.  The matrix instructions of block u + 1 are issued
     // between the lookups and compares that bucketize block u, so that a wavefront keeps both the
     // matrix pipe and the vector ALU busy instead of alternating between them (two wavefronts
@@ -477,15 +477,23 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                 // 4 | idx[2j+1]), so that a word is built as word = (word << 4) + base + (thr < y):
                 // two instructions per element for index and packing.
                 auto ord = [](int st) { return 8 * (st >> 3) + (6 - 2 * ((st & 7) >> 1)) + (st & 1); };
-                constexpr int kSteps = 8 * NT > 20 ? 8 * NT : 20;
+                constexpr int kTerms = kBf16 ? NT : 2;           // fp16 rows: hi and lo, an accumulator each
+                constexpr int kSteps = 8 * kTerms > 20 ? 8 * kTerms : 20;
+                float16v acc_lo;
 #pragma unroll
                 for (int st = 0; st < kSteps; ++st) {
-                    if (st < 8 * NT) {
-                        const int ks = st / NT, t = NT - 1 - st % NT;
-                        const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
+                    if (st < 8 * kTerms) {
+                        const int ks = st / kTerms, t = kTerms - 1 - st % kTerms;
                         // (the first product starts from the constant 0, not from cleared registers)
-                        if (st == 0) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, float16v{}, 0, 0, 0);
-                        else acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc, 0, 0, 0);
+                        if constexpr (kBf16) {
+                            const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
+                            if (st == 0) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, float16v{}, 0, 0, 0);
+                            else acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc, 0, 0, 0);
+                        } else {
+                            const half8 b = *reinterpret_cast<const half8*>(brow + ks * 32);
+                            if (t == 1) acc_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_lo[ks], b, ks == 0 ? float16v{} : acc_lo, 0, 0, 0);
+                            else acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[ks], b, ks == 0 ? float16v{} : acc, 0, 0, 0);
+                        }
                     }
                     if (st < 16) {
                         yv[st] = acc_in[ord(st)] * inv;
@@ -498,7 +506,12 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                 }
                 const uint2v o = {word[0], word[1]};
                 *reinterpret_cast<uint2v*>(&ob[(32 * ftb + n32) * C::OUT_STRIDE + 16 * cb + 8 * kg]) = o;
-                acc_out = acc;
+                if constexpr (kBf16) {
+                    acc_out = acc;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc_out[i] = __builtin_fmaf(acc_lo[i], kLoScale, acc[i]);
+                }
             };
 
             Origin org = origin_of(blockIdx.x);
@@ -509,11 +522,23 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             float16v acc_a = {}, acc_b = {};
             {   // block (tile, 0): nothing to overlap with yet
                 const uint8_t* brow = &xs[0][n32 * C::XS_STRIDE + kg * 16];
+                if constexpr (kBf16) {
 #pragma unroll
-                for (int st = 0; st < 8 * NT; ++st) {
-                    const int ks = st / NT, t = NT - 1 - st % NT;
-                    const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
-                    acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc_a, 0, 0, 0);
+                    for (int st = 0; st < 8 * NT; ++st) {
+                        const int ks = st / NT, t = NT - 1 - st % NT;
+                        const bf16x8 b = *reinterpret_cast<const bf16x8*>(brow + ks * 32);
+                        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_t[t][ks], b, acc_a, 0, 0, 0);
+                    }
+                } else {
+                    float16v lo = {};
+#pragma unroll
+                    for (int ks = 0; ks < C::NK; ++ks) {
+                        const half8 b = *reinterpret_cast<const half8*>(brow + ks * 32);
+                        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_hi[ks], b, acc_a, 0, 0, 0);
+                        lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_lo[ks], b, lo, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc_a[i] = __builtin_fmaf(lo[i], kLoScale, acc_a[i]);
                 }
             }
             for (int it = 0; tile < num_tiles; tile += G, ++it) {
@@ -604,7 +629,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
 // fp16 route: one instantiation)
 template <int D, int DT>
 int bf16_terms() {
-    if (DT != FQ_BF16 || D > 128) return 3;
+    if (DT != FQ_BF16) return 3;
     return fq_host::option(FQ_OPT_COMPRESS_THREE_TERMS) != 0 ? 3 : 2;
 }
 

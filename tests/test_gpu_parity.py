@@ -189,7 +189,7 @@ def test_compress_scales_and_adversarial_rows():
     assert torch.equal(packed.cpu(), want_p) and torch.equal(norms.cpu(), want_n)
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, 256])
 def test_compress_bf16_two_and_three_matrix_terms(d, kernel_option):
     """bf16 rows are rotated against the matrix as two bf16 terms (default) or three (the float32
     matrix exactly).  Measured on 2 M coordinates against the oracle: the two-term mode may move a few
