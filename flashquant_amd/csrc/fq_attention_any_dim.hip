@@ -53,7 +53,7 @@ struct AnyDimCfg {
 };
 
 template <int D, int DT, bool PAGED>
-__global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimParams p) {
+__global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyDimParams p) {
     using C = AnyDimCfg<D>;
     constexpr int NJ = D / 32;          // k-steps of the score product
     constexpr int NCB = D / 16;         // 16-coordinate output blocks
@@ -224,17 +224,31 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
                 const _Float16 hn = _Float16(nk[u]);
                 const half2v n2 = {hn, hn};
                 uint32_t* dst = reinterpret_cast<uint32_t*>(ks + (2 * tp + u) * C::KSTRIDE + 2 * BPT * part);
+                uint32_t wd[BPT];
 #pragma unroll
                 for (int j = 0; j < BPT; ++j) {
                     const uint32_t byte = (kw[u][j >> 2] >> (8 * (j & 3))) & 0xffu;
                     const half2v c2 = __builtin_bit_cast(half2v, pair_k[byte]) * n2;
-                    dst[j] = __builtin_bit_cast(uint32_t, c2);
+                    wd[j] = __builtin_bit_cast(uint32_t, c2);
+                }
+                // the thread's run of the row in 8- or 16-byte stores (single dwords from 64 lanes that lie 16
+                // to 32 bytes apart fall into a few banks)
+                if constexpr (BPT == 2) {
+                    *reinterpret_cast<uint2v*>(dst) = uint2v{wd[0], wd[1]};
+                } else {
+#pragma unroll
+                    for (int j = 0; j < BPT; j += 4) *reinterpret_cast<uint4v*>(dst + j) = uint4v{wd[j], wd[j + 1], wd[j + 2], wd[j + 3]};
                 }
             }
             // V, transposed: a 2 x 2 nibble transpose makes a byte hold one coordinate of the two tokens,
             // so one lookup yields the dword (token 2 tp, token 2 tp + 1) of a coordinate row
             {
                 const half2v n2 = {_Float16(nv[0]), _Float16(nv[1])};
+                // The rows of the 16 threads of a token pair lie 2 BPT rows apart, a multiple of 64 banks at 256
+                // coordinates: with the pair's own column every one of their stores would hit the same bank.
+                // The groups of four columns (8 tokens, what an operand read takes) are rotated by the thread's
+                // index, so that the 64 lanes of a store spread over 16 banks (the 16 columns of a row).
+                const int vcol = (tp + 4 * part) & 15;
 #pragma unroll
                 for (int c = 0; c < (BPT + 3) / 4; ++c) {
                     const uint32_t X = (vw[0][c] & 0xF0F0F0F0u) | ((vw[1][c] >> 4) & 0x0F0F0F0Fu);   // even coordinates
@@ -244,8 +258,8 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
                         const int d = 2 * (BPT * part + 4 * c + j);
                         const half2v xe = __builtin_bit_cast(half2v, pair_v[(X >> (8 * j)) & 0xffu]) * n2;
                         const half2v yo = __builtin_bit_cast(half2v, pair_v[(Y >> (8 * j)) & 0xffu]) * n2;
-                        *reinterpret_cast<uint32_t*>(vt + d * C::VSTRIDE + 2 * tp) = __builtin_bit_cast(uint32_t, xe);
-                        *reinterpret_cast<uint32_t*>(vt + (d + 1) * C::VSTRIDE + 2 * tp) = __builtin_bit_cast(uint32_t, yo);
+                        *reinterpret_cast<uint32_t*>(vt + d * C::VSTRIDE + 2 * vcol) = __builtin_bit_cast(uint32_t, xe);
+                        *reinterpret_cast<uint32_t*>(vt + (d + 1) * C::VSTRIDE + 2 * vcol) = __builtin_bit_cast(uint32_t, yo);
                     }
                 }
             }
@@ -266,6 +280,8 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
         }
         // lane (n16, g4): rows 4 g4 + i, tokens t0 + n16 and t0 + 16 + n16
         float pv[2][4];
+        float alphas[4];
+        bool moved = false;
         const int kx[2] = {k_exc[n16], k_exc[16 + n16]}, vx[2] = {v_exc[n16], v_exc[16 + n16]};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -292,8 +308,15 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
                 rs += pv[tb][i];
             }
             l_run[i] = __builtin_fmaf(l_run[i], alpha, rs);     // per-lane partial; summed over the row at the end
+            alphas[i] = alpha;
+            moved = moved || alpha != 1.0f;
+        }
+        // the accumulators are rescaled only when some row's maximum moved (after the first tiles it rarely does)
+        if (__any(moved)) {
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) O[cb][i] *= alpha;
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) O[cb][i] *= alphas[i];
         }
         // P (C layout) -> LDS patch -> A layout
 #pragma unroll
@@ -304,7 +327,9 @@ __global__ __launch_bounds__(256) void tq_attention_any_dim_kernel(const AnyDimP
         const half8 pa = *reinterpret_cast<const half8*>(pw + n16 * C::VSTRIDE + 8 * g4);
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
-            const half8 vb = *reinterpret_cast<const half8*>(vt + (16 * cb + n16) * C::VSTRIDE + 8 * g4);
+            // (the column groups of a row are rotated by the index of the thread that wrote it: row / (2 BPT))
+            const int vrow = 16 * cb + n16;
+            const half8 vb = *reinterpret_cast<const half8*>(vt + vrow * C::VSTRIDE + 8 * ((g4 + vrow / (2 * BPT)) & 3));
             O[cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, O[cb], 0, 0, 0);
         }
         __syncthreads();                               // the tiles are free again
