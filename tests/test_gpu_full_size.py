@@ -73,6 +73,36 @@ def test_paged_decode_at_the_benchmark_size():
     assert rel <= 2e-2, f"max error {rel} of the row magnitude"
 
 
+def test_paged_decode_of_four_kv_heads_on_long_ragged_contexts():
+    """4 KV heads (rows of two tokens in the staged kernel) at contexts of thousands of tokens, odd and
+    even lengths, the library's own split count: against the oracle, and the direct kernel agrees."""
+    c, b, r = book(128)
+    lens, hq, hkv, bs = [4096, 4095, 2049, 1, 3001, 0, 4033, 640], 16, 4, 16
+
+    def rows(s, n):
+        return outlier_rows(n, hkv, 128, 6000 + 2 * s), outlier_rows(n, hkv, 128, 6001 + 2 * s)
+
+    cache, table, sl = _store_sequences(lens, rows, hkv, 128, bs, seed=2102, extra_blocks=5)
+    q = torch.randn(len(lens), hq, 128, generator=torch.Generator().manual_seed(1102)).to(torch.bfloat16)
+    want = O.split_k_paged_decode(q, cache, table, sl, c, c, r, hkv, 128, bs)
+    cd = c.to(DEV)
+    args = (q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), cd, cd, r.to(DEV), hkv, 128, bs)
+    got = K.split_k_paged_decode(*args)
+    from flashquant_amd import load_native
+    C = load_native()
+    old = C.set_option("decode_direct", True)
+    try:
+        direct = K.split_k_paged_decode(*args)
+    finally:
+        C.set_option("decode_direct", old)
+    assert torch.isfinite(got).all()
+    row_scale = want.float().abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+    for out in (got, direct):
+        rel = ((out.cpu().float() - want.float()).abs() / row_scale).max().item()
+        assert rel <= 2e-2, f"max error {rel} of the row magnitude"
+    assert (got[5] == 0).all()          # the empty sequence
+
+
 # ---- the benchmark's prefill workload on slices -------------------------------------------------
 
 def test_fused_prefill_at_the_benchmark_size():
