@@ -268,6 +268,42 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     const int cb = wave % C::CB;
     const int tb0 = wave / C::CB;
 
+    // ---- staging helpers -----------------------------------------------------
+    const int chunk = tid % C::CPR;
+    const int row_in_pass = tid / C::CPR;
+    uint4v pre[C::PASSES];
+
+    // Everything that depends on the tile alone is wave-uniform (scalar registers); a thread adds
+    // 32-bit offsets to it.  rows_in(tile): rows of the tile that exist (0..TT).
+    auto rows_in = [&](int64_t tile) -> int {
+        const int64_t left = M - tile * C::TT;
+        return left >= C::TT ? C::TT : (left > 0 ? int(left) : 0);
+    };
+    auto issue_loads = [&](int64_t tile) {
+        const int64_t row0 = tile * C::TT;
+        const int live = rows_in(tile);
+        const uint4v* base = x + row0 * C::CPR;
+        // paged mode: rows [rows_k, 2 rows_k) come from the value tensor; a tile may hold rows of both
+        int first_v = C::TT;
+        const uint4v* base_v = base;
+        if (PAGED) {
+            const int64_t k_left = pd.rows_k - row0;
+            first_v = k_left >= C::TT ? C::TT : (k_left > 0 ? int(k_left) : 0);
+            base_v = reinterpret_cast<const uint4v*>(reinterpret_cast<uintptr_t>(pd.x_value) +
+                                                     uintptr_t((row0 - pd.rows_k) * C::CPR * int64_t(sizeof(uint4v))));
+        }
+#pragma unroll
+        for (int p = 0; p < C::PASSES; ++p) {
+            const int r = p * C::ROWS_PER_PASS + row_in_pass;
+            const int off = p * C::ROWS_PER_PASS * C::CPR + tid;           // r * CPR + chunk
+            const uint4v* src = (PAGED && r >= first_v) ? base_v : base;
+            pre[p] = r < live ? __builtin_nontemporal_load(src + off) : uint4v{0, 0, 0, 0};
+        }
+    };
+    // the rows of the first tile are asked for before anything else: they arrive while the matrix rows are
+    // fetched and the bucket table is built (a small call is all prologue)
+    if (int64_t(blockIdx.x) < num_tiles) issue_loads(blockIdx.x);
+
     // ---- the rotation rows of this wave, split into two fp16 terms ----------
     // fp16 rows: R = hi + lo / 4096 in fp16.  bf16 rows go to the bf16 MFMA as they are, against
     // R = t0 + t1 (+ t2) in bf16 (3 x 8 bits: the float32 value exactly); bf16 terms keep the
@@ -309,38 +345,6 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     const bool slow = table.slow != 0;
     const uint32_t copy8 = 8u * uint32_t(n32);
 
-    // ---- staging helpers -----------------------------------------------------
-    const int chunk = tid % C::CPR;
-    const int row_in_pass = tid / C::CPR;
-    uint4v pre[C::PASSES];
-
-    // Everything that depends on the tile alone is wave-uniform (scalar registers); a thread adds
-    // 32-bit offsets to it.  rows_in(tile): rows of the tile that exist (0..TT).
-    auto rows_in = [&](int64_t tile) -> int {
-        const int64_t left = M - tile * C::TT;
-        return left >= C::TT ? C::TT : (left > 0 ? int(left) : 0);
-    };
-    auto issue_loads = [&](int64_t tile) {
-        const int64_t row0 = tile * C::TT;
-        const int live = rows_in(tile);
-        const uint4v* base = x + row0 * C::CPR;
-        // paged mode: rows [rows_k, 2 rows_k) come from the value tensor; a tile may hold rows of both
-        int first_v = C::TT;
-        const uint4v* base_v = base;
-        if (PAGED) {
-            const int64_t k_left = pd.rows_k - row0;
-            first_v = k_left >= C::TT ? C::TT : (k_left > 0 ? int(k_left) : 0);
-            base_v = reinterpret_cast<const uint4v*>(reinterpret_cast<uintptr_t>(pd.x_value) +
-                                                     uintptr_t((row0 - pd.rows_k) * C::CPR * int64_t(sizeof(uint4v))));
-        }
-#pragma unroll
-        for (int p = 0; p < C::PASSES; ++p) {
-            const int r = p * C::ROWS_PER_PASS + row_in_pass;
-            const int off = p * C::ROWS_PER_PASS * C::CPR + tid;           // r * CPR + chunk
-            const uint4v* src = (PAGED && r >= first_v) ? base_v : base;
-            pre[p] = r < live ? __builtin_nontemporal_load(src + off) : uint4v{0, 0, 0, 0};
-        }
-    };
     auto stage = [&](int64_t tile, Origin org, int buf) {
         const int live = rows_in(tile);
         const int64_t row0 = tile * C::TT;
@@ -515,8 +519,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             };
 
             Origin org = origin_of(blockIdx.x);
-            issue_loads(tile);
-            stage(tile, org, 0);
+            stage(tile, org, 0);                   // its loads were issued at the top of the kernel
             if (tile + G < num_tiles) issue_loads(tile + G);
             __syncthreads();
             float16v acc_a = {}, acc_b = {};
@@ -564,10 +567,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     }
 
     Origin org = origin_of(blockIdx.x);
-    if (tile < num_tiles) {
-        issue_loads(tile);
-        stage(tile, org, 0);
-    }
+    if (tile < num_tiles) stage(tile, org, 0);     // its loads were issued at the top of the kernel
     __syncthreads();
 
     for (int it = 0; tile < num_tiles; tile += gridDim.x, ++it) {
