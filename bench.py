@@ -282,6 +282,25 @@ def main():
 
     # ---- standalone compress / decompress (configs[1]) -----------------------------------
     if not args.skip_extra:
+        # a serving decode step as the attention implementation runs it (src/flashquant/vllm/impl.py:220-263,
+        # 362-394): the new token's K and V of every sequence are compressed into their cache rows, then the
+        # decode runs over the context (here the new token takes the last position of the same contexts)
+        ev_s, od_s = C.split_rotation(rot)
+        ev_s, od_s = ev_s.to(dev), od_s.to(dev)
+        k_new = torch.randn(BATCH, H_KV, D, device=dev).to(torch.bfloat16)
+        v_new = torch.randn(BATCH, H_KV, D, device=dev).to(torch.bfloat16)
+        last_slots = [(t.long()[:, (CTX - 1) // BS] * BS + (CTX - 1) % BS).contiguous() for _, t in caches]
+
+        def serving_step(i):
+            cache, table = caches[i % n_caches]
+            K.tq4_compress_and_store(k_new, v_new, rot_d, book[1], cache, last_slots[i % n_caches],
+                                     rotation_T_even=ev_s, rotation_T_odd=od_s)
+            K.split_k_paged_decode(q, cache, table, lens, cent_d, cent_d, rot_d, H_KV, D, BS, sm_scale=scale, out=out)
+
+        for i in range(args.warmup):
+            serving_step(i)
+        serve_ms, _ = time_events(serving_step, args.steps)
+        extra.update({"serving_step_us_cold": serve_ms * 1e3, "serving_tokens_per_s": BATCH / (serve_ms * 1e-3)})
         del caches
         torch.cuda.empty_cache()
         rows_tok = 32 * 65536
