@@ -313,16 +313,24 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     static_assert(NT == 2 || NT == 3, "two or three bf16 terms");
     half8 a_hi[kBf16 ? 1 : C::NK], a_lo[kBf16 ? 1 : C::NK];
     bf16x8 a_t[kBf16 ? NT : 1][kBf16 ? C::NK : 1];
+    // the matrix rows are asked for, the bucket table is built while they arrive, then they are split
+    float rr[C::NK][8];
     {
         const int j = 32 * cb + mfma_row_to_coord(n32);
         const float* src = (j & 1) ? rot_T_odd : rot_T_even;
         const int col = j >> 1;
 #pragma unroll
+        for (int ks = 0; ks < C::NK; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) rr[ks][e] = src[(16 * ks + 8 * kg + e) * (D / 2) + col];
+    }
+    build_bucket_table(table, boundaries, tid, C::THREADS);
+    {
+#pragma unroll
         for (int ks = 0; ks < C::NK; ++ks) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const int k = 16 * ks + 8 * kg + e;
-                const float r = src[k * (D / 2) + col];
+                const float r = rr[ks][e];
                 if constexpr (kBf16 && NT == 3) {
                     const __bf16 t0 = bf16_trunc(r);
                     const float r1 = r - bf16_value(t0);
@@ -340,7 +348,6 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             }
         }
     }
-    build_bucket_table(table, boundaries, tid, C::THREADS);
     const float inv_w = table.inv_w, offset = table.offset;
     const bool slow = table.slow != 0;
     const uint32_t copy8 = 8u * uint32_t(n32);
