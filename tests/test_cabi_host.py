@@ -112,6 +112,9 @@ def test_split_count_rules(lib):
     assert lib.fq_paged_decode_auto_splits(32, 1, 16, 256) <= 16
     assert lib.fq_paged_decode_auto_splits(32, 2, 16, 256) <= 16
     assert lib.fq_paged_decode_auto_splits(4, 4, 16, 2048) >= 32      # long contexts still fill the chip
+    # one long sequence: no more splits than the combine step takes in two passes
+    assert lib.fq_paged_decode_auto_splits(1, 8, 16, 2048) == 128
+    assert lib.fq_paged_decode_auto_splits(1, 8, 16, 16384) == 128    # 256K tokens: the minimum is 64
     f = lib.fq_paged_tq4_decode
     f.argtypes = ([ctypes.c_void_p] * 2 + [ctypes.c_int] + [ctypes.c_void_p] * 8 + [ctypes.c_int] * 6 +
                   [ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
