@@ -355,6 +355,7 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
     auto stage = [&](int64_t tile, Origin org, int buf) {
         const int live = rows_in(tile);
         const int64_t row0 = tile * C::TT;
+        float ss_mine = 0.0f, up_mine = 1.0f;
 #pragma unroll
         for (int p = 0; p < C::PASSES; ++p) {
             const int r = p * C::ROWS_PER_PASS + row_in_pass;
@@ -389,10 +390,6 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                 const auto sw = __builtin_amdgcn_permlane16_swap(float_to_bits(ss), float_to_bits(ss), false, false);
                 ss = bits_to_float(sw[0]) + bits_to_float(sw[1]);
             }
-            // v_sqrt_f32 (1 ulp), with a sum of squares in the subnormal range scaled into the normal one
-            const bool tiny = ss < 0x1p-96f;
-            const float nrm_s = __builtin_amdgcn_sqrtf(tiny ? ss * 0x1p64f : ss);
-            const float nrm = tiny ? nrm_s * 0x1p-32f : nrm_s;
             float up = 1.0f;
             uint4v h = pre[p];
             if constexpr (!kBf16) {
@@ -414,18 +411,31 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
                 h.w = pack_h2(_Float16(e[6] * down), _Float16(e[7] * down));
             }
             *reinterpret_cast<uint4v*>(&xs[buf][r * C::XS_STRIDE + chunk * 16]) = h;
-            if (chunk == 0) {
-                inv_s[buf][r] = up * __builtin_amdgcn_rcpf(nrm + 1e-10f);
-                if (r < live) {
-                    if (PAGED) {
-                        int head, is_v;
-                        uint8_t* dst = paged_row(org, r, head, is_v);
-                        if (dst) *reinterpret_cast<float*>(dst + pd.H * (D / 2) + 4 * head) = nrm;
-                    } else if (pd.append_n == 0u) {      // uniform
-                        (norms + row0)[r] = nrm;
-                    } else {
-                        norms[appended_row(org, r)] = nrm;
-                    }
+            // every lane of a row holds the row's sum: the lane of chunk p keeps the one of pass p
+            if (p == 0 || chunk == p) {
+                ss_mine = ss;
+                up_mine = up;
+            }
+        }
+        // ---- norm, row factor and the norm's store: once per tile, by the lanes of chunks 0..PASSES-1,
+        // each for the row it met in the pass of its chunk number ---------------------------------
+        static_assert(C::CPR >= C::PASSES, "a row has a lane for every pass");
+        // v_sqrt_f32 (1 ulp), with a sum of squares in the subnormal range scaled into the normal one
+        const bool tiny = ss_mine < 0x1p-96f;
+        const float nrm_s = __builtin_amdgcn_sqrtf(tiny ? ss_mine * 0x1p64f : ss_mine);
+        const float nrm = tiny ? nrm_s * 0x1p-32f : nrm_s;
+        if (chunk < C::PASSES) {
+            const int r = chunk * C::ROWS_PER_PASS + row_in_pass;
+            inv_s[buf][r] = up_mine * __builtin_amdgcn_rcpf(nrm + 1e-10f);
+            if (r < live) {
+                if (PAGED) {
+                    int head, is_v;
+                    uint8_t* dst = paged_row(org, r, head, is_v);
+                    if (dst) *reinterpret_cast<float*>(dst + pd.H * (D / 2) + 4 * head) = nrm;
+                } else if (pd.append_n == 0u) {      // uniform
+                    (norms + row0)[r] = nrm;
+                } else {
+                    norms[appended_row(org, r)] = nrm;
                 }
             }
         }
