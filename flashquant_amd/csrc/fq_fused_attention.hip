@@ -484,14 +484,31 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
 #pragma unroll
                 for (int r = 0; r < 16; ++r) O[ob][r] *= alpha;
         }
+        // The V operands of 16 tokens (one per 32-coordinate block) are read two such groups ahead of
+        // the products that use them (the compiler on its own reads one product ahead, which does
+        // not cover the LDS round trip): fences keep the groups in this order.
+        auto v_operand = [&](int ob, int s) {
+            const int c = (2 * s) ^ (4 * (ob & 1));
+            return *reinterpret_cast<const half8*>(kt + v_rd[c] + ob * 4096);
+        };
+        half8 va[4][NOB];
 #pragma unroll
-        for (int ob = 0; ob < NOB; ++ob)
+        for (int s = 0; s < 2; ++s)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int c = (2 * s) ^ (4 * (ob & 1));
-                const half8 a = *reinterpret_cast<const half8*>(kt + v_rd[c] + ob * 4096);
-                O[ob] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, __builtin_bit_cast(half8, pbv[s]), O[ob], 0, 0, 0);
+            for (int ob = 0; ob < NOB; ++ob) va[s][ob] = v_operand(ob, s);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            if (s + 2 < 4) {
+#pragma unroll
+                for (int ob = 0; ob < NOB; ++ob) va[s + 2][ob] = v_operand(ob, s + 2);
+                __builtin_amdgcn_sched_barrier(0);
             }
+#pragma unroll
+            for (int ob = 0; ob < NOB; ++ob)
+                O[ob] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[s][ob], __builtin_bit_cast(half8, pbv[s]), O[ob], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
 
     // ---- tiles ----------------------------------------------------------------------------------------
