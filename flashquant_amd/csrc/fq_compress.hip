@@ -292,6 +292,12 @@ __global__ __launch_bounds__(CompressCfg<D>::THREADS) void tq4_compress_kernel(
             base_v = reinterpret_cast<const uint4v*>(reinterpret_cast<uintptr_t>(pd.x_value) +
                                                      uintptr_t((row0 - pd.rows_k) * C::CPR * int64_t(sizeof(uint4v))));
         }
+        if (!PAGED && live == C::TT) {       // uniform: a whole tile needs no per-row conditions
+#pragma unroll
+            for (int p = 0; p < C::PASSES; ++p)
+                pre[p] = __builtin_nontemporal_load(base + p * C::ROWS_PER_PASS * C::CPR + tid);
+            return;
+        }
 #pragma unroll
         for (int p = 0; p < C::PASSES; ++p) {
             const int r = p * C::ROWS_PER_PASS + row_in_pass;
