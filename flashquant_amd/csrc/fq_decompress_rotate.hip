@@ -44,8 +44,17 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ float two_roundings(float c, float n) {
     float p = c * n;                       // float32 product first, as the reference rounds it
-    asm volatile("" : "+v"(p));            // (keeps the compiler from fusing it into the 16-bit conversion)
-    return p;
+    asm("" : "+v"(p));                     // (keeps the compiler from fusing it into the 16-bit conversion;
+    return p;                              // not volatile: the products of a row may be scheduled freely)
+}
+
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+
+// two float32 values rounded to nearest even and packed, the first in the low half
+template <int DT> __device__ __forceinline__ uint32_t round_pair(float a, float b) {
+    if constexpr (DT == FQ_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{a, b}, bf16x2v));
+    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{a, b}, half2v));
 }
 
 // MFMA row r of a 32-row block <-> output coordinate (within the block) such that accumulator
@@ -98,6 +107,17 @@ __global__ __launch_bounds__(DecRotCfg<D>::THREADS) void tq4_decompress_rotate_k
     uint32_t word[C::UPT];
     float nrm[C::UPT];
     auto issue_loads = [&](int64_t tile) {
+        if ((tile + 1) * C::TT <= M) {          // uniform: a whole tile needs no per-row conditions
+            const uint32_t* src = packed + tile * C::TT * C::UPR;
+            const float* nsrc = norms + tile * C::TT;
+#pragma unroll
+            for (int i = 0; i < C::UPT; ++i) {
+                const int u = tid + i * C::THREADS;
+                word[i] = __builtin_nontemporal_load(src + u);
+                nrm[i] = nsrc[u / C::UPR];
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < C::UPT; ++i) {
             const int u = tid + i * C::THREADS;
@@ -115,9 +135,7 @@ __global__ __launch_bounds__(DecRotCfg<D>::THREADS) void tq4_decompress_rotate_k
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
                 const uint32_t byte = (word[i] >> (8 * b)) & 0xffu;
-                const uint16_t hi = store_elem<DT>(two_roundings(lut[byte >> 4], nrm[i]));
-                const uint16_t lo = store_elem<DT>(two_roundings(lut[byte & 15u], nrm[i]));
-                h[b] = uint32_t(hi) | (uint32_t(lo) << 16);
+                h[b] = round_pair<DT>(two_roundings(lut[byte >> 4], nrm[i]), two_roundings(lut[byte & 15u], nrm[i]));
             }
             *reinterpret_cast<uint4v*>(&xs[buf][(u / C::UPR) * C::STRIDE + (u % C::UPR) * 16]) = uint4v{h[0], h[1], h[2], h[3]};
         }
