@@ -191,7 +191,7 @@ __global__ __launch_bounds__(DecRotCfg<D>::THREADS) void tq4_decompress_rotate_k
                     v0 = __builtin_fmaf(acc_lo[2 * i], 1.0f / 4096.0f, v0);
                     v1 = __builtin_fmaf(acc_lo[2 * i + 1], 1.0f / 4096.0f, v1);
                 }
-                w[i] = uint32_t(store_elem<DT>(v0)) | (uint32_t(store_elem<DT>(v1)) << 16);
+                w[i] = round_pair<DT>(v0, v1);
             }
             uint8_t* dst = &os[(32 * tb + n32) * C::STRIDE + (32 * cb + 16 * kg) * 2];
             *reinterpret_cast<uint4v*>(dst) = uint4v{w[0], w[1], w[2], w[3]};
