@@ -50,6 +50,16 @@ template <int DT> __device__ __forceinline__ uint16_t store_elem(float v);
 template <> __device__ __forceinline__ uint16_t store_elem<FQ_F16>(float v) { return float_to_f16(v); }
 template <> __device__ __forceinline__ uint16_t store_elem<FQ_BF16>(float v) { return float_to_bf16(v); }
 
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+
+// two float32 values rounded to nearest even and packed, the first in the low half
+// (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32: one instruction per pair)
+template <int DT> __device__ __forceinline__ uint32_t round_pair(float a, float b) {
+    if constexpr (DT == FQ_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{a, b}, bf16x2v));
+    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{a, b}, half2v));
+}
+
 __device__ __forceinline__ uint32_t pack_h2(_Float16 lo, _Float16 hi) {
     return uint32_t(__builtin_bit_cast(uint16_t, lo)) | (uint32_t(__builtin_bit_cast(uint16_t, hi)) << 16);
 }

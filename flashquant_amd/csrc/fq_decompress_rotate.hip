@@ -48,15 +48,6 @@ __device__ __forceinline__ float two_roundings(float c, float n) {
     return p;                              // not volatile: the products of a row may be scheduled freely)
 }
 
-typedef float float2v __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
-
-// two float32 values rounded to nearest even and packed, the first in the low half
-template <int DT> __device__ __forceinline__ uint32_t round_pair(float a, float b) {
-    if constexpr (DT == FQ_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{a, b}, bf16x2v));
-    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{a, b}, half2v));
-}
-
 // MFMA row r of a 32-row block <-> output coordinate (within the block) such that accumulator
 // register i of lane half h holds coordinate 16 h + i.
 __device__ __forceinline__ int row_to_coord(int r) { return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3); }
