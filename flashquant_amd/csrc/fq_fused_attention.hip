@@ -51,6 +51,10 @@ struct PrefillCfg {
     static constexpr int NOB = D / 32;                    // 32-coordinate blocks of the output
     static constexpr int NJ = D / 32;                     // 32-wide k-steps of the head rotations
     static constexpr int PB = D / 2;                      // packed bytes per token and head
+    // The rotation matrix as MFMA operands (two fp16 terms), shared by the wavefronts of a workgroup:
+    // block (column block cb, k-step j) holds one 16-byte operand per lane and term.  They lie where
+    // the lookup tables are between the query stage and the end of the tile loop (64 KB).
+    static constexpr int RTERM = NKS * NJ * 64 * 16;      // bytes per term: 32768 at D = 128
 };
 
 struct PrefillParams {
@@ -159,8 +163,8 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     }
     if (!unit_live) my_tiles = 0;
 
-    // ---- tables -----------------------------------------------------------------------------
-    fill_pair_tables<8>(lut, p.centroids_k[lane & 15], p.centroids_v[lane & 15], 15, w, lane);
+    // ---- tables: filled after the query stage, whose rotation operands use their place ----------
+    static_assert(2 * Cfg::RTERM <= int(sizeof(lut)), "the rotation operands fit where the tables are");
     // cleared here: the barriers of the query stage order this before the first dequantisation
     if (tid < 2) big_tile[tid] = 0;
     if (tid < 256) (&scale_exp[0][0])[tid] = 0;
@@ -306,6 +310,33 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
 
     issue_loads(0);
 
+    // ---- the rotation matrix, split once per workgroup ------------------------------------------------
+    // Wavefront cb fetches column block cb of R^T (or of R), splits it into two fp16 terms and
+    // leaves the operands in LDS; every wavefront then reads the blocks it multiplies with from
+    // there (each wavefront fetching and splitting the whole matrix for itself, three times per
+    // workgroup, was an eighth of the kernel's time).
+    uint8_t* rshare = reinterpret_cast<uint8_t*>(lut);
+    auto share_rotation = [&](bool transposed) {
+        if (w < NKS) {
+            float rbv[NJ][8];
+            load_rotation_any<D>(p.rotation, p.rot_col_major != 0, transposed, 16 * w, n16, g4, rbv);
+            half8 rhi[NJ], rlo[NJ];
+            split_rotation_block<D>(rbv, rhi, rlo);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                *reinterpret_cast<half8*>(rshare + ((w * NJ + j) * 64 + lane) * 16) = rhi[j];
+                *reinterpret_cast<half8*>(rshare + Cfg::RTERM + ((w * NJ + j) * 64 + lane) * 16) = rlo[j];
+            }
+        }
+    };
+    auto shared_rotation_block = [&](int cb, half8 (&rhi)[NJ], half8 (&rlo)[NJ]) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            rhi[j] = *reinterpret_cast<const half8*>(rshare + ((cb * NJ + j) * 64 + lane) * 16);
+            rlo[j] = *reinterpret_cast<const half8*>(rshare + Cfg::RTERM + ((cb * NJ + j) * 64 + lane) * 16);
+        }
+    };
+
     // ---- query: rotate this wavefront's 32 rows, round to the query dtype, scale to fp16 ----------
     half8 qb[NKS];
     float krow;
@@ -324,11 +355,11 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
             for (int j = 0; j < NJ; ++j) raw[j] = *reinterpret_cast<const uint4v*>(qbase + int64_t(pos) * q_stride + 32 * j + 8 * g4);
             rows_as_f16<D, DT>(raw, a[rb], up[rb]);
         }
+        share_rotation(true);
+        __syncthreads();
         for (int cb = 0; cb < NKS; ++cb) {
-            float rbv[NJ][8];
-            load_rotation_any<D>(p.rotation, p.rot_col_major != 0, true, 16 * cb, n16, g4, rbv);
             half8 rhi[NJ], rlo[NJ];
-            split_rotation_block<D>(rbv, rhi, rlo);
+            shared_rotation_block(cb, rhi, rlo);
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb) {
                 const float4v acc = rotate_block_f16<D>(a[rb], rhi, rlo);
@@ -360,8 +391,10 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
         for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
             for (int e = 0; e < 8; ++e) qb[ks][e] = _Float16(qf[ks][e] * down);
-        __syncthreads();   // the staging area becomes tile buffers
+        __syncthreads();   // the staging area becomes tile buffers, the rotation operands lookup tables
     }
+    fill_pair_tables<8>(lut, p.centroids_k[lane & 15], p.centroids_v[lane & 15], 15, w, lane);
+    __syncthreads();
 
     // ---- lane-constant LDS read offsets ----------------------------------------------------------
     const int k_rd = m32 * kPfKStride + 16 * hf;
@@ -535,6 +568,8 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     float* stf = reinterpret_cast<float*>(bufs + w * kPfStageBytes);   // (16 rows, D) float32
     uint16_t* obase = PAGED ? p.out + (q_row0 + hq) * D : p.out + (q_row0 + int64_t(hq) * NQ) * D;
+    __syncthreads();                // every wavefront is done with the lookup tables
+    share_rotation(false);          // (the barrier below orders it before its readers)
     for (int half_rows = 0; half_rows < 2; ++half_rows) {
         __syncthreads();
         if ((m32 >> 4) == half_rows) {
@@ -564,10 +599,8 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
         float up;
         rows_split_f16<D>(a, ahi, alo, up);
         for (int cb = 0; cb < NKS; ++cb) {
-            float rbv[NJ][8];
-            load_rotation_any<D>(p.rotation, p.rot_col_major != 0, false, 16 * cb, n16, g4, rbv);
             half8 rhi[NJ], rlo[NJ];
-            split_rotation_block<D>(rbv, rhi, rlo);
+            shared_rotation_block(cb, rhi, rlo);
             const float4v acc = rotate_block_f16x3<D>(ahi, alo, rhi, rlo);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
