@@ -457,6 +457,22 @@ def test_fused_attention_llama_heads(causal, dtype):
     _check_prefill(1, 32, 8, 200, 200, dtype, causal)
 
 
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_fused_attention_takes_the_rotation_in_either_layout(d):
+    """The wavefronts of a workgroup share the split matrix (head_dim 64 and 128): row-major and
+    column-major matrices must give the same bits, for the query rotation and the rotation back."""
+    q, kp, kn, vp, vn, c, r = _prefill_case(2, 8, 2, 150, 150, torch.bfloat16, 77, d=d)
+    args = [t.to(DEV) for t in (q, kp, kn, vp, vn, c, c)]
+    row_major = r.contiguous().to(DEV)
+    col_major = r.t().contiguous().t().to(DEV)
+    assert row_major.is_contiguous() and not col_major.is_contiguous()
+    a = K.fused_tq_attention(*args, row_major, is_causal=True)
+    b = K.fused_tq_attention(*args, col_major, is_causal=True)
+    assert torch.equal(a, b)
+    want = O.fused_tq_attention(q, kp, kn, vp, vn, c, c, r, is_causal=True)
+    assert (a.cpu().float() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
+
+
 @pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 4), (6, 2), (16, 2), (16, 1), (5, 1)])
 def test_fused_attention_group_sizes(hq, hkv):
     _check_prefill(2, hq, hkv, 97, 97, torch.bfloat16, True, seed=21)
