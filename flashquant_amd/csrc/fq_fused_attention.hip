@@ -492,23 +492,40 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
         m_run = mnew;
         uint4v pbv[4];
         float ps = 0.0f;
+        // two copies of the weight loop, so that the common one has no branch inside (the values of a
+        // loop with a rare branch in it are copied where the paths meet)
+        if (!big) {
+            const half2v ones = {_Float16(1.0f), _Float16(1.0f)};
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            float pe[8];
+            for (int s = 0; s < 4; ++s) {
+                float pe[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                pe[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[s >> 1][8 * (s & 1) + e], krow, -ms));
-                ps += pe[e];
+                for (int e = 0; e < 8; ++e)
+                    pe[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[s >> 1][8 * (s & 1) + e], krow, -ms));
+                const uint32_t pw[4] = {pack_rtz(pe[0], pe[1]), pack_rtz(pe[2], pe[3]), pack_rtz(pe[4], pe[5]), pack_rtz(pe[6], pe[7])};
+                // the denominator sums the weights as the second product sees them (fp16, one
+                // v_dot2_f32_f16 per pair)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) ps = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, pw[c]), ones, ps, false);
+                pbv[s] = uint4v{pw[0], pw[1], pw[2], pw[3]};
             }
-            if (big) {
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                float pe[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    pe[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[s >> 1][8 * (s & 1) + e], krow, -ms));
+                    ps += pe[e];
+                }
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
                     const int4v ev = exps_of(64 + 32 * (s >> 1) + 8 * (2 * (s & 1) + q) + 4 * hf);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) pe[4 * q + c] = __builtin_ldexpf(pe[4 * q + c], ev[c]);
                 }
+                pbv[s] = uint4v{pack_rtz(pe[0], pe[1]), pack_rtz(pe[2], pe[3]), pack_rtz(pe[4], pe[5]), pack_rtz(pe[6], pe[7])};
             }
-            pbv[s] = uint4v{pack_rtz(pe[0], pe[1]), pack_rtz(pe[2], pe[3]), pack_rtz(pe[4], pe[5]), pack_rtz(pe[6], pe[7])};
         }
         l_run = __builtin_fmaf(l_run, alpha, ps);
         if (__any(alpha != 1.0f)) {
