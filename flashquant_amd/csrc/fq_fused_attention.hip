@@ -254,15 +254,17 @@ __global__ __launch_bounds__(512) void fused_tq_attention_kernel(const PrefillPa
                 nv1 = *reinterpret_cast<const float*>(rb2 + H * (D + 4) + 4 * hkv);
             }
         } else {
+            // (32-bit offsets from the wave-uniform slab pointers: a slab of 2^31 / PB tokens is far beyond
+            // any context)
             if (does_k) {
-                kraw = *reinterpret_cast<const uint2v*>(kp + int64_t(tkk) * PB + 8 * gqk);
-                nk = knp[tkk];
+                kraw = *reinterpret_cast<const uint2v*>(kp + (uint32_t(tkk) * uint32_t(PB) + 8u * uint32_t(gqk)));
+                nk = knp[uint32_t(tkk)];
             }
             if (does_v) {
-                vra = *reinterpret_cast<const uint32_t*>(vp + int64_t(ta) * PB + 4 * jv);
-                vrb = *reinterpret_cast<const uint32_t*>(vp + int64_t(tb) * PB + 4 * jv);
-                nv0 = vnp[ta];
-                nv1 = vnp[tb];
+                vra = *reinterpret_cast<const uint32_t*>(vp + (uint32_t(ta) * uint32_t(PB) + 4u * uint32_t(jv)));
+                vrb = *reinterpret_cast<const uint32_t*>(vp + (uint32_t(tb) * uint32_t(PB) + 4u * uint32_t(jv)));
+                nv0 = vnp[uint32_t(ta)];
+                nv1 = vnp[uint32_t(tb)];
             }
         }
     };
@@ -667,6 +669,7 @@ extern "C" int fq_fused_tq_attention_strided(const void* q, const uint8_t* k_pac
     using namespace fq;
     if (B < 0 || H_Q <= 0 || H_KV <= 0 || N_Q < 0 || N_KV < 0 || H_Q % H_KV != 0) return FQ_ERR_BAD_SHAPE;
     if (k_capacity < N_KV || v_capacity < N_KV) return FQ_ERR_BAD_SHAPE;
+    if (N_KV > (1 << 24)) return FQ_ERR_BAD_SHAPE;      // the kernels address a slab's tokens with 32-bit byte offsets
     if (!fq_host::supported_dim(D)) return FQ_ERR_UNSUPPORTED_DIM;
     if (dtype != FQ_F16 && dtype != FQ_BF16) return FQ_ERR_UNSUPPORTED_DTYPE;
     if (B == 0 || N_Q == 0) return FQ_OK;

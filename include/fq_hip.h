@@ -229,7 +229,7 @@ int fq_tq4_decompress_rotated(const uint8_t* packed, const float* norms, const f
  *              ignored when N_Q == 1, as in the reference
  * D in {64, 128, 256}: 128 runs the tuned kernel, 64 and 256 a general one
  * (the switch FQ_OPT_ATTENTION_ANY_DIM sends 128 there too).  H_Q a multiple
- * of H_KV; N_KV >= 1.  K and V are dequantised to fp16 with the norm folded in, so a
+ * of H_KV; 1 <= N_KV <= 2^24.  K and V are dequantised to fp16 with the norm folded in, so a
  * row norm times a centroid must stay below 65504.
  */
 int fq_fused_tq_attention(const void* q, const uint8_t* k_packed, const float* k_norms,

@@ -215,6 +215,8 @@ def test_ring_buffer_and_rotated_decompress_argument_errors(lib):
     assert att(kcap=63) == FQ_SHAPE and att(vcap=10) == FQ_SHAPE      # a capacity below the length
     assert att(kcap=1000, vcap=2000) == FQ_NULL                       # accepted, then the NULL operands are found
     assert att(d=96) == FQ_DIM
+    big = (1 << 24) + 1
+    assert att(nkv=big, kcap=big, vcap=big) == FQ_SHAPE                # beyond the 32-bit offsets of a slab
     dr = lib.fq_tq4_decompress_rotated
     dr.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
                                            ctypes.c_void_p]
