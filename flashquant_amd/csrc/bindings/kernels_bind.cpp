@@ -50,6 +50,8 @@ int option_id(const std::string& name) {
     if (name == "attention_any_dim") return FQ_OPT_ATTENTION_ANY_DIM;
     if (name == "decode_tiny_spin") return FQ_OPT_DECODE_TINY_SPIN;
     if (name == "compress_three_terms") return FQ_OPT_COMPRESS_THREE_TERMS;
+    if (name == "decode_ring") return FQ_OPT_DECODE_RING;
+    if (name == "reduce_rows") return FQ_OPT_REDUCE_ROWS;
     throw std::invalid_argument("unknown option '" + name + "'");
 }
 
@@ -781,14 +783,15 @@ void bind_kernels(py::module_& m) {
     m.def("tq4_decompress_rotated", &tq4_decompress_rotated, py::arg("packed"), py::arg("norms"), py::arg("centroids"),
           py::arg("rotation"), py::arg("dtype"), py::arg("out") = py::none(),
           "tq4_decompress to dtype, then (x.float() @ rotation).to(dtype): original-space rows in one launch");
-    m.def("set_option", [](const std::string& name, bool value) {
+    m.def("set_option", [](const std::string& name, int value) {
               const int id = option_id(name);
               const int before = fq_get_option(id);
-              fqbind::raise_on_error(fq_set_option(id, value ? 1 : 0), "set_option");
-              return before != 0;
+              fqbind::raise_on_error(fq_set_option(id, value), "set_option");
+              return before;
           }, py::arg("name"), py::arg("value"),
-          "Set a kernel-variant switch ('decode_copy_waves', 'decode_direct', 'attention_any_dim', 'compress_three_terms'); returns the old value");
-    m.def("get_option", [](const std::string& name) { return fq_get_option(option_id(name)) != 0; }, py::arg("name"));
+          "Set a kernel-variant switch ('decode_copy_waves', 'decode_direct', 'decode_ring', 'attention_any_dim', "
+          "'compress_three_terms': 0 / 1; 'reduce_rows': 0, 4, 8 or 16); returns the old value");
+    m.def("get_option", [](const std::string& name) { return fq_get_option(option_id(name)); }, py::arg("name"));
     m.def("paged_decode_fault_count", []() {
               unsigned int n = 0;
               fqbind::raise_on_error(fq_paged_decode_fault_count(&n), "paged_decode_fault_count");

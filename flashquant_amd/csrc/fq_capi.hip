@@ -25,6 +25,10 @@ void init_options() {
         g_options[FQ_OPT_DECODE_TINY_SPIN] = 0;
         v = std::getenv("FQ_COMPRESS_THREE_TERMS");
         g_options[FQ_OPT_COMPRESS_THREE_TERMS] = (v != nullptr && v[0] == '1') ? 1 : 0;
+        v = std::getenv("FQ_REDUCE_ROWS");
+        g_options[FQ_OPT_REDUCE_ROWS] = v != nullptr ? std::atoi(v) : 0;
+        v = std::getenv("FQ_DECODE_RING");
+        g_options[FQ_OPT_DECODE_RING] = (v != nullptr && v[0] == '1') ? 1 : 0;
     });
 }
 }  // namespace
@@ -47,7 +51,7 @@ extern "C" int fq_get_option(int option) {
 extern "C" int fq_set_option(int option, int value) {
     if (option < 0 || option >= FQ_OPTION_COUNT) return FQ_ERR_BAD_SHAPE;
     init_options();
-    g_options[option].store(value != 0 ? 1 : 0, std::memory_order_relaxed);
+    g_options[option].store(option == FQ_OPT_REDUCE_ROWS ? value : (value != 0 ? 1 : 0), std::memory_order_relaxed);
     return FQ_OK;
 }
 

@@ -263,6 +263,27 @@ __device__ __forceinline__ void split_rotation_block_bf16(const float (&b)[D / 3
             t[2][j][e] = bf16_top(r1 - bf16_as_float(t1));
         }
 }
+// The same three terms with the element pairs packed by v_perm_b32 and the remainders taken with an
+// and + a subtraction (5.5 vector instructions per element instead of about 10).
+template <int D>
+__device__ __forceinline__ void split_rotation_block_bf16_packed(const float (&b)[D / 32][8], bf16v8 (&t)[3][D / 32]) {
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+        uint32_t w[3][4];
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            const uint32_t a0 = float_to_bits(b[j][e]), a1 = float_to_bits(b[j][e + 1]);
+            w[0][e / 2] = __builtin_amdgcn_perm(a1, a0, 0x07060302u);            // top halves of the pair
+            const float r0 = b[j][e] - bits_to_float(a0 & 0xffff0000u), r1 = b[j][e + 1] - bits_to_float(a1 & 0xffff0000u);
+            const uint32_t c0 = float_to_bits(r0), c1 = float_to_bits(r1);
+            w[1][e / 2] = __builtin_amdgcn_perm(c1, c0, 0x07060302u);
+            const float s0 = r0 - bits_to_float(c0 & 0xffff0000u), s1 = r1 - bits_to_float(c1 & 0xffff0000u);
+            w[2][e / 2] = __builtin_amdgcn_perm(float_to_bits(s1), float_to_bits(s0), 0x07060302u);
+        }
+#pragma unroll
+        for (int k = 0; k < 3; ++k) t[k][j] = __builtin_bit_cast(bf16v8, uint4v{w[k][0], w[k][1], w[k][2], w[k][3]});
+    }
+}
 template <int D>
 __device__ __forceinline__ float4v rotate_block_bf16(const bf16v8 (&a)[D / 32], const bf16v8 (&t)[3][D / 32]) {
     float4v acc = {0.f, 0.f, 0.f, 0.f};

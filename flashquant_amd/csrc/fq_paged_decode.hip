@@ -56,6 +56,7 @@
 
 #include "fq_common.hpp"
 #include "fq_device.hpp"
+#include "fq_paged_decode.hpp"
 
 namespace fq_host {
 // The switch FQ_OPT_DECODE_DIRECT routes every shape to the direct kernel (both kernels are kept
@@ -67,30 +68,6 @@ int device_cu_count();
 namespace fq {
 
 
-struct DecodeParams {
-    const void* q_rot;          // (S, H_Q, D) query dtype: rotated, or un-rotated when `rotation` is set
-    int rot_col_major;          // layout of `rotation` / of the matrix given to the side kernels
-    const float* rotation;      // staged kernel only: rotate the query in the prologue (NULL: already rotated)
-    const float* sketch;        // TurboQuantProd pages only: the (D, D) sign-sketch matrix S
-    const uint8_t* cache;       // (num_blocks, BS, H_KV*(D+8))
-    const int32_t* block_table; // (S, max_blocks)
-    const int32_t* seq_lens;    // (S,)
-    const float* centroids_k;
-    const float* centroids_v;
-    float* part_acc;            // (S, H_Q, NS, D)
-    float* part_m;              // (S, H_Q, NS)
-    float* part_l;              // (S, H_Q, NS)
-    int H_Q, H_KV, G;           // G = H_Q / H_KV
-    int max_blocks;
-    int num_blocks;
-    int num_splits;
-    int two_tables;             // centroids_v differs from centroids_k
-    float scale_log2e;          // sm_scale * log2(e)
-    int heads_per_wg;           // direct kernel: KV heads a workgroup serves; its other wavefronts take further splits
-    int spin_limit;             // staged kernel: polls of a bounded wait between wavefronts before it gives up
-    int balance_slots;          // staged kernel: > 0 lets the workgroups size the token chunks from the actual
-                                // sequence lengths, for this many workgroups running at a time (num_seqs <= 64)
-};
 
 
 // head_dim 256 keeps 64 accumulator registers per lane and runs with at most four wavefronts per workgroup,
@@ -810,70 +787,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // leave their last splits empty
     int chunk = (((p.max_blocks * BS + NS - 1) / NS) + 63) & ~63;
     int L_known = -1;
-    if (p.balance_slots > 0) {
-        // Ragged batches of long contexts (at most 64 sequences, one lane each).  With the chunk
-        // of the longest possible context the live workgroups are all the same size and their
-        // count is whatever the lengths add up to, e.g. 2.1 rounds over the chip, which costs 3.
-        // Every workgroup evaluates the same 64 candidate chunk sizes (one per lane) on the
-        // actual lengths, cost = rounds x (chunk + a prologue's worth of tokens), and takes the
-        // cheapest: same inputs, same arithmetic, same answer in every workgroup.  Larger chunks
-        // only: the split count bounds the chunk from below.
-        const int cap = rowwide ? chunk * NS : 64 * PVR * BS;       // page ids of a split: 64 * PVR lanes
-        const int step = ((chunk >> 4) + 63) & ~63;
-        int cand = chunk + lane * step;
-        cand = cand < cap ? cand : cap;
-        cand = cand > chunk ? cand : chunk;
-        const float rc = __builtin_amdgcn_rcpf(float(cand));
-        const int nseq = int(gridDim.x);
-        int l_real = lane < nseq ? p.seq_lens[lane] : 0;
-        l_real = l_real < 0 ? 0 : (l_real > p.max_blocks * BS * (HALF ? 2 : 1) ? p.max_blocks * BS * (HALF ? 2 : 1) : l_real);
-        const int l_mine = HALF ? (l_real + 1) >> 1 : l_real;      // in rows
-        float groups = 0.0f;
-        for (int sq = 0; sq < nseq; ++sq)
-            groups += __builtin_ceilf(float(__builtin_amdgcn_readlane(l_mine, sq)) * rc - 0.0009765625f);
-        const float rounds = __builtin_ceilf(groups * __builtin_amdgcn_rcpf(float(p.balance_slots)) - 0.0009765625f);
-        const float cost = (rounds < 1.0f ? 1.0f : rounds) * float(cand + 96);
-        uint32_t key = (uint32_t(cost) << 6) | uint32_t(lane);
-#pragma unroll
-        for (int mask = 1; mask < 64; mask <<= 1) {
-            const uint32_t other = uint32_t(__shfl_xor(int(key), mask, kWave));
-            key = other < key ? other : key;
-        }
-        const int best = chunk + int(key & 63u) * step;
-        chunk = best < cap ? best : (cap > chunk ? cap : chunk);
-
-        // The live (sequence, split) pairs first, in sequence order, then the empty ones: the w-th
-        // workgroup of the grid takes the w-th pair of that list.  Live workgroups are all of one
-        // size and now consecutive, so they spread evenly over the XCDs and CUs whatever the lengths.
-        auto scan = [&](int v) {
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int t = __shfl_up(v, d, kWave);
-                v += lane >= d ? t : 0;
-            }
-            return v;
-        };
-        int n_mine = lane < nseq ? (l_mine + chunk - 1) / chunk : 0;
-        n_mine = n_mine < NS ? n_mine : NS;
-        const int live_incl = scan(n_mine);
-        const int total_live = __builtin_amdgcn_readlane(live_incl, 63);
-        const int w = int(blockIdx.x) + int(gridDim.x) * int(blockIdx.y);
-        if (w < total_live) {
-            const int s_idx = __builtin_popcountll(__ballot(live_incl <= w));
-            seq = s_idx;
-            split = w - __builtin_amdgcn_readlane(live_incl - n_mine, s_idx);
-        } else {
-            const int e = w - total_live;
-            const int dead_mine = lane < nseq ? NS - n_mine : 0;
-            const int dead_incl = scan(dead_mine);
-            int s_idx = __builtin_popcountll(__ballot(dead_incl <= e));
-            s_idx = s_idx < nseq ? s_idx : nseq - 1;
-            seq = s_idx;
-            split = __builtin_amdgcn_readlane(n_mine, s_idx) + (e - __builtin_amdgcn_readlane(dead_incl - dead_mine, s_idx));
-            split = split < NS ? split : NS - 1;
-        }
-        L_known = __builtin_amdgcn_readlane(l_real, seq);
-    }
+    if (p.balance_slots > 0) balance_chunks<PVR, BS, HALF>(p, lane, NS, rowwide, chunk, seq, split, L_known);
 
     const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + (int64_t(seq) * p.H_Q + hq0) * 128;
     uint4v q_pre[2][4];
@@ -1518,9 +1432,10 @@ __global__ __launch_bounds__(256) void rotate_q_kernel(const uint16_t* __restric
 // Combine of the split partials: out_rot = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
 // (0 when every split is empty), rounded to the query dtype as the reference's
 // rotated-space result is (cpu_reference.py:366), then multiplied by R in float32 and
-// rounded again (paged_decode.py:123).  rows = num_seqs * H_Q; a workgroup owns 16 rows:
-// each wavefront combines 4 of them into LDS, then all rotate from there.
-template <int D, int DT>
+// rounded again (paged_decode.py:123).  rows = num_seqs * H_Q; a workgroup owns RW rows
+// (4, 8 or 16: the fewer, the more workgroups share the combine, the more often the matrix is
+// fetched): 256 / RW threads combine a row into LDS, then all rotate from there.
+template <int D, int DT, int RW>
 __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restrict__ part_acc,
                                                             const float* __restrict__ part_m,
                                                             const float* __restrict__ part_l,
@@ -1528,126 +1443,139 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
                                                             int64_t rows, int NS, int col_major) {
     constexpr int CBW = D / 64;            // 16-column blocks per wavefront
     constexpr int OSTRIDE = D + 8;         // 16-bit words per staged row (padded: conflict-free operand reads)
-    __shared__ __attribute__((aligned(16))) uint16_t os[kRotRows * OSTRIDE];   // combined rows, query dtype
+    constexpr int TPR = 256 / RW;          // threads that combine one row
+    constexpr int CPT = D / TPR < 2 ? 2 : D / TPR;      // coordinates per thread and pass (2, 4 or 8)
+    constexpr int ACTIVE = D / CPT < TPR ? D / CPT : TPR;   // threads of a row that have coordinates
+    __shared__ __attribute__((aligned(16))) uint16_t os[RW * OSTRIDE];   // combined rows, query dtype
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
-    const int64_t row0 = int64_t(blockIdx.x) * kRotRows;
+    const int64_t row0 = int64_t(blockIdx.x) * RW;
 
-    // the matrix columns of this wavefront are asked for first: they arrive during the combine
+    // ---- combine: the loads of up to eight splits (maximum, denominator, accumulator) are all in
+    // flight together; they are asked for before the matrix, which is needed later ------------------
+    const int r = threadIdx.x / TPR, t = threadIdx.x % TPR;
+    const int64_t row = row0 + r < rows ? row0 + r : rows - 1;
+    const int64_t base = row * NS;
+    float mstar = -__builtin_inff();
+    bool poisoned = false;      // a split published NaN as its maximum: its workgroup could not vouch for it
+    // bit c: the chunk of eight splits c (mod 64) holds a split that wrote something.  Splits
+    // beyond a sequence's length are empty (m = -inf), whole chunks of them when the split count
+    // was chosen for the longest possible context: those are not read at all.
+    uint64_t live_chunks = ~0ull;
+    if (NS > 8) {
+        // the threads of a row share the maxima: thread t reads those of splits t, t + TPR, ...,
+        // four at a time, so that 4 TPR splits cost one round trip
+        uint32_t live_lo = 0u, live_hi = 0u;
+        for (int s0 = 0; s0 < NS; s0 += 4 * TPR) {
+            float mv[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int idx = s0 + t + TPR * k;
+                mv[k] = part_m[base + (idx < NS ? idx : NS - 1)];
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int idx = s0 + t + TPR * k;
+                const bool wrote = idx < NS && mv[k] != -__builtin_inff();
+                poisoned = poisoned || (idx < NS && mv[k] != mv[k]);
+                mstar = wrote ? __builtin_fmaxf(mstar, mv[k]) : mstar;
+                const int chunk = (idx >> 3) & 63;
+                live_lo |= (wrote && chunk < 32) ? 1u << chunk : 0u;
+                live_hi |= (wrote && chunk >= 32) ? 1u << (chunk - 32) : 0u;
+            }
+        }
+#pragma unroll
+        for (int mask = 1; mask < TPR; mask <<= 1) {
+            mstar = __builtin_fmaxf(mstar, xor_shuffle(mstar, mask));
+            poisoned = poisoned || __shfl_xor(int(poisoned), mask, kWave) != 0;
+            live_lo |= uint32_t(__shfl_xor(int(live_lo), mask, kWave));
+            live_hi |= uint32_t(__shfl_xor(int(live_hi), mask, kWave));
+        }
+        live_chunks = (uint64_t(live_hi) << 32) | live_lo;
+    }
+    float num[CPT];
+#pragma unroll
+    for (int e = 0; e < CPT; ++e) num[e] = 0.0f;
+    float den = 0.0f;
+    const int c0 = CPT * (t < ACTIVE ? t : 0);
+    for (int s0 = 0; s0 < NS; s0 += 8) {
+        if (!((live_chunks >> ((s0 >> 3) & 63)) & 1ull)) continue;
+        float mv[8], lv[8];
+        float pv[8][CPT];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int sidx = s0 + k < NS ? s0 + k : NS - 1;
+            mv[k] = part_m[base + sidx];
+            lv[k] = part_l[base + sidx];
+            // An empty split (m = -inf) never wrote its accumulator; it is read all the same
+            // (and ignored below), so that no load has to wait for another one.
+            const float* src = part_acc + (base + sidx) * D + c0;
+            if constexpr (CPT == 2) {
+                const float2v v = *reinterpret_cast<const float2v*>(src);
+                pv[k][0] = v.x; pv[k][1] = v.y;
+            } else {
+#pragma unroll
+                for (int q4 = 0; q4 < CPT / 4; ++q4) {
+                    const float4v v = reinterpret_cast<const float4v*>(src)[q4];
+                    pv[k][4 * q4] = v.x; pv[k][4 * q4 + 1] = v.y; pv[k][4 * q4 + 2] = v.z; pv[k][4 * q4 + 3] = v.w;
+                }
+            }
+        }
+        if (NS <= 8) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                mstar = __builtin_fmaxf(mstar, mv[k]);
+                poisoned = poisoned || mv[k] != mv[k];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const bool use = s0 + k < NS && mv[k] != -__builtin_inff();
+            const float w = use ? __builtin_amdgcn_exp2f(mv[k] - mstar) : 0.0f;
+            den = __builtin_fmaf(lv[k], w, den);
+            // a weight of 0 must also silence a NaN or Inf in memory that no split wrote
+#pragma unroll
+            for (int e = 0; e < CPT; ++e) num[e] = use ? __builtin_fmaf(pv[k][e], w, num[e]) : num[e];
+        }
+    }
+    // the matrix columns of this wavefront: asked for behind the partials, they arrive during the combine
     float rbv[CBW][D / 32][8];
     if (R != nullptr) {
 #pragma unroll
         for (int i = 0; i < CBW; ++i) load_rotation_any<D>(R, col_major != 0, false, 16 * (wave + 4 * i), n, g, rbv[i]);
     }
-
-    // ---- combine: thread t handles 8 consecutive coordinates of row t / 16; the loads of up to
-    // eight splits (maximum, denominator, accumulator) are all in flight together -------------------
     {
-        const int r = threadIdx.x >> 4;
-        const int64_t row = row0 + r < rows ? row0 + r : rows - 1;
-        const int64_t base = row * NS;
-        float mstar = -__builtin_inff();
-        bool poisoned = false;      // a split published NaN as its maximum: its workgroup could not vouch for it
-        // bit c: the chunk of eight splits c (mod 64) holds a split that wrote something.  Splits
-        // beyond a sequence's length are empty (m = -inf), whole chunks of them when the split count
-        // was chosen for the longest possible context: those are not read at all.
-        uint64_t live_chunks = ~0ull;
-        if (NS > 8) {
-            // the 16 threads of a row share the maxima: thread t reads those of splits t, t + 16, ...,
-            // four at a time, so that up to 64 splits cost one round trip
-            const int t16 = threadIdx.x & 15;
-            uint32_t live_lo = 0u, live_hi = 0u;
-            for (int s0 = 0; s0 < NS; s0 += 64) {
-                float mv[4];
+        const bool live = row0 + r < rows && den > 0.0f;
+        const float inv = live ? 1.0f / den : 0.0f;
+        uint32_t wds[CPT / 2];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int idx = s0 + t16 + 16 * k;
-                    mv[k] = part_m[base + (idx < NS ? idx : NS - 1)];
-                }
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int idx = s0 + t16 + 16 * k;
-                    const bool wrote = idx < NS && mv[k] != -__builtin_inff();
-                    poisoned = poisoned || (idx < NS && mv[k] != mv[k]);
-                    mstar = wrote ? __builtin_fmaxf(mstar, mv[k]) : mstar;
-                    const int chunk = (idx >> 3) & 63;
-                    live_lo |= (wrote && chunk < 32) ? 1u << chunk : 0u;
-                    live_hi |= (wrote && chunk >= 32) ? 1u << (chunk - 32) : 0u;
-                }
-            }
-#pragma unroll
-            for (int mask = 1; mask < 16; mask <<= 1) {
-                mstar = __builtin_fmaxf(mstar, xor_shuffle(mstar, mask));
-                poisoned = poisoned || __shfl_xor(int(poisoned), mask, kWave) != 0;
-                live_lo |= uint32_t(__shfl_xor(int(live_lo), mask, kWave));
-                live_hi |= uint32_t(__shfl_xor(int(live_hi), mask, kWave));
-            }
-            live_chunks = (uint64_t(live_hi) << 32) | live_lo;
+        for (int e = 0; e < CPT / 2; ++e) {
+            // a poisoned row comes out NaN, never as a plausible number
+            const uint32_t a0 = poisoned ? store_elem<DT>(__builtin_nanf("")) : (live ? store_elem<DT>(num[2 * e] / den) : 0u);
+            const uint32_t a1 = poisoned ? store_elem<DT>(__builtin_nanf("")) : (live ? store_elem<DT>(num[2 * e + 1] / den) : 0u);
+            wds[e] = a0 | (a1 << 16);
         }
-        for (int c0 = 8 * (threadIdx.x & 15); c0 < D; c0 += 128) {
-            float num[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) num[e] = 0.0f;
-            float den = 0.0f;
-            for (int s0 = 0; s0 < NS; s0 += 8) {
-                if (!((live_chunks >> ((s0 >> 3) & 63)) & 1ull)) continue;
-                float mv[8], lv[8];
-                float4v lo[8], hi[8];
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    const int sidx = s0 + k < NS ? s0 + k : NS - 1;
-                    mv[k] = part_m[base + sidx];
-                    lv[k] = part_l[base + sidx];
-                    // An empty split (m = -inf) never wrote its accumulator; it is read all the same
-                    // (and ignored below), so that no load has to wait for another one.
-                    const float4v* src = reinterpret_cast<const float4v*>(part_acc + (base + sidx) * D + c0);
-                    lo[k] = src[0];
-                    hi[k] = src[1];
-                }
-                if (NS <= 8) {
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) {
-                        mstar = __builtin_fmaxf(mstar, mv[k]);
-                        poisoned = poisoned || mv[k] != mv[k];
-                    }
-                }
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    const bool use = s0 + k < NS && mv[k] != -__builtin_inff();
-                    const float w = use ? __builtin_amdgcn_exp2f(mv[k] - mstar) : 0.0f;
-                    den = __builtin_fmaf(lv[k], w, den);
-                    // a weight of 0 must also silence a NaN or Inf in memory that no split wrote
-                    num[0] = use ? __builtin_fmaf(lo[k].x, w, num[0]) : num[0]; num[1] = use ? __builtin_fmaf(lo[k].y, w, num[1]) : num[1];
-                    num[2] = use ? __builtin_fmaf(lo[k].z, w, num[2]) : num[2]; num[3] = use ? __builtin_fmaf(lo[k].w, w, num[3]) : num[3];
-                    num[4] = use ? __builtin_fmaf(hi[k].x, w, num[4]) : num[4]; num[5] = use ? __builtin_fmaf(hi[k].y, w, num[5]) : num[5];
-                    num[6] = use ? __builtin_fmaf(hi[k].z, w, num[6]) : num[6]; num[7] = use ? __builtin_fmaf(hi[k].w, w, num[7]) : num[7];
-                }
-            }
-            const bool live = row0 + r < rows && den > 0.0f;
-            uint32_t wds[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                // a poisoned row comes out NaN, never as a plausible number
-                const uint32_t a0 = poisoned ? store_elem<DT>(__builtin_nanf("")) : (live ? store_elem<DT>(num[2 * e] / den) : 0u);
-                const uint32_t a1 = poisoned ? store_elem<DT>(__builtin_nanf("")) : (live ? store_elem<DT>(num[2 * e + 1] / den) : 0u);
-                wds[e] = a0 | (a1 << 16);
-            }
-            *reinterpret_cast<uint4v*>(&os[r * OSTRIDE + c0]) = uint4v{wds[0], wds[1], wds[2], wds[3]};
+        (void)inv;
+        if (t < ACTIVE) {
+            if constexpr (CPT == 2) *reinterpret_cast<uint32_t*>(&os[r * OSTRIDE + c0]) = wds[0];
+            else if constexpr (CPT == 4) *reinterpret_cast<uint2v*>(&os[r * OSTRIDE + c0]) = uint2v{wds[0], wds[1]};
+            else *reinterpret_cast<uint4v*>(&os[r * OSTRIDE + c0]) = uint4v{wds[0], wds[1], wds[2], wds[3]};
         }
     }
     __syncthreads();
     if (R == nullptr) {
-        for (int c = threadIdx.x; c < kRotRows * (D / 8); c += 256) {
-            const int r = c / (D / 8), q = c % (D / 8);
-            const int64_t row = row0 + r;
-            if (row < rows) reinterpret_cast<uint4v*>(out + row * D)[q] = *reinterpret_cast<const uint4v*>(&os[r * OSTRIDE + 8 * q]);
+        for (int c = threadIdx.x; c < RW * (D / 8); c += 256) {
+            const int rr = c / (D / 8), q = c % (D / 8);
+            const int64_t orow = row0 + rr;
+            if (orow < rows) reinterpret_cast<uint4v*>(out + orow * D)[q] = *reinterpret_cast<const uint4v*>(&os[rr * OSTRIDE + 8 * q]);
         }
         return;
     }
-    // ---- rotate back on the fp16 MFMA: the rows are exact in fp16 up to a power of two ----------------
+    // ---- rotate back on the fp16 MFMA: the rows are exact in fp16 up to a power of two.  With fewer
+    // than 16 rows the operand rows repeat (row n % RW) and only the first RW result rows are kept. ----
     uint4v raw[D / 32];
 #pragma unroll
-    for (int j = 0; j < D / 32; ++j) raw[j] = *reinterpret_cast<const uint4v*>(&os[n * OSTRIDE + 32 * j + 8 * g]);
+    for (int j = 0; j < D / 32; ++j) raw[j] = *reinterpret_cast<const uint4v*>(&os[(n % RW) * OSTRIDE + 32 * j + 8 * g]);
     half8 a[D / 32];
     float up;
     rows_as_f16<D, DT>(raw, a, up);
@@ -1659,8 +1587,9 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
         const int cb = wave + 4 * i;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const int64_t row = row0 + 4 * g + k;
-            if (row < rows) out[row * D + 16 * cb + n] = store_elem<DT>(acc[k] * up);
+            const int rr = 4 * g + k;
+            const int64_t orow = row0 + rr;
+            if (rr < RW && orow < rows) out[orow * D + 16 * cb + n] = store_elem<DT>(acc[k] * up);
         }
     }
 }
@@ -1681,14 +1610,6 @@ inline WorkspaceLayout workspace_layout(int S, int H_Q, int D, int NS) {
     return w;
 }
 
-// Launch with `lds` bytes of dynamic LDS; more than 64 KB per workgroup has to be
-// allowed per kernel function first.
-template <typename K>
-int launch_with_lds(K kernel, const DecodeParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
-    if (lds > 32768 && !fq_host::lds_limit_raised(reinterpret_cast<const void*>(kernel), lds)) return FQ_ERR_LAUNCH;
-    hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
-    return fq_host::check_launch();
-}
 
 // Workgroups that run at a time (one per CU) when the staged kernel should size its chunks from
 // the actual sequence lengths, 0 when the fixed chunks already fill the chip in one round or the
@@ -1792,6 +1713,8 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
         ps.balance_slots = staged_balance_slots(S, p.num_splits * groups);
         if (ps.balance_slots > 0) ps.balance_slots = ps.balance_slots / groups > 0 ? ps.balance_slots / groups : 1;
         // a chosen chunk may span up to 256 pages: four page-id registers
+        if (fq_host::option(FQ_OPT_DECODE_RING) != 0)
+            return launch_ring(ps, S, BS, wide || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256), DT, stream);
         return launch_staged_any<DT, false>(ps, S, BS, wide || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256),
                                             stream);
     }
@@ -1845,13 +1768,30 @@ template <int DT>
 int launch_reduce(const float* acc, const float* m, const float* l, const float* R, int col_major, void* out, int S, int H_Q,
                   int D, int NS, hipStream_t stream) {
     const int64_t rows = int64_t(S) * H_Q;
-    const dim3 grid(unsigned((rows + kRotRows - 1) / kRotRows)), block(256);
+    // Rows per workgroup: as few as it takes to put a workgroup on every CU, at most 16.  The rows of a
+    // decode step are few (1024 at 32 sequences x 32 heads) and the kernel is a chain of latencies
+    // (partials, combine, rotate, store), so what counts is how short that chain is per workgroup.
+    const int cus = fq_host::device_cu_count();
+    const int rw_opt = fq_host::option(FQ_OPT_REDUCE_ROWS);
+    int rw = rows <= 4 * int64_t(cus) ? 4 : (rows <= 8 * int64_t(cus) ? 8 : 16);
+    if (rw_opt == 4 || rw_opt == 8 || rw_opt == 16) rw = rw_opt;
+    const dim3 grid(unsigned((rows + rw - 1) / rw)), block(256);
     uint16_t* dst = reinterpret_cast<uint16_t*>(out);
+#define FQ_REDUCE(DD, RWV) \
+    hipLaunchKernelGGL((reduce_rotate_kernel<DD, DT, RWV>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major)
+#define FQ_REDUCE_D(DD)                       \
+    do {                                      \
+        if (rw == 4) FQ_REDUCE(DD, 4);        \
+        else if (rw == 8) FQ_REDUCE(DD, 8);   \
+        else FQ_REDUCE(DD, 16);               \
+    } while (0)
     switch (D) {
-        case 64: hipLaunchKernelGGL((reduce_rotate_kernel<64, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major); break;
-        case 128: hipLaunchKernelGGL((reduce_rotate_kernel<128, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major); break;
-        default: hipLaunchKernelGGL((reduce_rotate_kernel<256, DT>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major); break;
+        case 64: FQ_REDUCE_D(64); break;
+        case 128: FQ_REDUCE_D(128); break;
+        default: FQ_REDUCE_D(256); break;
     }
+#undef FQ_REDUCE_D
+#undef FQ_REDUCE
     return fq_host::check_launch();
 }
 

@@ -62,7 +62,12 @@ typedef enum fq_option {
                                      rotated against the matrix as two bf16 terms (|error| <= 2^-18 per
                                      element: about 6 indices in a million differ from the float32 result);
                                      1: three terms, the float32 matrix exactly, at 3/2 of the matrix work */
-    FQ_OPTION_COUNT = 5
+    FQ_OPT_DECODE_RING = 5,       /* FQ_DECODE_RING, default 0: 1 sends groups of 8 KV heads of dimension 128 to the
+                                     ring decode kernel (16 computing wavefronts, direct-to-LDS loads)
+                                     instead of the staged kernel with copy wavefronts                    */
+    FQ_OPT_REDUCE_ROWS = 6,       /* FQ_REDUCE_ROWS, default 0: rows per workgroup of the combine kernel chosen from
+                                     the row count; 4, 8 or 16 forces that many                          */
+    FQ_OPTION_COUNT = 7
 } fq_option;
 int fq_get_option(int option);
 int fq_set_option(int option, int value);

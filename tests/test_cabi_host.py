@@ -244,11 +244,15 @@ def test_static_scratch_decode_refuses_before_touching_the_gpu(lib):
 
 def test_option_switches(lib):
     assert lib.fq_get_option(99) == -1 and lib.fq_set_option(99, 1) == FQ_SHAPE
-    for opt in range(5):
+    for opt in range(6):
         old = lib.fq_get_option(opt)
         assert old in (0, 1)
         assert lib.fq_set_option(opt, 1 - old) == FQ_OK and lib.fq_get_option(opt) == 1 - old
         assert lib.fq_set_option(opt, old) == FQ_OK and lib.fq_get_option(opt) == old
+    # rows per workgroup of the combine kernel: a number, not a switch
+    assert lib.fq_get_option(6) == 0
+    assert lib.fq_set_option(6, 8) == FQ_OK and lib.fq_get_option(6) == 8
+    assert lib.fq_set_option(6, 0) == FQ_OK and lib.fq_get_option(6) == 0
 
 
 def test_shape_limits_of_the_staged_and_prod_decodes(lib):

@@ -268,9 +268,40 @@ def test_paged_decode_split_counts_beyond_64(num_splits):
 
 @pytest.mark.parametrize("hq,bs", [(32, 16), (64, 8), (128, 32)])
 def test_paged_decode_without_copy_wavefronts(hq, bs, kernel_option):
-    """Switch decode_copy_waves off: the eight wavefronts of the staged kernel copy and compute in turn."""
+    """Switches decode_copy_waves off: the eight wavefronts of the staged kernel copy and compute in turn."""
     kernel_option("decode_copy_waves", False)
     _decode_case([37, 0, 16, 300, 64, 65, 1, 129], hq=hq, hkv=8, bs=bs, num_splits=3)
+
+
+@pytest.mark.parametrize("hq,hkv,bs,dtype", [(32, 8, 16, torch.bfloat16), (64, 8, 8, torch.float16), (128, 8, 32, torch.bfloat16),
+                                             (32, 16, 16, torch.bfloat16), (48, 24, 32, torch.float16)])
+def test_paged_decode_ring_kernel(hq, hkv, bs, dtype, kernel_option):
+    """Switch decode_ring on: groups of 8 KV heads run the ring kernel (16 computing wavefronts, token
+    rows loaded straight into LDS) instead of the staged one; same cases, same oracle, and the two
+    kernels agree."""
+    for lens, splits in (([37, 0, 16, 300, 64, 65, 1, 129], 3), ([1500, 0, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0)):
+        kernel_option("decode_ring", True)
+        _decode_case(lens, hq=hq, hkv=hkv, bs=bs, num_splits=splits, dtype=dtype)
+        kernel_option("decode_ring", False)
+        _decode_case(lens, hq=hq, hkv=hkv, bs=bs, num_splits=splits, dtype=dtype)
+
+
+def test_paged_decode_ring_kernel_two_codebooks_and_prerotated_query(kernel_option):
+    """The ring kernel with a value codebook of its own, and through the partials entry point with a
+    query that is already rotated."""
+    kernel_option("decode_ring", True)
+    C = load_native()
+    c, b, r = book(128)
+    cv = (c * 1.25).contiguous()
+    q, cache, table, sl = build_paged_case([300, 17, 1000], 32, 8, seed=77)
+    want = O.split_k_paged_decode(q, cache, table, sl, c, cv, r, 8, 128, 16)
+    dev = [t.to(DEV) for t in (q, cache, table, sl, c, cv, r)]
+    got = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[5], dev[6], 8, 128, 16, num_splits=4)
+    assert (got.cpu().float() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
+    q_rot = (q.float() @ r.T).to(q.dtype).to(DEV)
+    acc, m, l = C.paged_tq4_decode_partials(q_rot, dev[1], dev[2], dev[3], dev[4], dev[5], 8, 128, 16, 1.0 / math.sqrt(128), 4)
+    out = C.split_k_reduce(acc, m, l, dev[6], q.dtype)
+    assert (out.cpu().float() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
 
 
 def test_prod_paged_decode_without_copy_wavefronts(kernel_option):
