@@ -10,8 +10,9 @@ launch of this library:
   prefill              _tq4_prefill + flash_attn_varlen_func + post-rotation, impl.py:317-336, 470-512
   decompress_cache     _decompress_cache, impl.py:265-318
 
-A backend written against vLLM calls these from its ``forward`` with the fields of its attention
-metadata; nothing here imports vLLM."""
+``get_flashquant_impl_class`` builds ``FlashQuantAttentionImpl``, the subclass of vLLM's
+FlashAttentionImpl whose ``forward`` is these launches (needs vLLM, imported on first use); the rest
+of the module imports without it."""
 from __future__ import annotations
 
 from typing import Optional, Tuple
@@ -88,3 +89,60 @@ class TQ4AttentionKernels:
             key_out = C.tq4_decompress(k_packed, k_norms, self.centroids, compute_dtype, out_k)
             value_out = C.tq4_decompress(v_packed, v_norms, self.centroids, compute_dtype, out_v)
         return key_out.reshape(nb, bs, h, d), value_out.reshape(nb, bs, h, d)
+
+
+_impl_class = None
+
+
+def _make_impl_class() -> type:
+    from vllm.v1.attention.backends.flash_attn import FlashAttentionImpl
+
+    class FlashQuantAttentionImpl(FlashAttentionImpl):  # type: ignore[misc, valid-type]
+        """forward(): store the new tokens in the packed cache, then attend straight from it.
+
+        Where the reference decompresses the whole cache and hands it to a FlashAttention library
+        (src/flashquant/vllm/impl.py:395-512), a batch of single-token queries runs the split-K paged
+        decode and everything else the paged prefill, both reading the packed pages; neither
+        allocates, so a decode step can be captured in a graph."""
+
+        def __init__(self, *args, **kwargs) -> None:
+            super().__init__(*args, **kwargs)
+            from vllm.config import get_current_vllm_config_or_none
+            cfg = get_current_vllm_config_or_none()
+            device = cfg.device_config.device if cfg is not None else torch.device("cuda")
+            self._tq4 = TQ4AttentionKernels(self.num_kv_heads, self.head_size, self.scale, device)
+
+        def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None, output_scale=None,
+                    output_block_scale=None):
+            if output is None:
+                raise ValueError("FlashQuantAttentionImpl needs a pre-allocated output")
+            if output_scale is not None or output_block_scale is not None:
+                raise NotImplementedError("fused output quantisation is not supported by the FlashQuant backend")
+            if attn_metadata is None:                       # profiling run
+                output.zero_()
+                return output
+            from vllm.v1.attention.backend import AttentionType
+            n = attn_metadata.num_actual_tokens
+            if self.attn_type in (AttentionType.ENCODER_ONLY, AttentionType.ENCODER):
+                return self._forward_encoder_attention(query[:n], key[:n], value[:n], output[:n], attn_metadata, layer)
+            if getattr(attn_metadata, "use_cascade", False):
+                raise NotImplementedError("cascade attention is not supported by the FlashQuant backend")
+            if key is not None and value is not None:
+                self._tq4.compress_and_store(key, value, kv_cache, attn_metadata.slot_mapping)
+            if attn_metadata.max_query_len == 1:
+                self._tq4.decode(query[:n], kv_cache, attn_metadata.block_table, attn_metadata.seq_lens, out=output[:n])
+            else:
+                self._tq4.prefill(query[:n], attn_metadata.query_start_loc, attn_metadata.max_query_len, kv_cache,
+                                  attn_metadata.block_table, attn_metadata.seq_lens, out=output[:n],
+                                  causal=getattr(attn_metadata, "causal", True))
+            return output
+
+    return FlashQuantAttentionImpl
+
+
+def get_flashquant_impl_class() -> type:
+    """FlashQuantAttentionImpl, created on first call (needs vLLM)."""
+    global _impl_class
+    if _impl_class is None:
+        _impl_class = _make_impl_class()
+    return _impl_class
