@@ -111,19 +111,37 @@ def time_region(fn, iters):
     return first.elapsed_time(last) / iters
 
 
-def committed_traffic(kernel_prefix):
-    """HBM bytes per launch of the dominant kernel as the committed counter summary states them
-    (a line `TRAFFIC_BYTES_PER_LAUNCH <kernel> <bytes>` in profiles/paged_decode_hbm_traffic_pmc.txt,
-    written from the FETCH_SIZE / WRITE_SIZE runs); None when the summary does not cover the kernel."""
-    path = os.path.join(ROOT, "profiles", "paged_decode_hbm_traffic_pmc.txt")
+def committed_traffic(kernel):
+    """HBM bytes per launch of the dominant kernel as the committed counter summary states them (a line
+    `TRAFFIC_BYTES_PER_LAUNCH <kernel> <bytes>` in profiles/paged_decode_hbm_traffic_pmc.txt, written from
+    FETCH_SIZE / WRITE_SIZE runs), with where the figure comes from: the file, a hash of its bytes and
+    the kernel it names.  The figure is None, and `stale` says why, when the summary names another kernel
+    than the one this run times: a committed number is only as fresh as the profile it was read from."""
+    import hashlib
+    rel = os.path.join("profiles", "paged_decode_hbm_traffic_pmc.txt")
+    src = {"file": rel, "sha256_16": None, "kernel_in_file": None, "stale": None}
     try:
-        for ln in open(path):
-            parts = ln.split()
-            if len(parts) == 3 and parts[0] == "TRAFFIC_BYTES_PER_LAUNCH" and parts[1].startswith(kernel_prefix):
-                return float(parts[2])
+        raw = open(os.path.join(ROOT, rel), "rb").read()
     except OSError:
-        pass
-    return None
+        src["stale"] = "summary file missing"
+        return None, src
+    src["sha256_16"] = hashlib.sha256(raw).hexdigest()[:16]
+    for ln in raw.decode().splitlines():
+        parts = ln.split()
+        if len(parts) == 3 and parts[0] == "TRAFFIC_BYTES_PER_LAUNCH":
+            src["kernel_in_file"] = parts[1]
+            if parts[1] == kernel:
+                return float(parts[2]), src
+    src["stale"] = f"the summary does not cover {kernel}"
+    return None, src
+
+
+def output_ulps(err, want, dtype):
+    """|err| in units in the last place of the output dtype at the magnitude of the expected value."""
+    mant = 7 if dtype == torch.bfloat16 else 10
+    mag = want.abs().clamp_min(2.0 ** -14)
+    ulp = torch.exp2(torch.floor(torch.log2(mag)) - mant)
+    return (err / ulp).max().item()
 
 
 def main():
@@ -174,6 +192,16 @@ def main():
         K.split_k_paged_decode(q, cache, table, lens, cent_d, cent_d, rot_d, H_KV, D, BS,
                                sm_scale=scale, out=out)
 
+    # Untimed, before the W warm-up steps: a quarter of a second of the same steps.  The GPU's clocks take
+    # some tens of milliseconds of work to come up from idle (the first few hundred 40 us steps after a
+    # pause run 10-25 % slower than the following ones), which W = 20 steps do not cover.
+    t_ramp = time.perf_counter()
+    i_ramp = 0
+    while time.perf_counter() - t_ramp < 0.25:
+        for _ in range(50):
+            step(i_ramp)
+            i_ramp += 1
+        torch.cuda.synchronize()
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -182,9 +210,12 @@ def main():
         step(i)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    # the figure reported: the median over the steps of the GPU time of one step
-    step_ms, step_mean_ms = time_events(step, args.steps)
-    warm_ms, _ = time_events(lambda i: step(0), args.steps)
+    # The figure reported: exactly K steps back to back between two GPU events, synchronised on both
+    # sides, divided by K (the host-side wall clock around the same loop is reported next to it: it
+    # also holds what the host needs to issue a step).
+    step_ms = time_region(step, args.steps)
+    step_median_ms, step_mean_ms = time_events(step, args.steps)
+    warm_ms = time_region(lambda i: step(0), args.steps)
 
     # ---- dominant kernel alone (the split-K decode), cold ----------------------------
     parts = (torch.empty(BATCH, H_Q, n_splits, D, device=dev), torch.empty(BATCH, H_Q, n_splits, device=dev),
@@ -204,6 +235,7 @@ def main():
     extra = {
         "decode_tokens_per_s": BATCH / (step_ms * 1e-3),
         "decode_step_us_cold": step_ms * 1e3,
+        "decode_step_us_cold_event_median": step_median_ms * 1e3,
         "decode_step_us_warm": warm_ms * 1e3,
         "decode_step_us_wallclock": wall_ms * 1e3,
         "decode_step_us_cold_mean": step_mean_ms * 1e3,
@@ -235,6 +267,7 @@ def main():
         got = K.split_k_paged_decode(q, cache0, table0, lens, cent_d, cent_d, rot_d, H_KV, D, BS,
                                      sm_scale=scale).float().cpu()
         done, spent, worst, worst_abs = 0, 0.0, 0.0, 0.0
+        n_elems, n_flat, worst_ulps = 0, 0, 0.0
         while spent < 10.0 and done < 40 * BATCH:      # about 10 s of CPU work, whole sequences
             s_i = done % BATCH
             t1 = time.perf_counter()
@@ -248,6 +281,11 @@ def main():
             row_scale = w_f.abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
             worst = max(worst, ((got[s_i] - w_f).abs() / row_scale).max().item())
             worst_abs = max(worst_abs, (got[s_i] - w_f).abs().max().item())
+            if done <= BATCH:
+                err = (got[s_i] - w_f).abs()
+                n_elems += err.numel()
+                n_flat += int((err <= 2e-2).sum().item())
+                worst_ulps = max(worst_ulps, output_ulps(err, w_f, q.dtype))
         # the reference's CPU fallback as written, a Python loop over tokens and heads, at a reduced shape
         lb, ll = 2, 512
         lens_l = torch.full((lb,), ll, dtype=torch.int32)
@@ -276,6 +314,10 @@ def main():
         check = {
             "max_err_of_row_magnitude": worst, "max_abs_err": worst_abs, "sequences_checked": min(done, BATCH),
             "tolerance": "2e-2 of the row's largest |x|, at least 2e-2 absolute",
+            # the same errors read without the scaling: the share of the output elements within a flat
+            # 2e-2, and the largest error in units in the last place of the bfloat16 output
+            "share_within_flat_2e-2": n_flat / max(n_elems, 1),
+            "max_err_ulps_of_output_dtype": worst_ulps,
             "loop_form_max_abs_err": worst_l, "ok": bool(worst <= 2e-2 and worst_l <= 2e-2),
         }
         del cache_h
@@ -547,6 +589,7 @@ def main():
             extra["other_shapes"] = shapes
 
     value = kv_bytes / (step_ms * 1e-3) / 1e9
+    traffic, traffic_src = committed_traffic(DOMINANT_KERNEL)
     line = {
         "metric": "tq4_paged_decode_hbm_gbps",
         "value": value,
@@ -573,14 +616,21 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a plain copy, as the
             # committed counter summary states them for this kernel (null when it does not cover it)
-            "traffic": committed_traffic(DOMINANT_KERNEL),
+            "traffic": traffic,
+            "traffic_source": traffic_src,
             "kernel": DOMINANT_KERNEL,
         },
         "cpu_baseline": cpu,
         "check": check,
+        "check_ok": None if check is None else check["ok"],
+        "check_max_abs_err": None if check is None else check["max_abs_err"],
+        "decode_step_us_wallclock": wall_ms * 1e3,
         "extra": extra,
     }
     print(json.dumps(line), flush=True)
+    if check is not None and not check["ok"]:
+        log("bench.py: the output check against the oracle FAILED:", json.dumps(check))
+        sys.exit(1)
 
 
 if __name__ == "__main__":

@@ -194,6 +194,113 @@ def test_prod_paged_decode_on_long_ragged_contexts():
     assert math.isfinite(err) and err <= 2e-2, f"max abs error {err}"
 
 
+def test_prod_paged_decode_at_the_benchmark_batch():
+    """The long-context workload at its real batch: 8 sequences, lengths drawn uniformly from 16K to
+    128K tokens with seed 1004, 64 query heads over 8 KV heads, N(0,1) rows with outlier channels.
+    The pages are written by the library's own TurboQuantProd compress (covered against the oracle
+    elsewhere); the decode of every sequence runs in one call, and three of the eight (the shortest,
+    the longest and one in between) are checked against the oracle on the same pages."""
+    from tests.conftest import outlier_rows as rows_cpu
+    c3, b3 = O.lloyd_max_gaussian(128, 3)
+    c4, b4 = O.lloyd_max_gaussian(128, 4)
+    r, s = O.haar_orthogonal(128, 42), O.qjl_matrix(128, 42)
+    hq, hkv, d, bs, nseq = 64, 8, 128, 16, 8
+    g = torch.Generator(device="cpu").manual_seed(1004)
+    lens = torch.randint(16384, 131072 + 1, (nseq,), generator=g)
+    pages = (lens + bs - 1) // bs
+    total_pages, max_pages = int(pages.sum()), int(pages.max())
+    row_bytes = K.prod_page_layout(hkv, d)[4]
+    cache = torch.zeros(total_pages, bs, row_bytes, dtype=torch.uint8, device=DEV)
+    perm = torch.randperm(total_pages, generator=g)
+    table = torch.zeros(nseq, max_pages, dtype=torch.int32)
+    rd, sd, b3d, c3d, b4d = r.to(DEV), s.to(DEV), b3.to(DEV), c3.to(DEV), b4.to(DEV)
+    first = 0
+    for i in range(nseq):
+        L, npg = int(lens[i]), int(pages[i])
+        table[i, :npg] = perm[first:first + npg].int()
+        first += npg
+        t = torch.arange(L)
+        slots = (table[i].long()[t // bs] * bs + t % bs).to(DEV)
+        for t0 in range(0, L, 32768):                       # bounded memory
+            n = min(32768, L - t0)
+            kx = rows_cpu(n, hkv, d, 1400 + 16 * i + t0 // 32768).to(torch.bfloat16).to(DEV)
+            vx = rows_cpu(n, hkv, d, 1500 + 16 * i + t0 // 32768).to(torch.bfloat16).to(DEV)
+            kp, kn, kg = K.prod_compress(kx, rd, sd, b3d, c3d)
+            vp, vn = K.tq4_compress(vx, rd, b4d)
+            K.prod_store_rows(cache, slots[t0:t0 + n], kp, kn, kg, vp, vn)
+    q = torch.randn(nseq, hq, d, generator=g).to(torch.bfloat16)
+    sl = lens.to(torch.int32)
+    got = K.prod_paged_decode(q.to(DEV), cache, table.to(DEV), sl.to(DEV), c3d, c4.to(DEV), rd, sd, hkv, d, bs)
+    torch.cuda.synchronize()
+    got = got.cpu().float()
+    assert torch.isfinite(got).all()
+    cache_h = cache.cpu()
+    order = torch.argsort(lens)
+    for i in (int(order[0]), int(order[nseq // 2]), int(order[-1])):
+        want = O.prod_paged_decode(q[i:i + 1], cache_h, table[i:i + 1], sl[i:i + 1], c3, c4, r, s, hkv, d, bs)
+        # outlier channels push some output rows past |x| = 4, where one bfloat16 step is 0.03: 2e-2 of
+        # the row's magnitude (never less than 2e-2 absolute), as for the TQ4 decode above
+        row_scale = want[0].float().abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+        rel = ((got[i] - want[0].float()).abs() / row_scale).max().item()
+        assert rel <= 2e-2, f"sequence {i} of {int(lens[i])} tokens: max error {rel} of the row magnitude"
+
+
+def test_compress_at_the_benchmark_size():
+    """The standalone compress workload at full size: 32 layers x 65,536 tokens x 8 KV heads = 16,777,216
+    bfloat16 rows of 128 coordinates (N(0,1) with four x10 outlier channels per head), one call.
+    Properties over every row, computed on the GPU with torch: the stored norms equal torch's norms of
+    the rows, the rows come back from decompress + rotation with the relative squared error of a
+    16-level Lloyd-Max quantiser (0.0095) and no row is off by more than what a 4-bit code allows.
+    Against the oracle on a sample of 1,048,576 rows spread over the input: index mismatches on at most
+    1e-4 of the entries, packing bit-exact given the indices, norms to 1e-6."""
+    c, b, r = book(128)
+    hkv, d = 8, 128
+    n_tok = 32 * 65536
+    x = torch.empty(n_tok, hkv, d, dtype=torch.bfloat16, device=DEV)
+    chunk = 262144
+    gd = torch.Generator(device=DEV).manual_seed(1001)
+    gc = torch.Generator().manual_seed(1001)
+    chans = [torch.randperm(d, generator=gc)[:4].to(DEV) for _ in range(hkv)]
+    for t0 in range(0, n_tok, chunk):
+        xf = torch.randn(chunk, hkv, d, generator=gd, device=DEV)
+        for h in range(hkv):
+            xf[:, h, chans[h]] *= 10.0
+        x[t0:t0 + chunk] = xf.to(torch.bfloat16)
+    rd, bd, cd = r.to(DEV), b.to(DEV), c.to(DEV)
+    packed, norms = K.tq4_compress(x, rd, bd)
+    torch.cuda.synchronize()
+    assert packed.shape == (n_tok, hkv, d // 2) and norms.shape == (n_tok, hkv, 1)
+    worst_norm, err_sq, ref_sq, worst_row = 0.0, 0.0, 0.0, 0.0
+    for t0 in range(0, n_tok, chunk):
+        xs = x[t0:t0 + chunk].float()
+        want_n = xs.norm(dim=-1, keepdim=True)
+        got_n = norms[t0:t0 + chunk]
+        worst_norm = max(worst_norm, ((got_n - want_n).abs() / want_n.clamp_min(1e-30)).max().item())
+        back = K.tq4_decompress_rotated(packed[t0:t0 + chunk], got_n, cd, rd, torch.bfloat16).float()
+        e = ((back - xs) ** 2).sum(dim=-1)
+        err_sq += e.sum().item()
+        ref_sq += (xs ** 2).sum().item()
+        worst_row = max(worst_row, (e / (xs ** 2).sum(dim=-1).clamp_min(1e-30)).max().item())
+    assert worst_norm <= 1e-5, worst_norm
+    rel = err_sq / ref_sq
+    assert 0.0085 <= rel <= 0.0105, rel
+    assert worst_row <= 0.1, worst_row
+    # the oracle on 16 slices of 8192 tokens (x 8 heads = 1,048,576 rows)
+    mismatched, entries = 0, 0
+    for k in range(16):
+        t0 = k * (n_tok // 16) + 4099 * k
+        xs = x[t0:t0 + 8192].cpu()
+        idx_want, norms_want, _ = O.compress_indices(xs, r, b)
+        got_p = packed[t0:t0 + 8192].cpu()
+        idx_got = O.nibble_unpack(got_p)
+        mismatched += int((idx_got != idx_want).sum().item())
+        entries += idx_want.numel()
+        assert torch.equal(O.nibble_pack(idx_got), got_p)
+        assert ((norms[t0:t0 + 8192].cpu() - norms_want).abs() / norms_want.clamp_min(1e-30)).max().item() <= 1e-6
+    assert entries == 1048576 * d
+    assert mismatched / entries <= 1e-4, mismatched / entries
+
+
 # ---- magnitudes of the reference's adversarial tests, through decode and prefill ------------------
 
 def _adversarial_rows(kind, n, h, d, seed):
