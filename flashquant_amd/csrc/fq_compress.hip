@@ -737,6 +737,8 @@ extern "C" int fq_tq4_compress(const void* x, int x_dtype, const float* rot_T_ev
 #undef FQ_COMPRESS_CASE
 }
 
+// Shares the compress kernel, and so its rotation precision: bf16 rows of head_dim 64 / 128 against two
+// bf16 terms of the matrix unless FQ_OPT_COMPRESS_THREE_TERMS asks for the third (compress_matrix_terms).
 extern "C" int fq_tq4_compress_append(const void* x, int x_dtype, const float* rot_T_even, const float* rot_T_odd,
                                       const float* boundaries, uint8_t* packed, float* norms, int64_t outer,
                                       int64_t n_new, int64_t capacity, int64_t position, int D, void* stream) {
@@ -770,6 +772,8 @@ extern "C" int fq_tq4_compress_append(const void* x, int x_dtype, const float* r
 #undef FQ_APPEND_CASE
 }
 
+// Rotation precision as in fq_tq4_compress: two bf16 matrix terms by default for bf16 rows of head_dim
+// 64 / 128, three with FQ_OPT_COMPRESS_THREE_TERMS (compress_matrix_terms).
 extern "C" int fq_tq4_compress_store(const void* key, const void* value, int x_dtype,
                                      const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
                                      uint8_t* kv_cache, const int64_t* slot_mapping,

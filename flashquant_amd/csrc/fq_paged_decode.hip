@@ -59,9 +59,6 @@
 #include "fq_paged_decode.hpp"
 
 namespace fq_host {
-// The switch FQ_OPT_DECODE_DIRECT routes every shape to the direct kernel (both kernels are kept
-// tested).
-bool force_direct_decode();
 int device_cu_count();
 }
 
@@ -1619,9 +1616,26 @@ inline int staged_balance_slots(int num_seqs, int num_splits) {
     return (num_seqs <= 64 && int64_t(num_seqs) * num_splits > cus) ? cus : 0;
 }
 
+// The kernel-variant switches as one decode call sees them.  They are process-wide and may be changed
+// by another thread at any time (fq_set_option): a call reads them once, here, and everything that
+// depends on them (which kernel runs, how many partials it writes, how the workspace is laid out, how
+// many the combine kernel merges) is derived from this one reading.
+struct DecodeVariant {
+    bool direct;        // FQ_OPT_DECODE_DIRECT
+    bool ring;          // FQ_OPT_DECODE_RING
+    int copy_waves;     // 4 or 0 (FQ_OPT_DECODE_COPY_WAVES)
+};
+inline DecodeVariant read_decode_variant() {
+    DecodeVariant v;
+    v.direct = fq_host::option(FQ_OPT_DECODE_DIRECT) != 0;
+    v.ring = fq_host::option(FQ_OPT_DECODE_RING) != 0;
+    v.copy_waves = fq_host::option(FQ_OPT_DECODE_COPY_WAVES) != 0 ? 4 : 0;
+    return v;
+}
+
 // The staged kernel covers KV heads of dimension 128 in groups of 8.
-inline bool staged_applies(int D, int H_KV) {
-    return D == 128 && H_KV >= 8 && H_KV % 8 == 0 && !fq_host::force_direct_decode();
+inline bool staged_applies(int D, int H_KV, const DecodeVariant& v) {
+    return D == 128 && H_KV >= 8 && H_KV % 8 == 0 && !v.direct;
 }
 
 template <bool PROD, typename K>
@@ -1633,16 +1647,15 @@ int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream, in
 
 // The staged kernel runs with four more wavefronts that only copy; the switch
 // FQ_OPT_DECODE_COPY_WAVES = 0 selects the form in which the eight wavefronts copy and compute in turn.
-inline int staged_copy_waves() { return fq_host::option(FQ_OPT_DECODE_COPY_WAVES) != 0 ? 4 : 0; }
 
 // Staged kernel for every page size and group size; PROD selects the TurboQuantProd page format.
 template <int DT, bool PROD>
-int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream_t stream) {
+int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream_t stream, int copy_waves) {
 #define FQ_STAGED_GP(BSL, GPV)                                                                                  \
     /* TurboQuantProd pages come with at most 64 query heads (8 per KV head) */                                 \
     if constexpr (PROD && GPV == 16) return FQ_ERR_BAD_SHAPE;                                                   \
     else {                                                                                                      \
-        if (staged_copy_waves() == 4)                                                                           \
+        if (copy_waves == 4)                                                                                    \
             return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4>, p, S, stream, 4) \
                         : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 4>, p, S, stream, 4); \
         return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 0>, p, S, stream) \
@@ -1666,8 +1679,8 @@ int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream
 
 // 4 KV heads of dimension 128 on pages of 16 or 32 tokens: the staged kernel on rows of two tokens
 // (`rows_per_page` = block_size / 2), with its copy wavefronts.
-inline bool staged_half_applies(int D, int H_KV, int block_size) {
-    return D == 128 && H_KV == 4 && block_size >= 16 && !fq_host::force_direct_decode() && staged_copy_waves() == 4;
+inline bool staged_half_applies(int D, int H_KV, int block_size, const DecodeVariant& v) {
+    return D == 128 && H_KV == 4 && block_size >= 16 && !v.direct && v.copy_waves == 4;
 }
 template <int DT>
 int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wide, hipStream_t stream) {
@@ -1689,8 +1702,8 @@ int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wid
 }
 
 template <int D, int DT>
-int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bool allow_half) {
-    if (allow_half && staged_half_applies(D, p.H_KV, BS)) {
+int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bool allow_half, const DecodeVariant& var) {
+    if (allow_half && staged_half_applies(D, p.H_KV, BS, var)) {
         // the kernel counts rows of two tokens: half the page size, chunks of rows
         const int rows_per_page = BS / 2;
         const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
@@ -1706,17 +1719,17 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
     const bool wide = chunk / BS > 64;   // begin is a multiple of 64 tokens, hence page aligned
 
     // four page-id registers also when they can hold the whole block-table row
-    if (staged_applies(D, p.H_KV)) {
+    if (staged_applies(D, p.H_KV, var)) {
         DecodeParams ps = p;
         // every group of 8 heads is a slice of the grid with the same (sequence, split) pairs
         const int groups = p.H_KV / 8;
         ps.balance_slots = staged_balance_slots(S, p.num_splits * groups);
         if (ps.balance_slots > 0) ps.balance_slots = ps.balance_slots / groups > 0 ? ps.balance_slots / groups : 1;
         // a chosen chunk may span up to 256 pages: four page-id registers
-        if (fq_host::option(FQ_OPT_DECODE_RING) != 0)
+        if (var.ring)
             return launch_ring(ps, S, BS, wide || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256), DT, stream);
         return launch_staged_any<DT, false>(ps, S, BS, wide || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256),
-                                            stream);
+                                            stream, var.copy_waves);
     }
 
     const int max_waves = D == 256 ? 4 : 8;
@@ -1829,7 +1842,6 @@ bool lds_limit_raised(const void* kernel, size_t bytes) {
     done[{kernel, dev}] = bytes;
     return true;
 }
-bool force_direct_decode() { return option(FQ_OPT_DECODE_DIRECT) != 0; }
 }
 
 // A split keeps its page ids in at most 4 registers of 64 lanes: it may span at most
@@ -1909,7 +1921,7 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
                     const int32_t* seq_lens, const float* centroids_k, const float* centroids_v, float* partial_acc,
                     float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D, int block_size,
                     int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype, int num_splits,
-                    void* stream, bool allow_half = false) {
+                    void* stream, const DecodeVariant& var, bool allow_half = false) {
     const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
                                        num_splits);
     if (bad != FQ_OK) return bad;
@@ -1935,8 +1947,8 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define FQ_DECODE_D(DD)                                                                 \
     case DD:                                                                            \
-        return dtype == FQ_F16 ? launch_partials<DD, FQ_F16>(p, num_seqs, block_size, s, allow_half) \
-                               : launch_partials<DD, FQ_BF16>(p, num_seqs, block_size, s, allow_half);
+        return dtype == FQ_F16 ? launch_partials<DD, FQ_F16>(p, num_seqs, block_size, s, allow_half, var) \
+                               : launch_partials<DD, FQ_BF16>(p, num_seqs, block_size, s, allow_half, var);
     switch (D) {
         FQ_DECODE_D(64)
         FQ_DECODE_D(128)
@@ -1959,7 +1971,7 @@ extern "C" int fq_paged_decode_fault_count(unsigned int* count) {
 
 extern "C" int fq_paged_decode_fuses_rotation(int D, int H_KV, int shared_codebook) {
     (void)shared_codebook;   // both codebooks fit the kernel's table
-    return fq::staged_applies(D, H_KV) ? 1 : 0;
+    return fq::staged_applies(D, H_KV, fq::read_decode_variant()) ? 1 : 0;
 }
 
 extern "C" int fq_paged_tq4_decode(const void* q, const float* rotation, int rotation_col_major,
@@ -1968,10 +1980,11 @@ extern "C" int fq_paged_tq4_decode(const void* q, const float* rotation, int rot
                                    float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D,
                                    int block_size, int max_blocks_per_seq, int64_t num_blocks, float sm_scale,
                                    int dtype, int num_splits, void* stream) {
-    if (rotation && !fq::staged_applies(D, H_KV)) return FQ_ERR_BAD_SHAPE;
+    const fq::DecodeVariant var = fq::read_decode_variant();      // one reading of the switches per call
+    if (rotation && !fq::staged_applies(D, H_KV, var)) return FQ_ERR_BAD_SHAPE;
     return fq::decode_partials(q, rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k,
                                centroids_v, partial_acc, partial_m, partial_l, num_seqs, H_Q, H_KV, D, block_size,
-                               max_blocks_per_seq, num_blocks, sm_scale, dtype, num_splits, stream);
+                               max_blocks_per_seq, num_blocks, sm_scale, dtype, num_splits, stream, var);
 }
 
 extern "C" int fq_split_k_reduce(const float* partial_acc, const float* partial_m, const float* partial_l,
@@ -2003,8 +2016,11 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     if (!q || !out) return FQ_ERR_NULL_POINTER;
     if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16)) return FQ_ERR_MISALIGNED;
     num_splits = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
+    // One reading of the kernel-variant switches for the whole call: the kernel choice, the number of
+    // partials it writes, the workspace layout and what the combine kernel merges all follow from it.
+    const DecodeVariant var = read_decode_variant();
     // 4 KV heads: the staged kernel reads rows of two tokens and writes one partial per token parity
-    const bool half = staged_half_applies(D, H_KV, block_size);
+    const bool half = staged_half_applies(D, H_KV, block_size, var);
     const int num_partials = half ? 2 * num_splits : num_splits;
     const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_partials);
     if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
@@ -2016,7 +2032,7 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     const void* q_in = q;
     const float* fused_rotation = nullptr;
     if (rotation) {
-        if (centroids_k && (half || staged_applies(D, H_KV))) {
+        if (centroids_k && (half || staged_applies(D, H_KV, var))) {
             fused_rotation = rotation;       // the staged kernel rotates the query in its prologue
         } else {
             const int st = fq_rotate_query(q, rotation, rotation_col_major, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
@@ -2026,7 +2042,7 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     }
     int st = decode_partials(q_in, fused_rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m,
                              l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
-                             num_splits, stream, half);
+                             num_splits, stream, var, half);
     if (st != FQ_OK) return st;
     return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_partials, stream);
 }
@@ -2086,8 +2102,10 @@ extern "C" int fq_split_k_paged_decode_static(const void* q, const uint8_t* kv_c
     if (bad != FQ_OK) return bad;
     if (num_seqs == 0) return FQ_OK;
     const int ns = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
-    // the partials of this launch must fit the array: a larger problem is refused, not truncated
-    const int num_partials = staged_half_applies(D, H_KV, block_size) ? 2 * ns : ns;
+    // the partials of this launch must fit the array: a larger problem is refused, not truncated (room
+    // for the two partials per split of the 4-KV-head staged decode whatever the switches say, as in
+    // fq_paged_decode_workspace_bytes: the call below reads the switches once for itself)
+    const int num_partials = (D == 128 && H_KV == 4 && block_size >= 16) ? 2 * ns : ns;
     if (workspace_layout(num_seqs, H_Q, D, num_partials).total > kStaticScratchBytes) return FQ_ERR_WORKSPACE;
     void* ws = nullptr;
     const int st = static_scratch_address(&ws);
@@ -2145,8 +2163,9 @@ extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, cons
     const int64_t chunk = (((max_ctx + num_splits - 1) / num_splits) + 63) & ~int64_t(63);
     const bool wide = chunk / block_size > 64 || p.balance_slots > 0 ||
                       (max_blocks_per_seq > 64 && max_blocks_per_seq <= 256);
-    const int st = dtype == FQ_F16 ? launch_staged_any<FQ_F16, true>(p, num_seqs, block_size, wide, s)
-                                   : launch_staged_any<FQ_BF16, true>(p, num_seqs, block_size, wide, s);
+    const int copy_waves = read_decode_variant().copy_waves;
+    const int st = dtype == FQ_F16 ? launch_staged_any<FQ_F16, true>(p, num_seqs, block_size, wide, s, copy_waves)
+                                   : launch_staged_any<FQ_BF16, true>(p, num_seqs, block_size, wide, s, copy_waves);
     if (st != FQ_OK) return st;
     return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_splits, stream);
 }

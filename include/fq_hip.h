@@ -46,7 +46,10 @@ typedef enum fq_dtype {
 /*
  * Kernel-variant switches, for tests and measurements.  Each takes its first value from an
  * environment variable that is read once per process; fq_set_option changes it afterwards
- * (value 0 or 1), fq_get_option reads it (-1 for an unknown option).
+ * (value 0 or 1), fq_get_option reads it (-1 for an unknown option).  Every entry point reads the
+ * switches once, when it is called, so one call never mixes two settings; fq_set_option itself is not
+ * ordered against calls running on other host threads, so change a switch only while no other thread
+ * is inside the library.
  */
 typedef enum fq_option {
     FQ_OPT_DECODE_COPY_WAVES = 0, /* FQ_DECODE_COPY_WAVES, default 1: the staged decode kernel runs with
@@ -139,6 +142,16 @@ int fq_project_rows(const void* x, int x_dtype, const float* matrix, int matrix_
  *   packed      (M, D/2) uint8 out, 16-byte aligned: byte j = idx[2j]<<4 | idx[2j+1]
  *   norms       (M,) float32 out
  * D in {64, 128, 256}.  M == 0 is a no-op.
+ *
+ * Precision of the rotation (this entry point, fq_tq4_compress_append and fq_tq4_compress_store
+ * alike).  fp16 rows, and bf16 rows of head_dim 256, are rotated against two fp16 terms of the
+ * matrix (22 bits: the float32 product to within summation order).  bf16 rows of head_dim 64 / 128
+ * are by default rotated against TWO bf16 terms of the matrix (16 bits): a rotated coordinate is
+ * then off by up to 1e-6, and 5 to 7 indices in a million land in the neighbouring bucket of the
+ * reference's float32 result (each such coordinate lies within 2e-6 of a boundary).  The switch
+ * FQ_OPT_COMPRESS_THREE_TERMS (environment FQ_COMPRESS_THREE_TERMS=1) adds the third term: the
+ * float32 matrix exactly, indices equal to the reference's wherever the coordinate is not within
+ * float32 rounding of a boundary, at about 1.2 x the time.
  */
 int fq_tq4_compress(const void* x, int x_dtype,
                     const float* rot_T_even, const float* rot_T_odd,
@@ -155,7 +168,8 @@ int fq_tq4_compress(const void* x, int x_dtype,
  *   packed     (outer, capacity, D/2) uint8 buffer, norms (outer, capacity) float32 buffer;
  *              row (o, t) of x lands in row (o, position + t)
  * position >= 0 and position + n_new <= capacity, else FQ_ERR_BAD_SHAPE (the reference raises
- * on overflow, buffer_pool.py:100-107).
+ * on overflow, buffer_pool.py:100-107).  Rotation precision and its switch: as fq_tq4_compress
+ * (two bf16 matrix terms by default for bf16 rows of head_dim 64 / 128).
  */
 int fq_tq4_compress_append(const void* x, int x_dtype,
                            const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
@@ -175,7 +189,9 @@ int fq_tq4_compress_append(const void* x, int x_dtype,
  *   slot_mapping  (num_mapped,) int64: flat slot of token i; tokens i >= num_mapped are
  *                 not stored (impl.py:259-261).  A negative or out-of-range slot is
  *                 skipped (the reference's index assignment would wrap a negative one).
- * Tokens that map to the same slot race, as they do in the reference.
+ * Tokens that map to the same slot race, as they do in the reference.  Rotation precision and
+ * its switch: as fq_tq4_compress (two bf16 matrix terms by default for bf16 rows of head_dim
+ * 64 / 128).
  */
 int fq_tq4_compress_store(const void* key, const void* value, int x_dtype,
                           const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
@@ -462,7 +478,10 @@ size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_KV, int D,
  * size is refused with FQ_ERR_WORKSPACE.  All calls on one GPU share the array: calls that
  * overlap on one GPU (different streams, different threads) race; calls ordered on one stream
  * do not.  Calls no hipMalloc / hipFree; the first call on a device asks the runtime for the
- * array's address (hipGetSymbolAddress).
+ * array's address (hipGetSymbolAddress) and for the device's properties, and the first launch of
+ * a kernel may make the runtime load its code: make one call on each device before a stream
+ * capture begins (or in any other region where the runtime must not be asked for such things);
+ * later calls on that device only launch kernels.
  */
 #define FQ_STATIC_SCRATCH_BYTES (16u << 20)
 size_t fq_static_scratch_bytes(void);

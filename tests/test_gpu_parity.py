@@ -214,6 +214,36 @@ def test_compress_bf16_two_and_three_matrix_terms(d, kernel_option):
     assert rates[True] <= 5e-6, rates
 
 
+@pytest.mark.parametrize("d", [64, 128])
+def test_compress_three_terms_equals_the_oracle_away_from_ties(d, kernel_option):
+    """With the third matrix term the bf16 rotation is the float32 one up to summation order (rotated
+    coordinates within 1e-6), so every row whose rotated coordinates all lie more than 2e-5 from every
+    boundary must come out with exactly the oracle's indices: through the plain compress and through
+    the fused compress-and-store, which share the kernel body."""
+    c, b, r = book(d)
+    h = 8
+    x = outlier_rows(4096, h, d, seed=78, dtype=torch.bfloat16)
+    idx_want, norms_want, y = O.compress_indices(x, r, b)
+    clear = ((y.unsqueeze(-1) - b).abs().min(dim=-1).values > 2e-5).all(dim=-1)       # (tokens, heads)
+    assert clear.float().mean() > 0.5
+    kernel_option("compress_three_terms", True)
+    packed, norms = K.tq4_compress(x.to(DEV), r.to(DEV), b.to(DEV))
+    idx_got = O.nibble_unpack(packed.cpu())
+    assert torch.equal(idx_got[clear], idx_want[clear])
+    assert ((norms.cpu() - norms_want).abs() / norms_want).max() < 2e-6
+    # the same rows through the paged store: key and value slabs of every stored token
+    n, bs = x.shape[0], 16
+    cache = torch.zeros(n // bs, bs, h * (d + 8), dtype=torch.uint8, device=DEV)
+    slots = torch.randperm(n, generator=torch.Generator().manual_seed(79)).long()
+    K.tq4_compress_and_store(x.to(DEV), x.flip(0).contiguous().to(DEV), r.to(DEV), b.to(DEV), cache, slots.to(DEV))
+    rows = cache.cpu().reshape(n, h * (d + 8))[slots]                                   # row of token i
+    half = h * (d // 2 + 4)
+    k_idx = O.nibble_unpack(rows[:, :h * (d // 2)].reshape(n, h, d // 2))
+    v_idx = O.nibble_unpack(rows[:, half:half + h * (d // 2)].reshape(n, h, d // 2))
+    assert torch.equal(k_idx[clear], idx_want[clear])
+    assert torch.equal(v_idx.flip(0)[clear], idx_want[clear])
+
+
 def test_compress_out_buffers_and_presplit_rotation():
     c, b, r = book(128)
     x = outlier_rows(33, 8, 128, seed=9, dtype=torch.bfloat16)
