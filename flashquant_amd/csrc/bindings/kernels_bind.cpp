@@ -248,7 +248,7 @@ at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache,
                                 const at::Tensor& centroids_v, const std::optional<at::Tensor>& rotation,
                                 int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
                                 std::optional<double> sm_scale, const std::optional<at::Tensor>& out,
-                                int64_t num_splits) {
+                                int64_t num_splits, const std::optional<at::Tensor>& workspace) {
     fqbind::require_gpu(q, "q");
     fqbind::require_gpu(kv_cache, "kv_cache");
     require(q.dim() == 3 && q.size(2) == head_dim, "q must have shape (num_seqs, H_Q, D)");
@@ -288,12 +288,20 @@ at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache,
     const int max_blocks = int(bt.size(1));
     const size_t ws_bytes = fq_paged_decode_workspace_bytes(S, HQ, int(num_kv_heads), D, int(block_size), max_blocks,
                                                             int(num_splits));
-    at::Tensor ws = at::empty({int64_t(ws_bytes)}, q.options().dtype(at::kByte));
+    at::Tensor ws;
+    if (workspace.has_value()) {      // the caller's scratch (any contents): nothing is allocated for it here
+        ws = *workspace;
+        require(ws.is_cuda() && ws.device() == q.device() && ws.is_contiguous() && ws.scalar_type() == at::kByte &&
+                    size_t(ws.numel()) >= ws_bytes,
+                "workspace must be a contiguous uint8 GPU tensor of at least paged_decode_workspace_bytes(...) bytes");
+    } else {
+        ws = at::empty({int64_t(ws_bytes)}, q.options().dtype(at::kByte));
+    }
     const int st = fq_split_k_paged_decode(
         qc.data_ptr(), kv_cache.data_ptr<uint8_t>(), bt.data_ptr<int32_t>(), sl.data_ptr<int32_t>(),
         ck.data_ptr<float>(), cv.data_ptr<float>(), rot.ptr, rot.col_major, result.data_ptr(),
         S, HQ, int(num_kv_heads), D, int(block_size), max_blocks, kv_cache.size(0), float(scale),
-        fqbind::dtype_code(q.scalar_type(), "split_k_paged_decode"), int(num_splits), ws.data_ptr(), ws_bytes,
+        fqbind::dtype_code(q.scalar_type(), "split_k_paged_decode"), int(num_splits), ws.data_ptr(), size_t(ws.numel()),
         fqbind::current_stream(q));
     fqbind::raise_on_error(st, "split_k_paged_decode");
     return result;
@@ -728,8 +736,9 @@ void bind_kernels(py::module_& m) {
     m.def("split_k_paged_decode", &split_k_paged_decode, py::arg("q"), py::arg("kv_cache"), py::arg("block_table"),
           py::arg("seq_lens"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),
-          py::arg("out") = py::none(), py::arg("num_splits") = 0,
-          "Split-K paged decode from the packed TQ4 cache; q un-rotated, result in the original space.");
+          py::arg("out") = py::none(), py::arg("num_splits") = 0, py::arg("workspace") = py::none(),
+          "Split-K paged decode from the packed TQ4 cache; q un-rotated, result in the original space.  "
+          "`workspace`: optional uint8 GPU scratch of paged_decode_workspace_bytes(...) bytes, contents arbitrary.");
     // Same operator under the name the vLLM attention impl looks for
     // (src/flashquant/vllm/impl.py:57-59, called with sm_scale= and out= keywords).
     m.def("split_k_paged_decode_static", &split_k_paged_decode_static, py::arg("q"), py::arg("kv_cache"),
@@ -745,7 +754,7 @@ void bind_kernels(py::module_& m) {
     m.def("fused_paged_tq4_decode", &split_k_paged_decode, py::arg("q"), py::arg("kv_cache"), py::arg("block_table"),
           py::arg("seq_lens"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),
-          py::arg("out") = py::none(), py::arg("num_splits") = 0,
+          py::arg("out") = py::none(), py::arg("num_splits") = 0, py::arg("workspace") = py::none(),
           "Alias of split_k_paged_decode.");
     m.def("fused_tq_attention", &fused_tq_attention, py::arg("q"), py::arg("k_packed"), py::arg("k_norms"),
           py::arg("v_packed"), py::arg("v_norms"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),

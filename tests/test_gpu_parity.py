@@ -334,6 +334,22 @@ def test_paged_decode_ring_kernel_two_codebooks_and_prerotated_query(kernel_opti
     assert (out.cpu().float() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
 
 
+def test_paged_decode_on_a_caller_workspace_with_arbitrary_contents():
+    """The caller's scratch is used as it comes: full of 0xff bytes, then with what the call before left."""
+    C = load_native()
+    c, b, r = book(128)
+    q, cache, table, sl = build_paged_case([300, 17, 1000, 0], 32, 8, seed=91)
+    dev = [t.to(DEV) for t in (q, cache, table, sl, c, r)]
+    want = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], 8, 128, 16, num_splits=5)
+    ws = torch.full((C.paged_decode_workspace_bytes(4, 32, 8, 128, 16, table.shape[1], 5),), 0xff, dtype=torch.uint8, device=DEV)
+    for _ in range(2):
+        out = torch.full_like(dev[0], float("nan"))
+        C.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], 8, 128, 16, None, out, 5, ws)
+        assert torch.equal(out, want)
+    with pytest.raises((ValueError, RuntimeError)):
+        C.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], 8, 128, 16, None, out, 5, ws[:1024])
+
+
 def test_prod_paged_decode_without_copy_wavefronts(kernel_option):
     kernel_option("decode_copy_waves", False)
     _check_prod_decode([300, 1, 77, 0, 129], 32, num_splits=5)
