@@ -618,8 +618,16 @@ __device__ unsigned int g_decode_faults = 0u;
 template <bool PROD, bool HALF>
 __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     constexpr int CPR = StagedCfg<PROD>::CHUNKS_PER_ROW;
-    if constexpr (PROD) return uint32_t(16 * cc);          // TurboQuantProd pages come with 8 KV heads
     const int r = cc / CPR, ci = cc - r * CPR;
+    if constexpr (PROD) {                                  // five sections: K nibbles, K norms, K residual norms, V idx, V norms
+        int off;
+        if (ci < 32) off = 512 * hgrp + 16 * ci;
+        else if (ci < 34) off = H * 64 + 32 * hgrp + 16 * (ci - 32);
+        else if (ci < 36) off = H * 68 + 32 * hgrp + 16 * (ci - 34);
+        else if (ci < 68) off = H * 72 + 512 * hgrp + 16 * (ci - 36);
+        else off = H * 136 + 32 * hgrp + 16 * (ci - 68);
+        return uint32_t(r * (H * 140) + off);
+    }
     if constexpr (HALF) {
         int tok, off;                                      // which of the two tokens, offset in its 544-byte row
         if (ci < 32) { tok = ci >> 4; off = 16 * (ci & 15); }                      // K indices, 256 bytes per token
@@ -1642,7 +1650,7 @@ template <bool PROD, typename K>
 int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream, int copy_waves = 0) {
     // dynamic part only; the 64 KB table is static
     const size_t lds = 2 * size_t(StagedCfg<PROD>::TILE_BYTES);
-    return launch_with_lds(kernel, p, dim3(S, p.num_splits, PROD ? 1 : p.H_KV / 8), dim3(512 + 64 * copy_waves), lds, stream);
+    return launch_with_lds(kernel, p, dim3(S, p.num_splits, p.H_KV / 8), dim3(512 + 64 * copy_waves), lds, stream);
 }
 
 // The staged kernel runs with four more wavefronts that only copy; the switch
@@ -2131,7 +2139,9 @@ extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, cons
                                        num_splits);
     if (bad != FQ_OK) return bad;
     if (D != 128) return FQ_ERR_UNSUPPORTED_DIM;
-    if (H_KV != 8 || H_Q > 64) return FQ_ERR_BAD_SHAPE;   // the kernel stages 8 KV heads per token row
+    // the kernel stages the token rows of 8 KV heads, and the sketched queries of a group of 8 (float32,
+    // beside the rotated ones) fit its LDS for up to 8 query heads per KV head
+    if (H_KV % 8 != 0 || H_Q / H_KV > 8) return FQ_ERR_BAD_SHAPE;
     if (num_seqs == 0) return FQ_OK;
     if (!q || !out || !kv_cache || !block_table || !seq_lens || !centroids_k3 || !centroids_v || !rotation || !sketch)
         return FQ_ERR_NULL_POINTER;
@@ -2156,7 +2166,11 @@ extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, cons
     p.num_blocks = int(num_blocks); p.num_splits = num_splits;
     p.two_tables = 1;
     p.scale_log2e = sm_scale * kLog2e;
-    p.balance_slots = staged_balance_slots(num_seqs, num_splits);
+    // every group of 8 heads is a slice of the grid with the same (sequence, split) pairs
+    const int groups = H_KV / 8;
+    p.balance_slots = staged_balance_slots(num_seqs, num_splits * groups);
+    if (p.balance_slots > 0) p.balance_slots = p.balance_slots / groups > 0 ? p.balance_slots / groups : 1;
+    p.heads_per_wg = 0;
     p.spin_limit = fq_host::option(FQ_OPT_DECODE_TINY_SPIN) != 0 ? 2 : (1 << 20);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t max_ctx = int64_t(max_blocks_per_seq) * block_size;

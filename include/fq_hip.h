@@ -427,7 +427,7 @@ int fq_unpack_2bit(const uint8_t* packed, int64_t* indices, int64_t n_packed, vo
  * fq_prod_paged_decode: split-K decode over such pages, un-rotated query in, original-space
  *   output out: score = <q, k_mse> + gamma sqrt(pi/2)/D <S q, signs> (quantizer.py:355-370),
  *   softmax, TQ4 values.  sketch is S itself, (D, D) row-major.  Workspace and num_splits as in
- *   fq_split_k_paged_decode.  D == 128, H_KV == 8, H_Q <= 64.
+ *   fq_split_k_paged_decode.  D == 128, H_KV a multiple of 8, H_Q / H_KV <= 8.
  */
 int fq_prod_compress(const void* x, int x_dtype, const float* rotation, int rotation_col_major,
                      const float* sketch_rot, const float* boundaries, const float* centroids,

@@ -272,8 +272,10 @@ def test_shape_limits_of_the_staged_and_prod_decodes(lib):
     assert prod(S=0) == FQ_OK
     assert prod(D=64) == FQ_DIM and prod(D=256) == FQ_DIM
     assert prod(HKV=4, HQ=16) == FQ_SHAPE
-    assert prod(HQ=128) == FQ_SHAPE           # more than 64 query heads
+    assert prod(HQ=128) == FQ_SHAPE           # more than 8 query heads per KV head
     assert prod(HQ=8 * 17) == FQ_SHAPE
+    assert prod(HKV=12, HQ=24) == FQ_SHAPE    # KV heads come in groups of 8
+    assert prod(HKV=16, HQ=128) == FQ_NULL and prod(HKV=32, HQ=32) == FQ_NULL
     assert prod() == FQ_NULL                  # a supported shape gets as far as the pointer check
     lib.fq_paged_decode_fuses_rotation.argtypes = [ctypes.c_int] * 3
     assert lib.fq_paged_decode_fuses_rotation(128, 8, 1) == 1

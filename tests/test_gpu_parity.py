@@ -870,9 +870,9 @@ def test_prod_compress_parity(dtype):
     assert torch.equal(nib_g[7], torch.full_like(nib_g[7], int((b3 < 0).sum())))
 
 
-def _prod_case(lens, hq, bs=16, seed=7, dtype=torch.bfloat16, extra_blocks=2):
+def _prod_case(lens, hq, bs=16, seed=7, dtype=torch.bfloat16, extra_blocks=2, hkv=8):
     c3, b3, c4, b4, r, s = _prod_books()
-    hkv, d = 8, 128
+    d = 128
     g = torch.Generator().manual_seed(seed)
     S = len(lens)
     max_blocks = max(1, (max(lens) + bs - 1) // bs)
@@ -893,12 +893,12 @@ def _prod_case(lens, hq, bs=16, seed=7, dtype=torch.bfloat16, extra_blocks=2):
     return q, cache, table, torch.tensor(lens, dtype=torch.int32)
 
 
-def _check_prod_decode(lens, hq, bs=16, num_splits=0, dtype=torch.bfloat16, seed=7):
+def _check_prod_decode(lens, hq, bs=16, num_splits=0, dtype=torch.bfloat16, seed=7, hkv=8):
     c3, b3, c4, b4, r, s = _prod_books()
-    q, cache, table, sl = _prod_case(lens, hq, bs, seed, dtype)
-    want = O.prod_paged_decode(q, cache, table, sl, c3, c4, r, s, 8, 128, bs)
+    q, cache, table, sl = _prod_case(lens, hq, bs, seed, dtype, hkv=hkv)
+    want = O.prod_paged_decode(q, cache, table, sl, c3, c4, r, s, hkv, 128, bs)
     got = K.prod_paged_decode(q.to(DEV), cache.to(DEV), table.to(DEV), sl.to(DEV), c3.to(DEV), c4.to(DEV), r.to(DEV),
-                              s.to(DEV), 8, 128, bs, num_splits=num_splits)
+                              s.to(DEV), hkv, 128, bs, num_splits=num_splits)
     torch.cuda.synchronize()
     err = (got.cpu().float() - want.float()).abs().max().item()
     assert err <= 2e-2, f"max abs error {err}"
@@ -908,6 +908,15 @@ def _check_prod_decode(lens, hq, bs=16, num_splits=0, dtype=torch.bfloat16, seed
 @pytest.mark.parametrize("num_splits", [0, 1, 5])
 def test_prod_paged_decode_group_sizes_and_splits(hq, num_splits):
     _check_prod_decode([300, 1, 77, 0, 129], hq, num_splits=num_splits)
+
+
+@pytest.mark.parametrize("hq,hkv,bs,dtype", [(16, 16, 16, torch.bfloat16), (64, 16, 16, torch.bfloat16), (128, 16, 8, torch.float16),
+                                             (48, 24, 32, torch.bfloat16), (96, 24, 16, torch.float16)])
+def test_prod_paged_decode_groups_of_eight_kv_heads(hq, hkv, bs, dtype):
+    """More than 8 KV heads: a workgroup serves one group of 8 and copies that group's slices of the five
+    sections of every token row."""
+    _check_prod_decode([300, 1, 77, 0, 129], hq, bs=bs, num_splits=3, dtype=dtype, hkv=hkv)
+    _check_prod_decode([900, 0, 37, 2100, 64, 1025, 1, 1500], hq, bs=bs, num_splits=40, dtype=dtype, hkv=hkv, seed=11)
 
 
 def test_prod_paged_decode_ragged_batch_with_more_splits_than_cus():
