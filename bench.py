@@ -339,10 +339,22 @@ def main():
                                      rotation_T_even=ev_s, rotation_T_odd=od_s)
             K.split_k_paged_decode(q, cache, table, lens, cent_d, cent_d, rot_d, H_KV, D, BS, sm_scale=scale, out=out)
 
+        bnd_d = book[1].to(dev)
+
+        def serving_step_one_call(i):
+            # the same step through the entry point that stores the new token inside the decode launch
+            cache, table = caches[i % n_caches]
+            K.tq4_store_and_decode(k_new, v_new, last_slots[i % n_caches], q, cache, table, lens, cent_d, cent_d, rot_d,
+                                   bnd_d, H_KV, D, BS, sm_scale=scale, out=out, rotation_T_even=ev_s, rotation_T_odd=od_s)
+
         for i in range(args.warmup):
             serving_step(i)
-        serve_ms, _ = time_events(serving_step, args.steps)
-        extra.update({"serving_step_us_cold": serve_ms * 1e3, "serving_tokens_per_s": BATCH / (serve_ms * 1e-3)})
+        serve2_ms = time_region(serving_step, args.steps)
+        for i in range(args.warmup):
+            serving_step_one_call(i)
+        serve_ms = time_region(serving_step_one_call, args.steps)
+        extra.update({"serving_step_us_cold": serve_ms * 1e3, "serving_tokens_per_s": BATCH / (serve_ms * 1e-3),
+                      "serving_step_us_cold_store_then_decode": serve2_ms * 1e3})
         del caches
         torch.cuda.empty_cache()
         rows_tok = 32 * 65536

@@ -307,6 +307,82 @@ at::Tensor split_k_paged_decode(const at::Tensor& q, const at::Tensor& kv_cache,
     return result;
 }
 
+// One serving step (src/flashquant/vllm/impl.py:362-394): the new token of every sequence into its cache
+// row, then the decode.  Everything must already be on the GPU (a serving loop's tensors are).
+at::Tensor tq4_store_and_decode(const at::Tensor& key, const at::Tensor& value, const at::Tensor& slot_mapping,
+                                const at::Tensor& rot_T_even, const at::Tensor& rot_T_odd, const at::Tensor& boundaries,
+                                const at::Tensor& q, at::Tensor kv_cache, const at::Tensor& block_table,
+                                const at::Tensor& seq_lens, const at::Tensor& centroids_k, const at::Tensor& centroids_v,
+                                const at::Tensor& rotation, int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                                std::optional<double> sm_scale, const std::optional<at::Tensor>& out, int64_t num_splits,
+                                const std::optional<at::Tensor>& workspace) {
+    const at::Tensor& cache_ref = kv_cache;
+    for (const at::Tensor* t : {&key, &value, &slot_mapping, &rot_T_even, &rot_T_odd, &boundaries, &q, &cache_ref,
+                                &block_table, &seq_lens, &centroids_k, &centroids_v, &rotation})
+        fqbind::require_gpu(*t, "every operand");
+    require(q.dim() == 3 && q.size(2) == head_dim, "q must have shape (num_seqs, H_Q, D)");
+    require(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, "q must be float16 or bfloat16");
+    const int64_t S = q.size(0), HQ = q.size(1), D = head_dim, H = num_kv_heads;
+    require(key.dim() == 3 && key.size(0) == S && key.size(1) == H && key.size(2) == D && value.sizes() == key.sizes() &&
+                key.scalar_type() == q.scalar_type() && value.scalar_type() == q.scalar_type(),
+            "key and value must have shape (num_seqs, H_KV, D) and the dtype of q");
+    require(slot_mapping.dim() == 1 && slot_mapping.size(0) == S && slot_mapping.scalar_type() == at::kLong,
+            "slot_mapping must be int64 of shape (num_seqs,)");
+    require(rot_T_even.scalar_type() == at::kFloat && rot_T_odd.scalar_type() == at::kFloat &&
+                boundaries.scalar_type() == at::kFloat && rot_T_even.dim() == 2 && rot_T_even.size(0) == D &&
+                rot_T_even.size(1) == D / 2 && rot_T_odd.sizes() == rot_T_even.sizes() && boundaries.numel() == 15,
+            "rotation halves must be float32 (D, D/2), boundaries 15 float32 values");
+    require(kv_cache.dim() == 3 && kv_cache.scalar_type() == at::kByte && kv_cache.is_contiguous() &&
+                kv_cache.size(1) == block_size && kv_cache.size(2) == H * (D + 8),
+            "kv_cache must be contiguous uint8 of shape (num_blocks, block_size, num_kv_heads * (head_dim + 8))");
+    require(block_table.dim() == 2 && block_table.scalar_type() == at::kInt && block_table.size(0) == S,
+            "block_table must be int32 of shape (num_seqs, max_blocks)");
+    require(seq_lens.scalar_type() == at::kInt && seq_lens.numel() == S, "seq_lens must be int32 (num_seqs,)");
+    require(centroids_k.numel() == 16 && centroids_v.numel() == 16 && centroids_k.scalar_type() == at::kFloat &&
+                centroids_v.scalar_type() == at::kFloat,
+            "centroids must be 16 float32 values");
+    require(num_splits >= 0, "num_splits must be >= 0");
+    c10::DeviceGuard guard(q.device());
+    const double scale = sm_scale.has_value() ? *sm_scale : 1.0 / std::sqrt(double(head_dim));
+    const at::Tensor kc = key.contiguous(), vc = value.contiguous(), qc = q.contiguous();
+    const at::Tensor re = rot_T_even.contiguous(), ro = rot_T_odd.contiguous(), bd = boundaries.contiguous();
+    const at::Tensor bt = block_table.contiguous(), sl = seq_lens.contiguous(), sm = slot_mapping.contiguous();
+    const at::Tensor ck = centroids_k.contiguous();
+    const bool same = centroids_v.is_same(centroids_k) || centroids_v.data_ptr() == centroids_k.data_ptr();
+    const at::Tensor cv = same ? ck : centroids_v.contiguous();
+    const RotationArg rot = rotation_arg(rotation, q.device(), int(D));
+    at::Tensor result;
+    if (out.has_value()) {
+        result = *out;
+        require(result.is_cuda() && result.is_contiguous() && result.scalar_type() == q.scalar_type() &&
+                    result.sizes() == q.sizes(),
+                "out must be a contiguous GPU tensor with the shape and dtype of q");
+    } else {
+        result = at::empty_like(qc);
+    }
+    const int max_blocks = int(bt.size(1));
+    const size_t ws_bytes = fq_paged_decode_workspace_bytes(int(S), int(HQ), int(H), int(D), int(block_size), max_blocks,
+                                                            int(num_splits));
+    at::Tensor ws;
+    if (workspace.has_value()) {
+        ws = *workspace;
+        require(ws.is_cuda() && ws.device() == q.device() && ws.is_contiguous() && ws.scalar_type() == at::kByte &&
+                    size_t(ws.numel()) >= ws_bytes,
+                "workspace must be a contiguous uint8 GPU tensor of at least paged_decode_workspace_bytes(...) bytes");
+    } else {
+        ws = at::empty({int64_t(ws_bytes)}, q.options().dtype(at::kByte));
+    }
+    const int st = fq_tq4_store_and_decode(
+        kc.data_ptr(), vc.data_ptr(), sm.data_ptr<int64_t>(), re.data_ptr<float>(), ro.data_ptr<float>(),
+        bd.data_ptr<float>(), qc.data_ptr(), kv_cache.data_ptr<uint8_t>(), bt.data_ptr<int32_t>(), sl.data_ptr<int32_t>(),
+        ck.data_ptr<float>(), cv.data_ptr<float>(), rot.ptr, rot.col_major, result.data_ptr(), int(S), int(HQ), int(H),
+        int(D), int(block_size), max_blocks, kv_cache.size(0), float(scale),
+        fqbind::dtype_code(q.scalar_type(), "tq4_store_and_decode"), int(num_splits), ws.data_ptr(), size_t(ws.numel()),
+        fqbind::current_stream(q));
+    fqbind::raise_on_error(st, "tq4_store_and_decode");
+    return result;
+}
+
 // Keys or values of (B, H, N, X) taken from a buffer of larger token capacity: a view
 // buffer[:, :, :N, :] (the reference's CompressedBuffer.get(), src/flashquant/cache/buffer_pool.py:128-140)
 // keeps the row layout of a contiguous tensor with N replaced by the capacity.  Returns that
@@ -733,6 +809,12 @@ void bind_kernels(py::module_& m) {
     m.def("tq4_decompress", &tq4_decompress, py::arg("packed"), py::arg("norms"), py::arg("centroids"),
           py::arg("dtype"), py::arg("out") = py::none(),
           "TQ4 decompress to (N, H, D) in dtype, rotated space.");
+    m.def("tq4_store_and_decode", &tq4_store_and_decode, py::arg("key"), py::arg("value"), py::arg("slot_mapping"),
+          py::arg("rotation_T_even"), py::arg("rotation_T_odd"), py::arg("boundaries"), py::arg("q"), py::arg("kv_cache"),
+          py::arg("block_table"), py::arg("seq_lens"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),
+          py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),
+          py::arg("out") = py::none(), py::arg("num_splits") = 0, py::arg("workspace") = py::none(),
+          "One serving step: every sequence's new token compressed into its cache row, then the split-K paged decode.");
     m.def("split_k_paged_decode", &split_k_paged_decode, py::arg("q"), py::arg("kv_cache"), py::arg("block_table"),
           py::arg("seq_lens"), py::arg("centroids_k"), py::arg("centroids_v"), py::arg("rotation"),
           py::arg("num_kv_heads"), py::arg("head_dim"), py::arg("block_size"), py::arg("sm_scale") = py::none(),

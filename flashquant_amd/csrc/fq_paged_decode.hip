@@ -644,9 +644,10 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     return uint32_t(r * (H * 136) + off);
 }
 
-template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false>
+template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false, bool STORE = false>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
+    static_assert(!STORE || (CW > 0 && !HALF && !PROD), "the new token is stored by the TQ4 form with copy wavefronts");
     using Cfg = StagedCfg<PROD>;
     constexpr int kStageBytes = Cfg::STAGE_BYTES;
     constexpr int kTileBytes = Cfg::TILE_BYTES;
@@ -666,7 +667,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // CW > 0: [0] rotated heads stored, [1] rotated (and sketched) heads read back, [2] a hand-off timed
     // out, [3 + s] tiles written to slot s (one count per copy wavefront and tile), [5 + s] tiles read
     // from slot s (one count per computing wavefront and tile)
-    __shared__ uint32_t flags[7];
+    // STORE: [7] computing wavefronts whose part of the new token's row has reached the cache
+    __shared__ uint32_t flags[8];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -829,7 +831,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         // The flags are cleared behind a barrier placed where nobody waits for anybody: every
         // wavefront has just asked for its sequence length and page ids and none has used them yet
         // (the barrier does not wait for loads from global memory).
-        if (tid < 7) flags[tid] = 0u;
+        if (tid < 8) flags[tid] = 0u;
         __syncthreads();
         load_matrix_columns();
         load_first_heads();
@@ -915,6 +917,10 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     for (int r = 0; r < PVR; ++r) pv[r] = pv[r] < 0 ? 0 : (pv[r] > max_page ? max_page : pv[r]);
     const int last_t0 = begin + ((end - begin - 1) & ~31);
     auto clamp_t0 = [&](int t) { return t < last_t0 ? t : last_t0; };
+    // STORE: this workgroup's split ends with the sequence's last token, the one this step adds: its
+    // computing wavefronts write that token's cache row in the prologue, and its copy wavefronts ask
+    // for the split's last tile only after that (uniform over the workgroup)
+    const bool stores_token = STORE && end == L;
 
     if constexpr (CW > 0) {
         if (copier) {
@@ -946,6 +952,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             const bool has_rest = kHalfTail || ct < REST;
             auto c_issue = [&](uint4v (&r)[NR], int t0) {
                 if (t0 > last_t0) return;             // beyond the split: nothing to fetch
+                if constexpr (STORE) {
+                    if (stores_token && t0 == last_t0 && !lds_flag_wait(&flags[7], 8u, p.spin_limit)) flags[2] = 1u;
+                }
                 const uint8_t* base[PPT];
                 const int p0 = (t0 >> BSL) - split_p0;
 #pragma unroll
@@ -1076,6 +1085,80 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                         const int head = 16 * rb + 4 * g + i;
                         if (head < HQG) qs2[head * D + 16 * h + n] = acc2[i] * up;
                     }
+                }
+            }
+            if constexpr (STORE) {
+                if (stores_token) {
+                    // ---- the new token: TQ4 compress of its 8 key and 8 value rows (one more block of 16
+                    // rows for the same matrix product) straight into the cache row: n = ||x||,
+                    // y = (x R^T) / (n + 1e-10), index = number of boundaries below y, two indices per byte
+                    // (cpu_reference.py:22-61, vllm/impl.py:220-263).  Wavefront h holds columns 16h..16h+15.
+                    const int64_t slot = p.new_slots[seq];
+                    const uint16_t* xrow = reinterpret_cast<const uint16_t*>(n < 8 ? p.new_key : p.new_value) +
+                                           (int64_t(seq) * p.H_KV + 8 * hgrp + (n & 7)) * D;
+                    uint4v raw[KS];
+#pragma unroll
+                    for (int j = 0; j < KS; ++j) raw[j] = *reinterpret_cast<const uint4v*>(xrow + 32 * j + 8 * g);
+                    const float bnd_mine = p.boundaries[lane < 15 ? lane : 14];
+                    float ss = 0.0f;         // sum of squares of row n: this lane's 32 elements, then over g
+#pragma unroll
+                    for (int j = 0; j < KS; ++j) {
+                        const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float a = load_elem<DT>(uint16_t(w[i] & 0xffffu)), b = load_elem<DT>(uint16_t(w[i] >> 16));
+                            ss = __builtin_fmaf(a, a, ss);
+                            ss = __builtin_fmaf(b, b, ss);
+                        }
+                    }
+                    ss += xor_shuffle(ss, 16);
+                    ss += xor_shuffle(ss, 32);
+                    float4v acc;
+                    float up = 1.0f;
+                    if constexpr (kRawBf16) {
+                        bf16v8 a[KS];
+#pragma unroll
+                        for (int j = 0; j < KS; ++j) a[j] = __builtin_bit_cast(bf16v8, raw[j]);
+                        acc = rotate_block_bf16<D>(a, rot_t);
+                    } else {
+                        half8 a[KS];
+                        rows_as_f16<D, DT>(raw, a, up);
+                        acc = rotate_block_f16<D>(a, rot_hi, rot_lo);
+                    }
+                    const bool stored = slot >= 0 && slot < p.num_slots;
+                    uint8_t* crow = p.cache_rw + (stored ? slot : 0) * int64_t(row_bytes);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int r = 4 * g + i;                     // row of the block: key head r, or value head r - 8
+                        const float ssr = __shfl(ss, r, kWave);
+                        const bool tiny = ssr < 0x1p-96f;            // as the compress kernel: v_sqrt_f32 on a normal number
+                        const float nrm_s = __builtin_amdgcn_sqrtf(tiny ? ssr * 0x1p64f : ssr);
+                        const float nrm = tiny ? nrm_s * 0x1p-32f : nrm_s;
+                        const float y = acc[i] * (up * __builtin_amdgcn_rcpf(nrm + 1e-10f));
+                        uint32_t idx = 0u;
+#pragma unroll
+                        for (int k = 0; k < 15; ++k)
+                            idx += bits_to_float(uint32_t(__builtin_amdgcn_readlane(int(float_to_bits(bnd_mine)), k))) < y ? 1u : 0u;
+                        // byte j of a head = index of coordinate 2j (high nibble) and 2j + 1: columns n, n + 1
+                        const uint32_t other = uint32_t(__shfl_xor(int(idx), 1, kWave));
+                        const uint32_t byte = (idx << 4) | other;                        // valid in even n
+                        uint32_t lo = (n & 9) == 0 ? byte << (4 * (n & 6)) : 0u;         // n = 0, 2, 4, 6: bytes 0..3
+                        uint32_t hi = (n & 9) == 8 ? byte << (4 * (n & 6)) : 0u;         // n = 8 .. 14: bytes 4..7
+#pragma unroll
+                        for (int mask = 2; mask < 16; mask <<= 1) {
+                            lo |= uint32_t(__shfl_xor(int(lo), mask, kWave));
+                            hi |= uint32_t(__shfl_xor(int(hi), mask, kWave));
+                        }
+                        const int head = 8 * hgrp + (r & 7);
+                        const int sect = r < 8 ? 0 : p.H_KV * (D / 2 + 4);               // key sections, then value sections
+                        if (stored && n == 0)
+                            *reinterpret_cast<uint2v*>(crow + sect + head * (D / 2) + 8 * h) = uint2v{lo, hi};
+                        if (stored && n == 1 && h == 0)
+                            *reinterpret_cast<float*>(crow + sect + p.H_KV * (D / 2) + 4 * head) = nrm;
+                    }
+                    // the row is in the cache before the copy wavefronts ask for it
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    lds_flag_signal(&flags[7], lane);
                 }
             }
             if constexpr (CW > 0) {
@@ -1641,6 +1724,15 @@ inline DecodeVariant read_decode_variant() {
     return v;
 }
 
+// The new token of a serving step, for the staged kernel that stores it (DecodeParams: new_key ...).
+struct NewToken {
+    const void* key;
+    const void* value;
+    const int64_t* slots;
+    const float* boundaries;
+    uint8_t* cache;
+};
+
 // The staged kernel covers KV heads of dimension 128 in groups of 8.
 inline bool staged_applies(int D, int H_KV, const DecodeVariant& v) {
     return D == 128 && H_KV >= 8 && H_KV % 8 == 0 && !v.direct;
@@ -1658,11 +1750,19 @@ int launch_staged(K kernel, const DecodeParams& p, int S, hipStream_t stream, in
 
 // Staged kernel for every page size and group size; PROD selects the TurboQuantProd page format.
 template <int DT, bool PROD>
-int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream_t stream, int copy_waves) {
+int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream_t stream, int copy_waves,
+                      bool store = false) {
 #define FQ_STAGED_GP(BSL, GPV)                                                                                  \
     /* TurboQuantProd pages come with at most 64 query heads (8 per KV head) */                                 \
     if constexpr (PROD && GPV == 16) return FQ_ERR_BAD_SHAPE;                                                   \
     else {                                                                                                      \
+        if constexpr (!PROD) {                                                                                  \
+            if (store) {                                                                                        \
+                if (copy_waves != 4) return FQ_ERR_LAUNCH;                                                      \
+                return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4, false, true>, p, S, stream, 4) \
+                            : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 4, false, true>, p, S, stream, 4); \
+            }                                                                                                   \
+        }                                                                                                       \
         if (copy_waves == 4)                                                                                    \
             return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4>, p, S, stream, 4) \
                         : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 4>, p, S, stream, 4); \
@@ -1712,6 +1812,7 @@ int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wid
 template <int D, int DT>
 int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bool allow_half, const DecodeVariant& var) {
     if (allow_half && staged_half_applies(D, p.H_KV, BS, var)) {
+        if (p.new_key != nullptr) return FQ_ERR_LAUNCH;
         // the kernel counts rows of two tokens: half the page size, chunks of rows
         const int rows_per_page = BS / 2;
         const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
@@ -1734,11 +1835,13 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
         ps.balance_slots = staged_balance_slots(S, p.num_splits * groups);
         if (ps.balance_slots > 0) ps.balance_slots = ps.balance_slots / groups > 0 ? ps.balance_slots / groups : 1;
         // a chosen chunk may span up to 256 pages: four page-id registers
+        if (var.ring && p.new_key != nullptr) return FQ_ERR_LAUNCH;
         if (var.ring)
             return launch_ring(ps, S, BS, wide || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256), DT, stream);
         return launch_staged_any<DT, false>(ps, S, BS, wide || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256),
-                                            stream, var.copy_waves);
+                                            stream, var.copy_waves, p.new_key != nullptr);
     }
+    if (p.new_key != nullptr) return FQ_ERR_LAUNCH;     // only the staged kernel stores the new token
 
     const int max_waves = D == 256 ? 4 : 8;
     // 1 or 2 KV heads: a full workgroup, its wavefronts beyond the heads on the next splits (measured on 8 x 32768
@@ -1929,7 +2032,7 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
                     const int32_t* seq_lens, const float* centroids_k, const float* centroids_v, float* partial_acc,
                     float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D, int block_size,
                     int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype, int num_splits,
-                    void* stream, const DecodeVariant& var, bool allow_half = false) {
+                    void* stream, const DecodeVariant& var, bool allow_half = false, const NewToken* token = nullptr) {
     const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
                                        num_splits);
     if (bad != FQ_OK) return bad;
@@ -1952,6 +2055,12 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
     p.balance_slots = 0;
     p.heads_per_wg = 0;
     p.spin_limit = fq_host::option(FQ_OPT_DECODE_TINY_SPIN) != 0 ? 2 : (1 << 20);
+    p.cache_rw = token ? token->cache : nullptr;
+    p.new_key = token ? token->key : nullptr;
+    p.new_value = token ? token->value : nullptr;
+    p.new_slots = token ? token->slots : nullptr;
+    p.boundaries = token ? token->boundaries : nullptr;
+    p.num_slots = num_blocks * block_size;
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define FQ_DECODE_D(DD)                                                                 \
     case DD:                                                                            \
@@ -2010,13 +2119,16 @@ extern "C" int fq_split_k_reduce(const float* partial_acc, const float* partial_
                : launch_reduce<FQ_BF16>(partial_acc, partial_m, partial_l, rotation, rotation_col_major, out, num_seqs, H_Q, D, num_splits, s);
 }
 
-extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
-                                       const int32_t* seq_lens, const float* centroids_k,
-                                       const float* centroids_v, const float* rotation, int rotation_col_major, void* out,
-                                       int num_seqs, int H_Q, int H_KV, int D, int block_size,
-                                       int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype,
-                                       int num_splits, void* workspace, size_t workspace_bytes, void* stream) {
-    using namespace fq;
+namespace fq {
+// fq_split_k_paged_decode for one reading `var` of the switches; `token`: the staged kernel (which must be
+// the one that `var` selects for this shape) also stores the step's new token.
+int split_k_paged_decode_impl(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
+                              const int32_t* seq_lens, const float* centroids_k,
+                              const float* centroids_v, const float* rotation, int rotation_col_major, void* out,
+                              int num_seqs, int H_Q, int H_KV, int D, int block_size,
+                              int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype,
+                              int num_splits, void* workspace, size_t workspace_bytes, void* stream,
+                              const DecodeVariant& var, const NewToken* token) {
     const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
                                        num_splits);
     if (bad != FQ_OK) return bad;
@@ -2024,9 +2136,6 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     if (!q || !out) return FQ_ERR_NULL_POINTER;
     if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16)) return FQ_ERR_MISALIGNED;
     num_splits = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
-    // One reading of the kernel-variant switches for the whole call: the kernel choice, the number of
-    // partials it writes, the workspace layout and what the combine kernel merges all follow from it.
-    const DecodeVariant var = read_decode_variant();
     // 4 KV heads: the staged kernel reads rows of two tokens and writes one partial per token parity
     const bool half = staged_half_applies(D, H_KV, block_size, var);
     const int num_partials = half ? 2 * num_splits : num_splits;
@@ -2050,9 +2159,60 @@ extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, c
     }
     int st = decode_partials(q_in, fused_rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m,
                              l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
-                             num_splits, stream, var, half);
+                             num_splits, stream, var, half, token);
     if (st != FQ_OK) return st;
     return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_partials, stream);
+}
+}  // namespace fq
+
+extern "C" int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* block_table,
+                                       const int32_t* seq_lens, const float* centroids_k,
+                                       const float* centroids_v, const float* rotation, int rotation_col_major, void* out,
+                                       int num_seqs, int H_Q, int H_KV, int D, int block_size,
+                                       int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype,
+                                       int num_splits, void* workspace, size_t workspace_bytes, void* stream) {
+    // One reading of the kernel-variant switches for the whole call: the kernel choice, the number of
+    // partials it writes, the workspace layout and what the combine kernel merges all follow from it.
+    return fq::split_k_paged_decode_impl(q, kv_cache, block_table, seq_lens, centroids_k, centroids_v, rotation,
+                                         rotation_col_major, out, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq,
+                                         num_blocks, sm_scale, dtype, num_splits, workspace, workspace_bytes, stream,
+                                         fq::read_decode_variant(), nullptr);
+}
+
+// One serving step: the new token of every sequence compressed into its cache row, then the decode over
+// the cache that holds it (src/flashquant/vllm/impl.py:362-394).  One launch fewer where the staged
+// kernel with copy wavefronts runs (KV heads of dimension 128 in groups of 8, a rotation matrix given):
+// the workgroup whose split ends with a sequence's last token compresses and stores that token itself.
+extern "C" int fq_tq4_store_and_decode(const void* key, const void* value, const int64_t* slot_mapping,
+                                       const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
+                                       const void* q, uint8_t* kv_cache, const int32_t* block_table,
+                                       const int32_t* seq_lens, const float* centroids_k, const float* centroids_v,
+                                       const float* rotation, int rotation_col_major, void* out, int num_seqs,
+                                       int H_Q, int H_KV, int D, int block_size, int max_blocks_per_seq,
+                                       int64_t num_blocks, float sm_scale, int dtype, int num_splits,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace fq;
+    const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
+                                       num_splits);
+    if (bad != FQ_OK) return bad;
+    if (num_seqs == 0) return FQ_OK;
+    if (!key || !value || !slot_mapping || !rot_T_even || !rot_T_odd || !boundaries || !rotation || !kv_cache)
+        return FQ_ERR_NULL_POINTER;
+    if (!fq_host::aligned(key, 16) || !fq_host::aligned(value, 16) || !fq_host::aligned(slot_mapping, 8) ||
+        !fq_host::aligned(kv_cache, 16) || !fq_host::aligned(boundaries, 4))
+        return FQ_ERR_MISALIGNED;
+    const DecodeVariant var = read_decode_variant();
+    const bool in_launch = centroids_k && staged_applies(D, H_KV, var) && !var.ring && var.copy_waves == 4;
+    const NewToken token{key, value, slot_mapping, boundaries, kv_cache};
+    if (!in_launch) {
+        const int st = fq_tq4_compress_store(key, value, dtype, rot_T_even, rot_T_odd, boundaries, kv_cache, slot_mapping,
+                                             num_seqs, num_seqs, H_KV, D, num_blocks * block_size, stream);
+        if (st != FQ_OK) return st;
+    }
+    return split_k_paged_decode_impl(q, kv_cache, block_table, seq_lens, centroids_k, centroids_v, rotation,
+                                     rotation_col_major, out, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq,
+                                     num_blocks, sm_scale, dtype, num_splits, workspace, workspace_bytes, stream, var,
+                                     in_launch ? &token : nullptr);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -2172,6 +2332,8 @@ extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, cons
     if (p.balance_slots > 0) p.balance_slots = p.balance_slots / groups > 0 ? p.balance_slots / groups : 1;
     p.heads_per_wg = 0;
     p.spin_limit = fq_host::option(FQ_OPT_DECODE_TINY_SPIN) != 0 ? 2 : (1 << 20);
+    p.cache_rw = nullptr; p.new_key = nullptr; p.new_value = nullptr; p.new_slots = nullptr; p.boundaries = nullptr;
+    p.num_slots = 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t max_ctx = int64_t(max_blocks_per_seq) * block_size;
     const int64_t chunk = (((max_ctx + num_splits - 1) / num_splits) + 63) & ~int64_t(63);

@@ -30,6 +30,15 @@ struct DecodeParams {
     int spin_limit;             // staged kernel: polls of a bounded wait between wavefronts before it gives up
     int balance_slots;          // staged kernel: > 0 lets the workgroups size the token chunks from the actual
                                 // sequence lengths, for this many workgroups running at a time (num_seqs <= 64)
+    // Staged kernel instantiated with STORE: the serving step in one launch.  The workgroup whose split
+    // holds a sequence's last token first compresses that token's new key and value rows into their
+    // cache row (slot new_slots[seq]; negative: not stored), then reads the row back with its tile.
+    uint8_t* cache_rw;          // the cache again, for the row that is written
+    const void* new_key;        // (S, H_KV, D) query dtype, one token per sequence
+    const void* new_value;
+    const int64_t* new_slots;   // (S,) flat slot of the new token
+    const float* boundaries;    // (15,) ascending
+    int64_t num_slots;          // num_blocks * block_size
 };
 
 

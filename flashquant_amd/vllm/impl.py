@@ -58,6 +58,18 @@ class TQ4AttentionKernels:
                                                self.rotation, self.num_kv_heads, self.head_size, kv_cache.shape[1],
                                                sm_scale=self.scale, out=out)
 
+    def decode_step(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, kv_cache: torch.Tensor,
+                    slot_mapping: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``compress_and_store`` of one new token per sequence followed by ``decode``, as one call
+        (src/flashquant/vllm/impl.py:362-394): ``key`` / ``value`` (S, H_KV, D), ``slot_mapping`` (S,) int64,
+        ``seq_lens`` counting the new token."""
+        require_gpu(query, "query")
+        return native().tq4_store_and_decode(key, value, slot_mapping, self.rot_T_even, self.rot_T_odd, self.boundaries,
+                                             query, kv_cache, block_table, seq_lens, self.centroids, self.centroids,
+                                             self.rotation, self.num_kv_heads, self.head_size, kv_cache.shape[1],
+                                             sm_scale=self.scale, out=out)
+
     def prefill(self, query: torch.Tensor, query_start_loc: torch.Tensor, max_query_len: int, kv_cache: torch.Tensor,
                 block_table: torch.Tensor, seq_lens: torch.Tensor, out: Optional[torch.Tensor] = None,
                 causal: bool = True) -> torch.Tensor:
@@ -127,8 +139,15 @@ def _make_impl_class() -> type:
                 return self._forward_encoder_attention(query[:n], key[:n], value[:n], output[:n], attn_metadata, layer)
             if getattr(attn_metadata, "use_cascade", False):
                 raise NotImplementedError("cascade attention is not supported by the FlashQuant backend")
+            slots = attn_metadata.slot_mapping
+            if (attn_metadata.max_query_len == 1 and key is not None and value is not None
+                    and n == attn_metadata.seq_lens.shape[0] and slots.shape[0] >= n):
+                # a pure decode step: one new token per sequence, stored and attended over in one call
+                self._tq4.decode_step(query[:n], key[:n], value[:n], kv_cache, slots[:n].long(), attn_metadata.block_table,
+                                      attn_metadata.seq_lens, out=output[:n])
+                return output
             if key is not None and value is not None:
-                self._tq4.compress_and_store(key, value, kv_cache, attn_metadata.slot_mapping)
+                self._tq4.compress_and_store(key, value, kv_cache, slots)
             if attn_metadata.max_query_len == 1:
                 self._tq4.decode(query[:n], kv_cache, attn_metadata.block_table, attn_metadata.seq_lens, out=output[:n])
             else:

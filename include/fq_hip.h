@@ -346,6 +346,41 @@ int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
                             void* stream);
 
 /*
+ * One serving step in one call: the step's new token of every sequence is
+ * compressed into its cache row (fq_tq4_compress_store on one token per
+ * sequence), then the decode runs over the cache that holds it
+ * (fq_split_k_paged_decode).  It is the sequence of
+ * src/flashquant/vllm/impl.py:362-394 (_compress_and_store, then the decode
+ * kernel) for a batch of single-token queries.
+ *
+ *   key, value    (S, H_KV, D) fp16/bf16 as q, contiguous, 16-byte aligned
+ *   slot_mapping  (S,) int64: flat slot of sequence s's new token; negative or
+ *                 out of range: not stored
+ *   rot_T_even, rot_T_odd, boundaries   as for fq_tq4_compress_store
+ *   kv_cache      read and written
+ *   everything else as for fq_split_k_paged_decode; rotation must not be NULL;
+ *   seq_lens counts the new token.
+ * Where the staged decode kernel runs (D == 128, H_KV a multiple of 8, default
+ * switches) this is one launch fewer: the workgroup whose split ends with a
+ * sequence's last token compresses and stores that token in its prologue and
+ * reads the row back with its last tile.  For that form slot_mapping[s] must be
+ * the slot of token seq_lens[s] - 1 of sequence s as the block table gives it
+ * (block_table[s][(L-1) / block_size] * block_size + (L-1) % block_size), which
+ * is what a decode step passes; a sequence of length 0 stores nothing.  The
+ * rotation there is the exact float32 one (three bf16 terms), so the stored
+ * indices are those of FQ_OPT_COMPRESS_THREE_TERMS.  Other shapes run the two
+ * entry points one after the other.
+ */
+int fq_tq4_store_and_decode(const void* key, const void* value, const int64_t* slot_mapping,
+                            const float* rot_T_even, const float* rot_T_odd, const float* boundaries,
+                            const void* q, uint8_t* kv_cache, const int32_t* block_table,
+                            const int32_t* seq_lens, const float* centroids_k, const float* centroids_v,
+                            const float* rotation, int rotation_col_major, void* out, int num_seqs,
+                            int H_Q, int H_KV, int D, int block_size, int max_blocks_per_seq,
+                            int64_t num_blocks, float sm_scale, int dtype, int num_splits,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The three stages of fq_split_k_paged_decode as separate launches, for callers
  * that hold the rotated query or want the partials (the reference exposes its
  * decode at this level: paged_tq4_decode_cuda, csrc/cuda/paged_decode.cu:346-368,

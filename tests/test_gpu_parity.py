@@ -830,6 +830,104 @@ def test_compress_and_store_then_decode_matches_oracle():
     assert (got.cpu().float() - want.float()).abs().max().item() <= 2e-2
 
 
+def _serving_case(lens, hq, hkv, d, bs, dtype, seed):
+    """A paged cache that holds tokens 0 .. L - 2 of every sequence (random bytes where token L - 1 will go),
+    the new token's key and value rows, its slot, and the query."""
+    q, cache, table, sl = build_paged_case([max(L - 1, 0) for L in lens], hq, hkv, d=d, bs=bs, seed=seed, dtype=dtype,
+                                           extra_blocks=len(lens) + 3)
+    # one more block-table column may be needed for the new token: give every sequence a fresh page for it
+    need = max(1, max((L + bs - 1) // bs for L in lens))
+    used = set(table.flatten().tolist())
+    free = [b for b in range(cache.shape[0]) if b not in used]
+    table2 = torch.zeros(len(lens), need, dtype=torch.int32)
+    table2[:, :table.shape[1]] = table[:, :need] if table.shape[1] >= need else table
+    for i, L in enumerate(lens):
+        old_pages = (max(L - 1, 0) + bs - 1) // bs
+        if L > 0 and (L + bs - 1) // bs > old_pages:
+            table2[i, old_pages] = free.pop()
+    g = torch.Generator().manual_seed(seed + 1000)
+    key = torch.randn(len(lens), hkv, d, generator=g).to(dtype)
+    value = torch.randn(len(lens), hkv, d, generator=g).to(dtype)
+    slots = torch.tensor([int(table2[i, (L - 1) // bs]) * bs + (L - 1) % bs if L > 0 else -1 for i, L in enumerate(lens)])
+    return q, cache, table2, torch.tensor(lens, dtype=torch.int32), key, value, slots
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs,dtype", [(32, 8, 128, 16, torch.bfloat16), (64, 8, 128, 8, torch.float16),
+                                               (128, 8, 128, 32, torch.bfloat16), (32, 16, 128, 16, torch.bfloat16),
+                                               (32, 4, 128, 16, torch.bfloat16), (8, 2, 64, 16, torch.float16)])
+def test_store_and_decode_equals_store_then_decode(hq, hkv, d, bs, dtype, kernel_option):
+    """The serving step as one call.  Where the staged kernel runs (the first four shapes) the workgroup
+    that owns a sequence's last token compresses and stores it itself, with the exact float32 rotation:
+    the cache must then hold what compress-and-store writes in its three-term mode (indices equal up to
+    coordinates within float32 rounding of a boundary, norms to 2e-6), nothing else in the cache may
+    change, and the output must be the decode over that cache and within the bar of the oracle's."""
+    c, b, r = book(d)
+    kernel_option("compress_three_terms", True)
+    cases = (([37, 1, 17, 300, 64, 65, 33, 129], 3), ([1500, 2, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0),
+             ([16, 32, 48, 1], 1), ([4097] * 4, 8))
+    for ci, (lens, splits) in enumerate(cases):
+        q, cache, table, sl, key, value, slots = _serving_case(lens, hq, hkv, d, bs, dtype, seed=300 + ci)
+        dev = [t.to(DEV) for t in (q, table, sl, key, value, slots, c, b, r)]
+        q_d, table_d, sl_d, key_d, value_d, slots_d, c_d, b_d, r_d = dev
+        cache_two = cache.clone().to(DEV)
+        K.tq4_compress_and_store(key_d, value_d, r_d, b_d, cache_two, slots_d)
+        want = K.split_k_paged_decode(q_d, cache_two, table_d, sl_d, c_d, c_d, r_d, hkv, d, bs, num_splits=splits)
+        cache_one = cache.clone().to(DEV)
+        got = K.tq4_store_and_decode(key_d, value_d, slots_d, q_d, cache_one, table_d, sl_d, c_d, c_d, r_d, b_d, hkv, d, bs,
+                                     num_splits=splits)
+        torch.cuda.synchronize()
+        one, two = cache_one.cpu().reshape(-1, hkv * (d + 8)), cache_two.cpu().reshape(-1, hkv * (d + 8))
+        keep = torch.ones(one.shape[0], dtype=torch.bool)
+        keep[slots[slots >= 0]] = False
+        assert torch.equal(one[keep], cache.reshape(-1, hkv * (d + 8))[keep])          # no other row touched
+        rows1, rows2 = one[slots[slots >= 0]], two[slots[slots >= 0]]
+        half = hkv * (d // 2 + 4)
+        for base in (0, half):
+            i1 = O.nibble_unpack(rows1[:, base:base + hkv * (d // 2)].contiguous())
+            i2 = O.nibble_unpack(rows2[:, base:base + hkv * (d // 2)].contiguous())
+            assert (i1 != i2).float().mean().item() <= 1e-4
+            assert (i1.int() - i2.int()).abs().max().item() <= 1
+            n1 = rows1[:, base + hkv * (d // 2):base + half].contiguous().view(torch.float32)
+            n2 = rows2[:, base + hkv * (d // 2):base + half].contiguous().view(torch.float32)
+            assert ((n1 - n2).abs() / n2).max().item() <= 2e-6
+        if torch.equal(rows1, rows2):
+            assert torch.equal(got, want), (lens, splits)
+        # the oracle's step: compress, store, decode
+        kp, kn = O.compress(key.float(), r, b)
+        vp, vn = O.compress(value.float(), r, b)
+        ref_cache = cache.clone()
+        live = (slots >= 0).nonzero().flatten()
+        O.store_rows(ref_cache, slots[live], kp[live], kn[live], vp[live], vn[live])
+        ref = O.split_k_paged_decode(q, ref_cache, table, sl, c, c, r, hkv, d, bs)
+        tol = 2e-2 * max(1.0, ref.float().abs().max().item())
+        assert (got.cpu().float() - ref.float()).abs().max().item() <= tol, (lens, splits)
+        assert (want.cpu().float() - ref.float()).abs().max().item() <= tol
+
+
+def test_store_and_decode_over_several_steps():
+    """Three decode steps in a row on one cache: every step's token is there for the next."""
+    c, b, r = book(128)
+    hq, hkv, d, bs = 32, 8, 128, 16
+    first = [18, 19, 203, 4]                         # lengths at the first step; three steps stay inside the last page
+    q, cache, table, sl, key, value, slots = _serving_case(first, hq, hkv, d, bs, torch.bfloat16, seed=77)
+    cache_d, ref_cache = cache.clone().to(DEV), cache.clone()
+    g = torch.Generator().manual_seed(5)
+    for step in range(3):
+        cur = [L + step for L in first]
+        key = torch.randn(len(cur), hkv, d, generator=g).to(torch.bfloat16)
+        value = torch.randn(len(cur), hkv, d, generator=g).to(torch.bfloat16)
+        qs = torch.randn(len(cur), hq, d, generator=g).to(torch.bfloat16)
+        slots = torch.tensor([int(table[i, (L - 1) // bs]) * bs + (L - 1) % bs for i, L in enumerate(cur)])
+        sl = torch.tensor(cur, dtype=torch.int32)
+        got = K.tq4_store_and_decode(key.to(DEV), value.to(DEV), slots.to(DEV), qs.to(DEV), cache_d, table.to(DEV), sl.to(DEV),
+                                     c.to(DEV), c.to(DEV), r.to(DEV), b.to(DEV), hkv, d, bs)
+        kp, kn = O.compress(key.float(), r, b)
+        vp, vn = O.compress(value.float(), r, b)
+        O.store_rows(ref_cache, slots, kp, kn, vp, vn)
+        ref = O.split_k_paged_decode(qs, ref_cache, table, sl, c, c, r, hkv, d, bs)
+        assert (got.cpu().float() - ref.float()).abs().max().item() <= 2e-2 * max(1.0, ref.float().abs().max().item()), step
+
+
 def test_compress_and_store_rejects_bad_arguments():
     c, bnd, r = book(128)
     key = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device=DEV)

@@ -186,6 +186,16 @@ def test_impl_forward_dispatch(monkeypatch, fresh_plugin):
     assert kw["out"].shape[0] == 3 and kw["out"].data_ptr() == out.data_ptr()
     kernels.prefill.assert_not_called()
 
+    # a pure decode step (one new token per sequence): stored and attended over in one call
+    md1 = MagicMock(num_actual_tokens=3, max_query_len=1, use_cascade=False, seq_lens=torch.tensor([5, 9, 1], dtype=torch.int32),
+                    slot_mapping=torch.tensor([4, 40, 64, -1]))
+    assert impl.forward(None, q, k, v, cache, md1, output=out) is out
+    args, kw = kernels.decode_step.call_args
+    assert [a.shape[0] for a in args[:3]] == [3, 3, 3] and args[3] is cache and args[4].tolist() == [4, 40, 64]
+    assert args[4].dtype == torch.int64 and args[5] is md1.block_table and args[6] is md1.seq_lens
+    assert kw["out"].shape[0] == 3 and kw["out"].data_ptr() == out.data_ptr()
+    assert kernels.compress_and_store.call_count == 1 and kernels.decode.call_count == 1      # not called again
+
     md2 = MagicMock(num_actual_tokens=4, max_query_len=4, use_cascade=False, causal=True)
     impl.forward(None, q, None, None, cache, md2, output=out)                 # nothing new to store
     assert kernels.compress_and_store.call_count == 1
