@@ -852,6 +852,48 @@ def _serving_case(lens, hq, hkv, d, bs, dtype, seed):
     return q, cache, table2, torch.tensor(lens, dtype=torch.int32), key, value, slots
 
 
+def _check_serving_step(lens, hq, hkv, d, bs, dtype, splits, seed):
+    """tq4_store_and_decode against compress-and-store followed by the decode (three-term mode must be on), and
+    against the oracle's compress -> store -> decode."""
+    c, b, r = book(d)
+    q, cache, table, sl, key, value, slots = _serving_case(lens, hq, hkv, d, bs, dtype, seed=seed)
+    dev = [t.to(DEV) for t in (q, table, sl, key, value, slots, c, b, r)]
+    q_d, table_d, sl_d, key_d, value_d, slots_d, c_d, b_d, r_d = dev
+    cache_two = cache.clone().to(DEV)
+    K.tq4_compress_and_store(key_d, value_d, r_d, b_d, cache_two, slots_d)
+    want = K.split_k_paged_decode(q_d, cache_two, table_d, sl_d, c_d, c_d, r_d, hkv, d, bs, num_splits=splits)
+    cache_one = cache.clone().to(DEV)
+    got = K.tq4_store_and_decode(key_d, value_d, slots_d, q_d, cache_one, table_d, sl_d, c_d, c_d, r_d, b_d, hkv, d, bs,
+                                 num_splits=splits)
+    torch.cuda.synchronize()
+    one, two = cache_one.cpu().reshape(-1, hkv * (d + 8)), cache_two.cpu().reshape(-1, hkv * (d + 8))
+    keep = torch.ones(one.shape[0], dtype=torch.bool)
+    keep[slots[slots >= 0]] = False
+    assert torch.equal(one[keep], cache.reshape(-1, hkv * (d + 8))[keep])          # no other row touched
+    rows1, rows2 = one[slots[slots >= 0]], two[slots[slots >= 0]]
+    half = hkv * (d // 2 + 4)
+    for base in (0, half):
+        i1 = O.nibble_unpack(rows1[:, base:base + hkv * (d // 2)].contiguous())
+        i2 = O.nibble_unpack(rows2[:, base:base + hkv * (d // 2)].contiguous())
+        assert (i1 != i2).float().mean().item() <= 1e-4
+        assert (i1.int() - i2.int()).abs().max().item() <= 1
+        n1 = rows1[:, base + hkv * (d // 2):base + half].contiguous().view(torch.float32)
+        n2 = rows2[:, base + hkv * (d // 2):base + half].contiguous().view(torch.float32)
+        assert ((n1 - n2).abs() / n2).max().item() <= 2e-6
+    if torch.equal(rows1, rows2):
+        assert torch.equal(got, want), (lens, splits)
+    # the oracle's step: compress, store, decode
+    kp, kn = O.compress(key.float(), r, b)
+    vp, vn = O.compress(value.float(), r, b)
+    ref_cache = cache.clone()
+    live = (slots >= 0).nonzero().flatten()
+    O.store_rows(ref_cache, slots[live], kp[live], kn[live], vp[live], vn[live])
+    ref = O.split_k_paged_decode(q, ref_cache, table, sl, c, c, r, hkv, d, bs)
+    tol = 2e-2 * max(1.0, ref.float().abs().max().item())
+    assert (got.cpu().float() - ref.float()).abs().max().item() <= tol, (lens, splits)
+    assert (want.cpu().float() - ref.float()).abs().max().item() <= tol
+
+
 @pytest.mark.parametrize("hq,hkv,d,bs,dtype", [(32, 8, 128, 16, torch.bfloat16), (64, 8, 128, 8, torch.float16),
                                                (128, 8, 128, 32, torch.bfloat16), (32, 16, 128, 16, torch.bfloat16),
                                                (32, 4, 128, 16, torch.bfloat16), (8, 2, 64, 16, torch.float16)])
@@ -861,47 +903,50 @@ def test_store_and_decode_equals_store_then_decode(hq, hkv, d, bs, dtype, kernel
     the cache must then hold what compress-and-store writes in its three-term mode (indices equal up to
     coordinates within float32 rounding of a boundary, norms to 2e-6), nothing else in the cache may
     change, and the output must be the decode over that cache and within the bar of the oracle's."""
-    c, b, r = book(d)
     kernel_option("compress_three_terms", True)
     cases = (([37, 1, 17, 300, 64, 65, 33, 129], 3), ([1500, 2, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0),
              ([16, 32, 48, 1], 1), ([4097] * 4, 8))
     for ci, (lens, splits) in enumerate(cases):
-        q, cache, table, sl, key, value, slots = _serving_case(lens, hq, hkv, d, bs, dtype, seed=300 + ci)
-        dev = [t.to(DEV) for t in (q, table, sl, key, value, slots, c, b, r)]
-        q_d, table_d, sl_d, key_d, value_d, slots_d, c_d, b_d, r_d = dev
-        cache_two = cache.clone().to(DEV)
-        K.tq4_compress_and_store(key_d, value_d, r_d, b_d, cache_two, slots_d)
-        want = K.split_k_paged_decode(q_d, cache_two, table_d, sl_d, c_d, c_d, r_d, hkv, d, bs, num_splits=splits)
-        cache_one = cache.clone().to(DEV)
-        got = K.tq4_store_and_decode(key_d, value_d, slots_d, q_d, cache_one, table_d, sl_d, c_d, c_d, r_d, b_d, hkv, d, bs,
-                                     num_splits=splits)
+        _check_serving_step(lens, hq, hkv, d, bs, dtype, splits, seed=300 + ci)
+
+
+def test_store_and_decode_in_a_captured_graph():
+    """The serving step recorded into a graph (caller workspace and output, nothing allocated) and replayed with
+    new keys, values and queries in the recorded tensors, the program's own eager work in between: every replay
+    must give what the eager call gives on the same inputs."""
+    C = load_native()
+    c, b, r = book(128)
+    hq, hkv, d, bs = 32, 8, 128, 16
+    lens = [100, 17, 1, 2500]
+    q, cache, table, sl, key, value, slots = _serving_case(lens, hq, hkv, d, bs, torch.bfloat16, seed=501)
+    ev, od = O.split_rotation(r)
+    st = [t.to(DEV).contiguous() for t in (key, value, slots, ev, od, b, q, table, sl, c, r)]
+    key_s, value_s, slots_s, ev_d, od_d, b_d, q_s, table_d, sl_d, c_d, r_d = st
+    cache_g = cache.clone().to(DEV)
+    out_g = torch.empty_like(q_s)
+    ws = torch.empty(C.paged_decode_workspace_bytes(len(lens), hq, hkv, d, bs, table.shape[1], 4), dtype=torch.uint8, device=DEV)
+
+    def step(cache_t, out_t):
+        C.tq4_store_and_decode(key_s, value_s, slots_s, ev_d, od_d, b_d, q_s, cache_t, table_d, sl_d, c_d, c_d, r_d, hkv, d, bs,
+                               None, out_t, 4, ws)
+
+    step(cache_g, out_g)                                   # first call outside the capture (runtime set-up)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(cache_g, out_g)
+    g = torch.Generator().manual_seed(9)
+    for rep in range(3):
+        key_s.copy_(torch.randn(key.shape, generator=g).to(torch.bfloat16))
+        value_s.copy_(torch.randn(value.shape, generator=g).to(torch.bfloat16))
+        q_s.copy_(torch.randn(q.shape, generator=g).to(torch.bfloat16))
+        graph.replay()
         torch.cuda.synchronize()
-        one, two = cache_one.cpu().reshape(-1, hkv * (d + 8)), cache_two.cpu().reshape(-1, hkv * (d + 8))
-        keep = torch.ones(one.shape[0], dtype=torch.bool)
-        keep[slots[slots >= 0]] = False
-        assert torch.equal(one[keep], cache.reshape(-1, hkv * (d + 8))[keep])          # no other row touched
-        rows1, rows2 = one[slots[slots >= 0]], two[slots[slots >= 0]]
-        half = hkv * (d // 2 + 4)
-        for base in (0, half):
-            i1 = O.nibble_unpack(rows1[:, base:base + hkv * (d // 2)].contiguous())
-            i2 = O.nibble_unpack(rows2[:, base:base + hkv * (d // 2)].contiguous())
-            assert (i1 != i2).float().mean().item() <= 1e-4
-            assert (i1.int() - i2.int()).abs().max().item() <= 1
-            n1 = rows1[:, base + hkv * (d // 2):base + half].contiguous().view(torch.float32)
-            n2 = rows2[:, base + hkv * (d // 2):base + half].contiguous().view(torch.float32)
-            assert ((n1 - n2).abs() / n2).max().item() <= 2e-6
-        if torch.equal(rows1, rows2):
-            assert torch.equal(got, want), (lens, splits)
-        # the oracle's step: compress, store, decode
-        kp, kn = O.compress(key.float(), r, b)
-        vp, vn = O.compress(value.float(), r, b)
-        ref_cache = cache.clone()
-        live = (slots >= 0).nonzero().flatten()
-        O.store_rows(ref_cache, slots[live], kp[live], kn[live], vp[live], vn[live])
-        ref = O.split_k_paged_decode(q, ref_cache, table, sl, c, c, r, hkv, d, bs)
-        tol = 2e-2 * max(1.0, ref.float().abs().max().item())
-        assert (got.cpu().float() - ref.float()).abs().max().item() <= tol, (lens, splits)
-        assert (want.cpu().float() - ref.float()).abs().max().item() <= tol
+        cache_e, out_e = cache.clone().to(DEV), torch.empty_like(q_s)
+        step(cache_e, out_e)                               # eager, on a fresh copy of the cache
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e), rep
+        assert torch.equal(cache_g, cache_e), rep
 
 
 def test_store_and_decode_over_several_steps():

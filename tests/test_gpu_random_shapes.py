@@ -12,6 +12,7 @@ import torch
 
 from tests import test_gpu_parity as P
 from tests.gpu_util import book
+from tests.test_gpu_parity import kernel_option  # noqa: F401  (fixture)
 
 pytestmark = pytest.mark.gpu
 
@@ -38,6 +39,28 @@ def test_random_paged_decode(case):
         lens[0] = 5
     P._decode_case(lens, hq=hq, hkv=hkv, d=d, bs=rng.choice([8, 16, 16, 32]), dtype=rng.choice([torch.bfloat16, torch.float16]),
                    num_splits=rng.choice([0, 1, 2, 3, 5, 8, 17]), seed=100 + case)
+
+
+@pytest.mark.parametrize("case", range(30))
+def test_random_store_and_decode(case, kernel_option):
+    """The serving step (new token stored, then decoded over) on random shapes: the in-launch store where the
+    staged kernel runs, the two launches elsewhere."""
+    kernel_option("compress_three_terms", True)
+    rng = random.Random(9500 + case)
+    d = rng.choice([128, 128, 128, 128, 64, 256])
+    hkv = rng.choice([8, 8, 8, 16, 24, 4, 2]) if d == 128 else rng.choice([8, 4, 2])
+    g = rng.choice([1, 2, 4, 4, 5, 8, 16]) if d != 256 else rng.choice([1, 2, 4])
+    n_seq = rng.choice([1, 2, 3, 5, 9, 17, 33])
+    longest = rng.choice([40, 130, 300, 700, 1500, 3000])
+    if n_seq > 9:
+        longest = min(longest, 700)
+    lens = [rng.randint(1, longest) for _ in range(n_seq)]
+    if rng.random() < 0.3:
+        lens[rng.randrange(n_seq)] = 0                      # a sequence with nothing to store (slot -1)
+    if max(lens) == 0:
+        lens[0] = 7
+    P._check_serving_step(lens, hkv * g, hkv, d, rng.choice([8, 16, 16, 32]), rng.choice([torch.bfloat16, torch.float16]),
+                          rng.choice([0, 1, 2, 3, 5, 8, 17]), seed=700 + case)
 
 
 @pytest.mark.parametrize("case", range(40))
