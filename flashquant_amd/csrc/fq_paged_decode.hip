@@ -647,7 +647,7 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
 template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false, bool STORE = false>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
-    static_assert(!STORE || (CW > 0 && !HALF && !PROD), "the new token is stored by the TQ4 form with copy wavefronts");
+    static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
     using Cfg = StagedCfg<PROD>;
     constexpr int kStageBytes = Cfg::STAGE_BYTES;
     constexpr int kTileBytes = Cfg::TILE_BYTES;
@@ -1089,13 +1089,18 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             }
             if constexpr (STORE) {
                 if (stores_token) {
-                    // ---- the new token: TQ4 compress of its 8 key and 8 value rows (one more block of 16
-                    // rows for the same matrix product) straight into the cache row: n = ||x||,
+                    // ---- the new token: TQ4 compress of its key and value rows (KH of each: one more block of
+                    // 16 rows for the same matrix product) straight into the cache row: n = ||x||,
                     // y = (x R^T) / (n + 1e-10), index = number of boundaries below y, two indices per byte
                     // (cpu_reference.py:22-61, vllm/impl.py:220-263).  Wavefront h holds columns 16h..16h+15.
+                    // Block row r: key head r for r < KH, value head r - KH for r < 2 KH.
+                    constexpr int KH = HALF ? 4 : 8;             // KV heads of this workgroup
+                    const int token_row_bytes = HALF ? 544 : row_bytes;
+                    const int kv_heads = HALF ? 4 : p.H_KV;
                     const int64_t slot = p.new_slots[seq];
-                    const uint16_t* xrow = reinterpret_cast<const uint16_t*>(n < 8 ? p.new_key : p.new_value) +
-                                           (int64_t(seq) * p.H_KV + 8 * hgrp + (n & 7)) * D;
+                    const int nr = n < 2 * KH ? n : 2 * KH - 1;
+                    const uint16_t* xrow = reinterpret_cast<const uint16_t*>(nr < KH ? p.new_key : p.new_value) +
+                                           (int64_t(seq) * kv_heads + KH * hgrp + (nr & (KH - 1))) * D;
                     uint4v raw[KS];
 #pragma unroll
                     for (int j = 0; j < KS; ++j) raw[j] = *reinterpret_cast<const uint4v*>(xrow + 32 * j + 8 * g);
@@ -1126,10 +1131,10 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                         acc = rotate_block_f16<D>(a, rot_hi, rot_lo);
                     }
                     const bool stored = slot >= 0 && slot < p.num_slots;
-                    uint8_t* crow = p.cache_rw + (stored ? slot : 0) * int64_t(row_bytes);
+                    uint8_t* crow = p.cache_rw + (stored ? slot : 0) * int64_t(token_row_bytes);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int r = 4 * g + i;                     // row of the block: key head r, or value head r - 8
+                        const int r = 4 * g + i;                     // row of the block
                         const float ssr = __shfl(ss, r, kWave);
                         const bool tiny = ssr < 0x1p-96f;            // as the compress kernel: v_sqrt_f32 on a normal number
                         const float nrm_s = __builtin_amdgcn_sqrtf(tiny ? ssr * 0x1p64f : ssr);
@@ -1149,12 +1154,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                             lo |= uint32_t(__shfl_xor(int(lo), mask, kWave));
                             hi |= uint32_t(__shfl_xor(int(hi), mask, kWave));
                         }
-                        const int head = 8 * hgrp + (r & 7);
-                        const int sect = r < 8 ? 0 : p.H_KV * (D / 2 + 4);               // key sections, then value sections
-                        if (stored && n == 0)
+                        const int head = KH * hgrp + (r & (KH - 1));
+                        const int sect = r < KH ? 0 : kv_heads * (D / 2 + 4);            // key sections, then value sections
+                        const bool row_live = stored && r < 2 * KH;
+                        if (row_live && n == 0)
                             *reinterpret_cast<uint2v*>(crow + sect + head * (D / 2) + 8 * h) = uint2v{lo, hi};
-                        if (stored && n == 1 && h == 0)
-                            *reinterpret_cast<float*>(crow + sect + p.H_KV * (D / 2) + 4 * head) = nrm;
+                        if (row_live && n == 1 && h == 0)
+                            *reinterpret_cast<float*>(crow + sect + kv_heads * (D / 2) + 4 * head) = nrm;
                     }
                     // the row is in the cache before the copy wavefronts ask for it
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1794,7 +1800,11 @@ template <int DT>
 int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wide, hipStream_t stream) {
     const size_t lds = 2 * size_t(StagedCfg<false>::TILE_BYTES);
     const dim3 grid(S, p.num_splits, 1), block(512 + 64 * 4);
+    const bool store = p.new_key != nullptr;
 #define FQ_HALF_GP(BSL, GPV)                                                                                      \
+    if (store)                                                                                                    \
+        return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, true, true>, p, grid, block, lds, stream) \
+                    : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, true, true>, p, grid, block, lds, stream); \
     return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, true>, p, grid, block, lds, stream) \
                 : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, true>, p, grid, block, lds, stream)
 #define FQ_HALF_BS(BSL)                          \
@@ -1812,7 +1822,6 @@ int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wid
 template <int D, int DT>
 int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bool allow_half, const DecodeVariant& var) {
     if (allow_half && staged_half_applies(D, p.H_KV, BS, var)) {
-        if (p.new_key != nullptr) return FQ_ERR_LAUNCH;
         // the kernel counts rows of two tokens: half the page size, chunks of rows
         const int rows_per_page = BS / 2;
         const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
@@ -2202,7 +2211,8 @@ extern "C" int fq_tq4_store_and_decode(const void* key, const void* value, const
         !fq_host::aligned(kv_cache, 16) || !fq_host::aligned(boundaries, 4))
         return FQ_ERR_MISALIGNED;
     const DecodeVariant var = read_decode_variant();
-    const bool in_launch = centroids_k && staged_applies(D, H_KV, var) && !var.ring && var.copy_waves == 4;
+    const bool in_launch = centroids_k && var.copy_waves == 4 &&
+                           ((staged_applies(D, H_KV, var) && !var.ring) || staged_half_applies(D, H_KV, block_size, var));
     const NewToken token{key, value, slot_mapping, boundaries, kv_cache};
     if (!in_launch) {
         const int st = fq_tq4_compress_store(key, value, dtype, rot_T_even, rot_T_odd, boundaries, kv_cache, slot_mapping,
