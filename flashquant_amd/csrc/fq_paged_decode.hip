@@ -836,6 +836,22 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         load_matrix_columns();
         load_first_heads();
     }
+    // STORE: the new token's rows and slot are asked for with the other prologue loads, by every workgroup
+    // (which one needs them depends on the sequence length, which is on its way)
+    constexpr int kNewHeads = HALF ? 4 : 8;                 // KV heads of this workgroup
+    uint4v new_raw[4];
+    int64_t new_slot = -1;
+    if constexpr (STORE) {
+        if (!copier) {
+            const int kv_heads = HALF ? 4 : p.H_KV;
+            const int nr = n < 2 * kNewHeads ? n : 2 * kNewHeads - 1;     // block row: key head nr, or value head nr - KH
+            const uint16_t* xrow = reinterpret_cast<const uint16_t*>(nr < kNewHeads ? p.new_key : p.new_value) +
+                                   (int64_t(seq) * kv_heads + kNewHeads * hgrp + (nr & (kNewHeads - 1))) * 128;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) new_raw[j] = *reinterpret_cast<const uint4v*>(xrow + 32 * j + 8 * g);
+            new_slot = p.new_slots[seq];
+        }
+    }
     L = L < 0 ? 0 : L;
     L = L > p.max_blocks * BS * (HALF ? 2 : 1) ? p.max_blocks * BS * (HALF ? 2 : 1) : L;
     // HALF: from here on L counts rows (token pairs); a wavefront's last row may hold a token of the
@@ -1094,16 +1110,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                     // y = (x R^T) / (n + 1e-10), index = number of boundaries below y, two indices per byte
                     // (cpu_reference.py:22-61, vllm/impl.py:220-263).  Wavefront h holds columns 16h..16h+15.
                     // Block row r: key head r for r < KH, value head r - KH for r < 2 KH.
-                    constexpr int KH = HALF ? 4 : 8;             // KV heads of this workgroup
+                    constexpr int KH = kNewHeads;
                     const int token_row_bytes = HALF ? 544 : row_bytes;
                     const int kv_heads = HALF ? 4 : p.H_KV;
-                    const int64_t slot = p.new_slots[seq];
-                    const int nr = n < 2 * KH ? n : 2 * KH - 1;
-                    const uint16_t* xrow = reinterpret_cast<const uint16_t*>(nr < KH ? p.new_key : p.new_value) +
-                                           (int64_t(seq) * kv_heads + KH * hgrp + (nr & (KH - 1))) * D;
+                    const int64_t slot = new_slot;
                     uint4v raw[KS];
 #pragma unroll
-                    for (int j = 0; j < KS; ++j) raw[j] = *reinterpret_cast<const uint4v*>(xrow + 32 * j + 8 * g);
+                    for (int j = 0; j < KS; ++j) raw[j] = new_raw[j];
                     const float bnd_mine = p.boundaries[lane < 15 ? lane : 14];
                     float ss = 0.0f;         // sum of squares of row n: this lane's 32 elements, then over g
 #pragma unroll
@@ -1162,9 +1175,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                         if (row_live && n == 1 && h == 0)
                             *reinterpret_cast<float*>(crow + sect + kv_heads * (D / 2) + 4 * head) = nrm;
                     }
-                    // the row is in the cache before the copy wavefronts ask for it
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                    lds_flag_signal(&flags[7], lane);
+                    // The row must be in the cache before the copy wavefronts ask for the split's last tile.  They
+                    // ask for the first two tiles at once; when the last tile is one of those the stores are waited
+                    // for here, otherwise after the first tile's arithmetic, when they have long completed.
+                    if (last_t0 < begin + 64) {
+                        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                        lds_flag_signal(&flags[7], lane);
+                    }
                 }
             }
             if constexpr (CW > 0) {
@@ -1443,6 +1460,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 handoff_failed = true;
             }
             compute_tile(t0, i & 1);
+            if constexpr (STORE) {
+                if (i == 0 && stores_token && last_t0 >= begin + 64) {      // (see the prologue)
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    lds_flag_signal(&flags[7], lane);
+                }
+            }
         }
     }
 
