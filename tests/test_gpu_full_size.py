@@ -194,6 +194,49 @@ def test_prod_paged_decode_on_long_ragged_contexts():
     assert math.isfinite(err) and err <= 2e-2, f"max abs error {err}"
 
 
+def test_serving_step_at_the_benchmark_size():
+    """The benchmark's serving step: batch 32, 4096 tokens of context of which the last is the step's new token,
+    stored and attended over in one call (fq_tq4_store_and_decode).  The oracle stores its own compress of the
+    same rows and decodes; every sequence is compared."""
+    c, b, r = book(128)
+    B, L, hq, hkv, bs = 32, 4096, 32, 8, 16
+
+    def rows(s, n):
+        return outlier_rows(n, hkv, 128, 6000 + 2 * s), outlier_rows(n, hkv, 128, 6001 + 2 * s)
+
+    # the cache holds tokens 0 .. L - 2; position L - 1 holds the bytes of an older token until the step writes it
+    cache, table, _ = _store_sequences([L] * B, rows, hkv, 128, bs, seed=2003, extra_blocks=3)
+    slots = (table.long()[:, (L - 1) // bs] * bs + (L - 1) % bs).contiguous()
+    key = outlier_rows(B, hkv, 128, 7001).to(torch.bfloat16)
+    value = outlier_rows(B, hkv, 128, 7002).to(torch.bfloat16)
+    q = torch.randn(B, hq, 128, generator=torch.Generator().manual_seed(1003)).to(torch.bfloat16)
+    sl = torch.full((B,), L, dtype=torch.int32)
+    ref_cache = cache.clone()
+    kp, kn = O.compress(key.float(), r, b)
+    vp, vn = O.compress(value.float(), r, b)
+    O.store_rows(ref_cache, slots, kp, kn, vp, vn)
+    want = O.split_k_paged_decode(q, ref_cache, table, sl, c, c, r, hkv, 128, bs)
+    cache_d, cd = cache.to(DEV), c.to(DEV)
+    got = K.tq4_store_and_decode(key.to(DEV), value.to(DEV), slots.to(DEV), q.to(DEV), cache_d, table.to(DEV), sl.to(DEV),
+                                 cd, cd, r.to(DEV), b.to(DEV), hkv, 128, bs)
+    torch.cuda.synchronize()
+    assert torch.isfinite(got).all()
+    row_scale = want.float().abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+    rel = ((got.cpu().float() - want.float()).abs() / row_scale).max().item()
+    assert rel <= 2e-2, f"max error {rel} of the row magnitude"
+    # the stored rows against the oracle's: at most 1e-4 of the indices differ, by one bucket; the rest of the cache untouched
+    flat_got, flat_ref = cache_d.cpu().reshape(-1, hkv * 136), ref_cache.reshape(-1, hkv * 136)
+    keep = torch.ones(flat_got.shape[0], dtype=torch.bool)
+    keep[slots] = False
+    assert torch.equal(flat_got[keep], flat_ref[keep])
+    half = hkv * 68
+    for base in (0, half):
+        i1 = O.nibble_unpack(flat_got[slots][:, base:base + hkv * 64].contiguous())
+        i2 = O.nibble_unpack(flat_ref[slots][:, base:base + hkv * 64].contiguous())
+        assert (i1 != i2).float().mean().item() <= 1e-4
+        assert (i1.int() - i2.int()).abs().max().item() <= 1
+
+
 def test_prod_paged_decode_at_the_benchmark_batch():
     """The long-context workload at its real batch: 8 sequences, lengths drawn uniformly from 16K to
     128K tokens with seed 1004, 64 query heads over 8 KV heads, N(0,1) rows with outlier channels.
