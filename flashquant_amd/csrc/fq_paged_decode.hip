@@ -521,13 +521,19 @@ __global__ __launch_bounds__(D == 256 ? 256 : 512) void paged_decode_kernel(cons
 // carries a second float32, the residual norm, so a token row is
 // [K nibbles H*64 | K norm H*4 | K residual norm H*4 | V idx H*64 | V norm H*4] = H*140 bytes
 // and a stage grows by 512 bytes of residual norms.
-template <bool PROD>
+// D64 (head_dim 64, TQ4 pages): two neighbouring KV heads of 64 coordinates are served as one "head" of 128
+// (their index bytes are contiguous in the token row), with two norms each for K and V: a row of 8 such
+// heads is 16 real heads, 72 chunks.
+template <bool PROD, bool D64 = false>
 struct StagedCfg {
-    static constexpr int CHUNKS_PER_ROW = PROD ? 70 : 68;          // 16-byte chunks of a token row, 8 heads
-    static constexpr int ROWB = 16 * CHUNKS_PER_ROW;               // 1088 / 1120
-    static constexpr int STAGE_BYTES = 16 * ROWB;                  // 17408 / 17920
+    static constexpr int CHUNKS_PER_ROW = PROD ? 70 : (D64 ? 72 : 68);   // 16-byte chunks of a token row, 8 heads
+    static constexpr int ROWB = 16 * CHUNKS_PER_ROW;               // 1088 / 1120 / 1152
+    static constexpr int STAGE_BYTES = 16 * ROWB;                  // 17408 / 17920 / 18432
     static constexpr int TILE_BYTES = 2 * STAGE_BYTES;             // 32 tokens
-    static constexpr int CHUNKS_PER_TILE = 32 * CHUNKS_PER_ROW;    // 2176 / 2240
+    static constexpr int CHUNKS_PER_TILE = 32 * CHUNKS_PER_ROW;    // 2176 / 2240 / 2304
+    static constexpr int NORM_BYTES = D64 ? 64 : 32;               // K (or V) norms of a row
+    static constexpr int KN_OFF = 16384;                           // K norms of the stage's 16 rows
+    static constexpr int VN_OFF = KN_OFF + 16 * NORM_BYTES;        // V norms
 };
 constexpr int kStageKnOff = 16384;
 constexpr int kStageVnOff = 16896;
@@ -539,10 +545,18 @@ __host__ __device__ constexpr int staged_slot(int h, int r, int q) {
 }
 
 // LDS byte offset (inside a tile slot) of the 16-byte chunk `ci` of tile row `row` (0..31).
-template <bool PROD>
+template <bool PROD, bool D64 = false>
 __host__ __device__ constexpr int staged_chunk_dst(int row, int ci) {
     const int stage = row >> 4, r = row & 15;
     int off = 0;
+    if (D64) {
+        using C = StagedCfg<false, true>;
+        if (ci < 32) off = 16 * staged_slot(ci >> 2, r, ci & 3);
+        else if (ci < 36) off = C::KN_OFF + 64 * r + 16 * (ci - 32);
+        else if (ci < 68) off = 8192 + 16 * staged_slot((ci - 36) >> 2, r, (ci - 36) & 3);
+        else off = C::VN_OFF + 64 * r + 16 * (ci - 68);
+        return stage * C::STAGE_BYTES + off;
+    }
     if (ci < 32) {
         off = 16 * staged_slot(ci >> 2, r, ci & 3);
     } else if (ci < 34) {
@@ -559,16 +573,17 @@ __host__ __device__ constexpr int staged_chunk_dst(int row, int ci) {
 
 // The same offsets for every chunk of a tile, worked out at compile time: a thread reads its
 // five entries instead of dividing by the row length and walking the layout.
-template <bool PROD>
+template <bool PROD, bool D64 = false>
 struct ChunkDstTable {
-    uint16_t off[StagedCfg<PROD>::CHUNKS_PER_TILE];
+    uint16_t off[StagedCfg<PROD, D64>::CHUNKS_PER_TILE];
     constexpr ChunkDstTable() : off() {
-        for (int c = 0; c < StagedCfg<PROD>::CHUNKS_PER_TILE; ++c)
-            off[c] = uint16_t(staged_chunk_dst<PROD>(c / StagedCfg<PROD>::CHUNKS_PER_ROW, c % StagedCfg<PROD>::CHUNKS_PER_ROW));
+        for (int c = 0; c < StagedCfg<PROD, D64>::CHUNKS_PER_TILE; ++c)
+            off[c] = uint16_t(staged_chunk_dst<PROD, D64>(c / StagedCfg<PROD, D64>::CHUNKS_PER_ROW,
+                                                          c % StagedCfg<PROD, D64>::CHUNKS_PER_ROW));
     }
 };
-template <bool PROD>
-__device__ const ChunkDstTable<PROD> kChunkDst{};
+template <bool PROD, bool D64 = false>
+__device__ const ChunkDstTable<PROD, D64> kChunkDst{};
 
 // TurboQuantProd sign operand: the fp16 pairs (+-1, +-1) of the eight sign bits (bit 3 of
 // every nibble) of one key dword.  Element e of the result belongs to the coordinate
@@ -615,10 +630,27 @@ __device__ unsigned int g_decode_faults = 0u;
 // HALF (4 KV heads): the kernel works on rows of 8 "heads" made of two consecutive tokens, head h of
 // the even token as head h and of the odd token as head 4 + h, so row r is the real rows 2 r and
 // 2 r + 1 (544 bytes each) with their sections interleaved; a page then holds half as many rows.
-template <bool PROD, bool HALF>
+template <bool PROD, bool HALF, bool D64 = false>
 __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
-    constexpr int CPR = StagedCfg<PROD>::CHUNKS_PER_ROW;
+    constexpr int CPR = StagedCfg<PROD, D64>::CHUNKS_PER_ROW;
     const int r = cc / CPR, ci = cc - r * CPR;
+    if constexpr (D64) {
+        // head_dim 64, H real heads: [K idx H*32 | K norms H*4 | V idx H*32 | V norms H*4] = 72 H bytes a token
+        if constexpr (HALF) {      // 8 real heads: a row is two tokens of 576 bytes
+            int tok, off;
+            if (ci < 32) { tok = ci >> 4; off = 16 * (ci & 15); }                            // K indices, 256 bytes per token
+            else if (ci < 36) { tok = (ci - 32) >> 1; off = 256 + 16 * ((ci - 32) & 1); }    // K norms, 32 bytes
+            else if (ci < 68) { tok = (ci - 36) >> 4; off = 288 + 16 * ((ci - 36) & 15); }   // V indices
+            else { tok = (ci - 68) >> 1; off = 544 + 16 * ((ci - 68) & 1); }                 // V norms
+            return uint32_t((2 * r + tok) * 576 + off);
+        }
+        int off;                   // group hgrp of 16 real heads
+        if (ci < 32) off = 512 * hgrp + 16 * ci;
+        else if (ci < 36) off = H * 32 + 64 * hgrp + 16 * (ci - 32);
+        else if (ci < 68) off = H * 36 + 512 * hgrp + 16 * (ci - 36);
+        else off = H * 68 + 64 * hgrp + 16 * (ci - 68);
+        return uint32_t(r * (H * 72) + off);
+    }
     if constexpr (PROD) {                                  // five sections: K nibbles, K norms, K residual norms, V idx, V norms
         int off;
         if (ci < 32) off = 512 * hgrp + 16 * ci;
@@ -644,11 +676,16 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     return uint32_t(r * (H * 136) + off);
 }
 
-template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false, bool STORE = false>
+template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false, bool STORE = false, bool D64 = false>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
-    using Cfg = StagedCfg<PROD>;
+    static_assert(!D64 || (!PROD && !STORE && CW > 0), "head_dim 64 is served by the TQ4 form with copy wavefronts");
+    // D64: the kernel's "heads" are pairs of real heads of 64 coordinates, and p.G is twice the real group size: the
+    // query heads of a pair are those of its first head followed by those of its second.  A query row is the real
+    // row in the half of its head and zeros in the other; its scores and outputs then are the real ones, with the
+    // norms of its own head and the output coordinates of its own half.
+    using Cfg = StagedCfg<PROD, D64>;
     constexpr int kStageBytes = Cfg::STAGE_BYTES;
     constexpr int kTileBytes = Cfg::TILE_BYTES;
     constexpr int kChunksPerRow = Cfg::CHUNKS_PER_ROW;
@@ -692,7 +729,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     const int hgrp = blockIdx.z;
     const int HQG = (HALF ? 4 : 8) * p.G;      // query heads of a group
     const int hq0 = hgrp * HQG;
-    const int row_bytes = HALF ? 1088 : p.H_KV * (PROD ? 140 : 136);   // a row of the cache as the kernel sees it
+    const int row_bytes = D64 ? (HALF ? 1152 : p.H_KV * 72)
+                              : (HALF ? 1088 : p.H_KV * (PROD ? 140 : 136));   // a row of the cache as the kernel sees it
+    const int qsub = D64 && (n % GP) >= p.G / 2 ? 1 : 0;    // D64: this lane's query head belongs to the pair's second head
     // HALF: wavefront h works on real head h % 4 and on the tokens of parity h / 4 (rows are token pairs)
     const int hr = HALF ? (h & 3) : h;
     const int tsel = HALF ? (h >> 2) & 1 : 0;
@@ -712,7 +751,17 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     float rot_s[4][8];
     auto load_matrix_columns = [&]() {
         if (p.rotation != nullptr && !copier) {
-            load_rotation_any<128>(p.rotation, p.rot_col_major != 0, true, 16 * h, n, g, rot_b);
+            if constexpr (D64) {
+                // the 64 x 64 matrix twice on the diagonal of the 128 x 128 one: wavefront h has columns 16 h .. 16 h + 15
+                float b64[2][8];
+                load_rotation_any<64>(p.rotation, p.rot_col_major != 0, true, 16 * (h & 3), n, g, b64);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) rot_b[j][e] = (j >> 1) == (h >> 2) ? b64[j & 1][e] : 0.0f;
+            } else {
+                load_rotation_any<128>(p.rotation, p.rot_col_major != 0, true, 16 * h, n, g, rot_b);
+            }
             if constexpr (PROD) load_rotation_any<128>(p.sketch, false, true, 16 * h, n, g, rot_s);
         }
     };
@@ -748,8 +797,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
         src_page[k] = pg;
         const int sub = (kSpreadTail && k == 4) ? 4 * (tid & 3) : 0;
-        src_off[k] = staged_src_offset<PROD, HALF>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
-        dst_off[k] = kChunkDst<PROD>.off[c] + sub;
+        src_off[k] = staged_src_offset<PROD, HALF, D64>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+        dst_off[k] = kChunkDst<PROD, D64>.off[c] + sub;
     }
     const bool has_round4 = kSpreadTail || tid < kChunksPerTile - 4 * 512;   // else whole wavefronts
     // ---- lane-constant LDS read offsets (inside a tile slot) -------------------------------
@@ -772,7 +821,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         else if (GP == 8) { blk = cls; row = 4 * g + e; }
         else { blk = e >> 2; row = 4 * g + (e & 3); }
         sc_tok[e] = 16 * blk + row;
-        n_rd[e] = blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
+        n_rd[e] = D64 ? blk * kStageBytes + Cfg::KN_OFF + 64 * row + 8 * h + 4 * qsub
+                      : blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
     }
 
     // dword d of the P operand holds slots 2d, 2d + 1: it is this lane's when its class owns them
@@ -796,7 +846,19 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     int L_known = -1;
     if (p.balance_slots > 0) balance_chunks<PVR, BS, HALF>(p, lane, NS, rowwide, chunk, seq, split, L_known);
 
-    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + (int64_t(seq) * p.H_Q + hq0) * 128;
+    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + (int64_t(seq) * p.H_Q + hq0) * (D64 ? 64 : 128);
+    // eight elements of query row `row` of this workgroup, from element `v` (a multiple of 8) of the 128 the kernel
+    // works on.  D64: the real row of 64 in the half of its head, zeros in the other half.
+    auto q_chunk = [&](int row, int v) -> uint4v {
+        if constexpr (!D64) {
+            return *reinterpret_cast<const uint4v*>(qseq + row * 128 + v);
+        } else {
+            const int in_group = row - (row / p.G) * p.G;
+            const int row_sub = in_group >= p.G / 2 ? 1 : 0;
+            const uint4v x = *reinterpret_cast<const uint4v*>(qseq + row * 64 + (v & 63));
+            return (v >> 6) == row_sub ? x : uint4v{0u, 0u, 0u, 0u};
+        }
+    };
     uint4v q_pre[2][4];
     auto load_first_heads = [&]() {
         if (p.rotation != nullptr && !copier) {
@@ -804,7 +866,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             for (int rb = 0; rb < 2; ++rb) {
                 const int row = 16 * rb + n < HQG ? 16 * rb + n : HQG - 1;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) q_pre[rb][j] = *reinterpret_cast<const uint4v*>(qseq + row * 128 + 32 * j + 8 * g);
+                for (int j = 0; j < 4; ++j) q_pre[rb][j] = q_chunk(row, 32 * j + 8 * g);
             }
         }
     };
@@ -947,7 +1009,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             constexpr int FULL = kChunksPerTile / CT;
             constexpr int REST = kChunksPerTile - FULL * CT;
             constexpr bool kHalfTail = REST * 2 == CT;   // else whole chunks by the first REST threads
-            constexpr int NR = FULL + 1;
+            constexpr int NR = REST > 0 ? FULL + 1 : FULL;   // register sets of a tile: the whole rounds and the rest
             const int ct = tid - 512;
             uint32_t c_src[NR];
             int c_page[NR];
@@ -962,8 +1024,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
                 c_page[k] = pg;
                 const int sub = (k < FULL || !kHalfTail) ? 0 : 8 * (ct & 1);
-                c_src[k] = staged_src_offset<PROD, HALF>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
-                c_dst[k] = kChunkDst<PROD>.off[c] + sub;
+                c_src[k] = staged_src_offset<PROD, HALF, D64>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+                c_dst[k] = kChunkDst<PROD, D64>.off[c] + sub;
             }
             const bool has_rest = kHalfTail || ct < REST;
             auto c_issue = [&](uint4v (&r)[NR], int t0) {
@@ -1074,8 +1136,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 uint4v raw[KS];
 #pragma unroll
                 for (int j = 0; j < KS; ++j)
-                    raw[j] = rb < 2 ? q_pre[rb & 1][j]
-                                    : *reinterpret_cast<const uint4v*>(qseq + row * D + 32 * j + 8 * g);
+                    raw[j] = rb < 2 ? q_pre[rb & 1][j] : q_chunk(row, 32 * j + 8 * g);
                 float4v acc, acc2 = {0.f, 0.f, 0.f, 0.f};
                 float up = 1.0f;
                 if constexpr (kRawBf16) {
@@ -1228,10 +1289,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             if constexpr (CW > 0) lds_flag_signal(&flags[1], lane);
             else if constexpr (PROD) __syncthreads();
         } else {
-            const uint16_t* qsrc = qseq + (hr * p.G + (live ? hd : 0)) * D + g * (D / 4);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const uint4v raw = *reinterpret_cast<const uint4v*>(qsrc + 8 * ks);
+                const uint4v raw = q_chunk(hr * p.G + (live ? hd : 0), g * (D / 4) + 8 * ks);
                 const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -1274,7 +1334,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
         for (int e = 0; e < NSC; ++e) {
             kn[e] = *reinterpret_cast<const float*>(tile + n_rd[e]);
-            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageVnOff - kStageKnOff));
+            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (D64 ? Cfg::VN_OFF - Cfg::KN_OFF : kStageVnOff - kStageKnOff));
             kg[e] = PROD ? *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageKgOff - kStageKnOff)) : 0.0f;
         }
         // These were all the reads of the slot (the lookups below go to the table): it is handed back
@@ -1502,8 +1562,11 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int head = 4 * g + i;
-            if (head < p.G) {
-                float* dst = p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS_out + split_out) * D + n * DPL;
+            // D64: a query head's output is the half of the 128 coordinates that belongs to its own head of 64
+            const bool mine = !D64 || (n >> 3) == (head >= p.G / 2 ? 1 : 0);
+            if (head < p.G && mine) {
+                float* dst = D64 ? p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS_out + split_out) * 64 + (n & 7) * DPL
+                                 : p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS_out + split_out) * D + n * DPL;
 #pragma unroll
                 for (int q4 = 0; q4 < DPL / 4; ++q4) {
                     const float4v v = {O[4 * q4][i], O[4 * q4 + 1][i], O[4 * q4 + 2][i], O[4 * q4 + 3][i]};
@@ -1842,8 +1905,56 @@ int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wid
 #undef FQ_HALF_GP
 }
 
+// head_dim 64 on the staged kernel: pairs of neighbouring KV heads as heads of 128 (16 real heads a group), or, with
+// 8 KV heads on pages of 16 or 32 tokens, rows of two tokens of four such pairs.  Up to 8 query heads per KV head.
+inline bool staged_d64_full_applies(int D, int H_KV, int G, const DecodeVariant& v) {
+    return D == 64 && H_KV % 16 == 0 && G <= 8 && !v.direct && v.copy_waves == 4;
+}
+inline bool staged_d64_half_applies(int D, int H_KV, int G, int block_size, const DecodeVariant& v) {
+    return D == 64 && H_KV == 8 && G <= 8 && block_size >= 16 && !v.direct && v.copy_waves == 4;
+}
+template <int DT>
+int launch_staged_d64(const DecodeParams& p, int S, int rows_per_page, bool wide, bool half, hipStream_t stream) {
+    const size_t lds = 2 * size_t(StagedCfg<false, true>::TILE_BYTES);
+    const dim3 grid(S, p.num_splits, half ? 1 : p.H_KV / 16), block(512 + 64 * 4);
+#define FQ_D64_GP(BSL, GPV, HALFV)                                                                                \
+    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, HALFV, false, true>, p, grid, block, lds, stream) \
+                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, HALFV, false, true>, p, grid, block, lds, stream)
+#define FQ_D64_BS(BSL, HALFV)                            \
+    do {                                                 \
+        if (p.G <= 4) { FQ_D64_GP(BSL, 4, HALFV); }      \
+        else if (p.G <= 8) { FQ_D64_GP(BSL, 8, HALFV); } \
+        else { FQ_D64_GP(BSL, 16, HALFV); }              \
+    } while (0)
+    if (half) {
+        if (rows_per_page == 8) FQ_D64_BS(3, true);
+        else FQ_D64_BS(4, true);
+    } else {
+        if (rows_per_page == 8) FQ_D64_BS(3, false);
+        else if (rows_per_page == 16) FQ_D64_BS(4, false);
+        else FQ_D64_BS(5, false);
+    }
+#undef FQ_D64_BS
+#undef FQ_D64_GP
+}
+
 template <int D, int DT>
 int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bool allow_half, const DecodeVariant& var) {
+    if constexpr (D == 64) {
+        const bool d64_half = allow_half && staged_d64_half_applies(D, p.H_KV, p.G, BS, var);
+        if (p.new_key == nullptr && (d64_half || staged_d64_full_applies(D, p.H_KV, p.G, var))) {
+            const int rows_per_page = d64_half ? BS / 2 : BS;
+            const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
+            const int64_t chunk_rows = (((max_rows + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
+            DecodeParams ps = p;
+            ps.G = 2 * p.G;                 // query heads of a pair of KV heads
+            const int groups = d64_half ? 1 : p.H_KV / 16;
+            ps.balance_slots = staged_balance_slots(S, p.num_splits * groups);
+            if (ps.balance_slots > 0) ps.balance_slots = ps.balance_slots / groups > 0 ? ps.balance_slots / groups : 1;
+            const bool wide_rows = chunk_rows / rows_per_page > 64 || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256);
+            return launch_staged_d64<DT>(ps, S, rows_per_page, wide_rows, d64_half, stream);
+        }
+    }
     if (allow_half && staged_half_applies(D, p.H_KV, BS, var)) {
         // the kernel counts rows of two tokens: half the page size, chunks of rows
         const int rows_per_page = BS / 2;
@@ -2038,7 +2149,7 @@ extern "C" size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_K
     if (num_seqs <= 0 || H_Q <= 0 || H_KV <= 0 || D <= 0) return 0;
     num_splits = fq::effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
     // room for the two partials per split of the 4-KV-head staged decode, whatever the switches say
-    if (D == 128 && H_KV == 4 && block_size >= 16) num_splits *= 2;
+    if ((D == 128 && H_KV == 4 && block_size >= 16) || (D == 64 && H_KV == 8 && block_size >= 16)) num_splits *= 2;
     return fq::workspace_layout(num_seqs, H_Q, D, num_splits).total;
 }
 
@@ -2169,7 +2280,8 @@ int split_k_paged_decode_impl(const void* q, const uint8_t* kv_cache, const int3
     if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16)) return FQ_ERR_MISALIGNED;
     num_splits = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
     // 4 KV heads: the staged kernel reads rows of two tokens and writes one partial per token parity
-    const bool half = staged_half_applies(D, H_KV, block_size, var);
+    const int G = H_Q / H_KV;
+    const bool half = staged_half_applies(D, H_KV, block_size, var) || staged_d64_half_applies(D, H_KV, G, block_size, var);
     const int num_partials = half ? 2 * num_splits : num_splits;
     const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_partials);
     if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
@@ -2181,7 +2293,7 @@ int split_k_paged_decode_impl(const void* q, const uint8_t* kv_cache, const int3
     const void* q_in = q;
     const float* fused_rotation = nullptr;
     if (rotation) {
-        if (centroids_k && (half || staged_applies(D, H_KV, var))) {
+        if (centroids_k && (half || staged_applies(D, H_KV, var) || (token == nullptr && staged_d64_full_applies(D, H_KV, G, var)))) {
             fused_rotation = rotation;       // the staged kernel rotates the query in its prologue
         } else {
             const int st = fq_rotate_query(q, rotation, rotation_col_major, ws + w.qrot, num_seqs, H_Q, D, dtype, stream);
@@ -2306,7 +2418,7 @@ extern "C" int fq_split_k_paged_decode_static(const void* q, const uint8_t* kv_c
     // the partials of this launch must fit the array: a larger problem is refused, not truncated (room
     // for the two partials per split of the 4-KV-head staged decode whatever the switches say, as in
     // fq_paged_decode_workspace_bytes: the call below reads the switches once for itself)
-    const int num_partials = (D == 128 && H_KV == 4 && block_size >= 16) ? 2 * ns : ns;
+    const int num_partials = ((D == 128 && H_KV == 4) || (D == 64 && H_KV == 8)) && block_size >= 16 ? 2 * ns : ns;
     if (workspace_layout(num_seqs, H_Q, D, num_partials).total > kStaticScratchBytes) return FQ_ERR_WORKSPACE;
     void* ws = nullptr;
     const int st = static_scratch_address(&ws);

@@ -350,6 +350,42 @@ def test_paged_decode_on_a_caller_workspace_with_arbitrary_contents():
         C.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], 8, 128, 16, None, out, 5, ws[:1024])
 
 
+@pytest.mark.parametrize("hq,hkv,bs,dtype", [(32, 8, 16, torch.bfloat16), (64, 8, 32, torch.float16), (8, 8, 16, torch.bfloat16),
+                                             (24, 8, 16, torch.float16), (32, 16, 16, torch.bfloat16), (64, 16, 8, torch.float16),
+                                             (128, 16, 32, torch.bfloat16), (96, 32, 16, torch.bfloat16), (16, 16, 16, torch.float16)])
+def test_paged_decode_head_dim_64_on_the_staged_kernel(hq, hkv, bs, dtype, kernel_option):
+    """head_dim 64 with 8 KV heads (pages of 16 / 32 tokens) or a multiple of 16: pairs of neighbouring heads run as
+    heads of 128 on the staged kernel, the query rotation in its prologue.  Against the oracle, and against the
+    direct kernel on the same inputs."""
+    c, b, r = book(64)
+    for lens, splits in (([37, 0, 16, 300, 64, 65, 1, 129], 3), ([1500, 0, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0)):
+        _decode_case(lens, hq=hq, hkv=hkv, d=64, bs=bs, num_splits=splits, dtype=dtype)
+        q, cache, table, sl = build_paged_case(lens, hq, hkv, d=64, bs=bs, seed=31, dtype=dtype)
+        dev = [t.to(DEV) for t in (q, cache, table, sl, c, r)]
+        got = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], hkv, 64, bs, num_splits=splits)
+        kernel_option("decode_direct", True)
+        direct = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], hkv, 64, bs, num_splits=splits)
+        kernel_option("decode_direct", False)
+        assert (got.float() - direct.float()).abs().max().item() <= 2e-2
+
+
+def test_paged_decode_head_dim_64_two_codebooks_and_prerotated_query():
+    """The same kernel with a value codebook of its own, and through the partials entry point with a query that
+    is already rotated (16 KV heads: the form that entry point reaches)."""
+    C = load_native()
+    c, b, r = book(64)
+    cv = (c * 1.25).contiguous()
+    q, cache, table, sl = build_paged_case([300, 17, 1000], 32, 16, d=64, seed=78)
+    want = O.split_k_paged_decode(q, cache, table, sl, c, cv, r, 16, 64, 16)
+    dev = [t.to(DEV) for t in (q, cache, table, sl, c, cv, r)]
+    got = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[5], dev[6], 16, 64, 16, num_splits=4)
+    assert (got.cpu().float() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
+    q_rot = (q.float() @ r.T).to(q.dtype).to(DEV)
+    acc, m, l = C.paged_tq4_decode_partials(q_rot, dev[1], dev[2], dev[3], dev[4], dev[5], 16, 64, 16, 1.0 / math.sqrt(64), 4)
+    out = C.split_k_reduce(acc, m, l, dev[6], q.dtype)
+    assert (out.cpu().float() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
+
+
 def test_prod_paged_decode_without_copy_wavefronts(kernel_option):
     kernel_option("decode_copy_waves", False)
     _check_prod_decode([300, 1, 77, 0, 129], 32, num_splits=5)
