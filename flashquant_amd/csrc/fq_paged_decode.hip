@@ -521,17 +521,18 @@ __global__ __launch_bounds__(D == 256 ? 256 : 512) void paged_decode_kernel(cons
 // carries a second float32, the residual norm, so a token row is
 // [K nibbles H*64 | K norm H*4 | K residual norm H*4 | V idx H*64 | V norm H*4] = H*140 bytes
 // and a stage grows by 512 bytes of residual norms.
-// D64 (head_dim 64, TQ4 pages): two neighbouring KV heads of 64 coordinates are served as one "head" of 128
-// (their index bytes are contiguous in the token row), with two norms each for K and V: a row of 8 such
-// heads is 16 real heads, 72 chunks.
-template <bool PROD, bool D64 = false>
+// DIM = 64 (TQ4 pages): two neighbouring KV heads of 64 coordinates are served as one "head" of 128 (their index
+// bytes are contiguous in the token row), with two norms each for K and V: a row of 8 such heads is 16 real
+// heads, 72 chunks.  DIM = 256: a KV head of 256 coordinates is served as two "heads" of 128 (the halves of its
+// index bytes) that share its norms: a row of 8 such heads is 4 real heads, 66 chunks.
+template <bool PROD, int DIM = 128>
 struct StagedCfg {
-    static constexpr int CHUNKS_PER_ROW = PROD ? 70 : (D64 ? 72 : 68);   // 16-byte chunks of a token row, 8 heads
-    static constexpr int ROWB = 16 * CHUNKS_PER_ROW;               // 1088 / 1120 / 1152
-    static constexpr int STAGE_BYTES = 16 * ROWB;                  // 17408 / 17920 / 18432
+    static constexpr int CHUNKS_PER_ROW = PROD ? 70 : (DIM == 64 ? 72 : (DIM == 256 ? 66 : 68));   // 16-byte chunks of a row
+    static constexpr int ROWB = 16 * CHUNKS_PER_ROW;               // 1088 / 1120 / 1152 / 1056
+    static constexpr int STAGE_BYTES = 16 * ROWB;                  // 17408 / 17920 / 18432 / 16896
     static constexpr int TILE_BYTES = 2 * STAGE_BYTES;             // 32 tokens
-    static constexpr int CHUNKS_PER_TILE = 32 * CHUNKS_PER_ROW;    // 2176 / 2240 / 2304
-    static constexpr int NORM_BYTES = D64 ? 64 : 32;               // K (or V) norms of a row
+    static constexpr int CHUNKS_PER_TILE = 32 * CHUNKS_PER_ROW;    // 2176 / 2240 / 2304 / 2112
+    static constexpr int NORM_BYTES = DIM == 64 ? 64 : (DIM == 256 ? 16 : 32);   // K (or V) norms of a row
     static constexpr int KN_OFF = 16384;                           // K norms of the stage's 16 rows
     static constexpr int VN_OFF = KN_OFF + 16 * NORM_BYTES;        // V norms
 };
@@ -545,16 +546,24 @@ __host__ __device__ constexpr int staged_slot(int h, int r, int q) {
 }
 
 // LDS byte offset (inside a tile slot) of the 16-byte chunk `ci` of tile row `row` (0..31).
-template <bool PROD, bool D64 = false>
+template <bool PROD, int DIM = 128>
 __host__ __device__ constexpr int staged_chunk_dst(int row, int ci) {
     const int stage = row >> 4, r = row & 15;
     int off = 0;
-    if (D64) {
-        using C = StagedCfg<false, true>;
+    if (DIM == 64) {
+        using C = StagedCfg<false, 64>;
         if (ci < 32) off = 16 * staged_slot(ci >> 2, r, ci & 3);
         else if (ci < 36) off = C::KN_OFF + 64 * r + 16 * (ci - 32);
         else if (ci < 68) off = 8192 + 16 * staged_slot((ci - 36) >> 2, r, (ci - 36) & 3);
         else off = C::VN_OFF + 64 * r + 16 * (ci - 68);
+        return stage * C::STAGE_BYTES + off;
+    }
+    if (DIM == 256) {
+        using C = StagedCfg<false, 256>;
+        if (ci < 32) off = 16 * staged_slot(ci >> 2, r, ci & 3);
+        else if (ci == 32) off = C::KN_OFF + 16 * r;
+        else if (ci < 65) off = 8192 + 16 * staged_slot((ci - 33) >> 2, r, (ci - 33) & 3);
+        else off = C::VN_OFF + 16 * r;
         return stage * C::STAGE_BYTES + off;
     }
     if (ci < 32) {
@@ -573,17 +582,17 @@ __host__ __device__ constexpr int staged_chunk_dst(int row, int ci) {
 
 // The same offsets for every chunk of a tile, worked out at compile time: a thread reads its
 // five entries instead of dividing by the row length and walking the layout.
-template <bool PROD, bool D64 = false>
+template <bool PROD, int DIM = 128>
 struct ChunkDstTable {
-    uint16_t off[StagedCfg<PROD, D64>::CHUNKS_PER_TILE];
+    uint16_t off[StagedCfg<PROD, DIM>::CHUNKS_PER_TILE];
     constexpr ChunkDstTable() : off() {
-        for (int c = 0; c < StagedCfg<PROD, D64>::CHUNKS_PER_TILE; ++c)
-            off[c] = uint16_t(staged_chunk_dst<PROD, D64>(c / StagedCfg<PROD, D64>::CHUNKS_PER_ROW,
-                                                          c % StagedCfg<PROD, D64>::CHUNKS_PER_ROW));
+        for (int c = 0; c < StagedCfg<PROD, DIM>::CHUNKS_PER_TILE; ++c)
+            off[c] = uint16_t(staged_chunk_dst<PROD, DIM>(c / StagedCfg<PROD, DIM>::CHUNKS_PER_ROW,
+                                                          c % StagedCfg<PROD, DIM>::CHUNKS_PER_ROW));
     }
 };
-template <bool PROD, bool D64 = false>
-__device__ const ChunkDstTable<PROD, D64> kChunkDst{};
+template <bool PROD, int DIM = 128>
+__device__ const ChunkDstTable<PROD, DIM> kChunkDst{};
 
 // TurboQuantProd sign operand: the fp16 pairs (+-1, +-1) of the eight sign bits (bit 3 of
 // every nibble) of one key dword.  Element e of the result belongs to the coordinate
@@ -630,11 +639,21 @@ __device__ unsigned int g_decode_faults = 0u;
 // HALF (4 KV heads): the kernel works on rows of 8 "heads" made of two consecutive tokens, head h of
 // the even token as head h and of the odd token as head 4 + h, so row r is the real rows 2 r and
 // 2 r + 1 (544 bytes each) with their sections interleaved; a page then holds half as many rows.
-template <bool PROD, bool HALF, bool D64 = false>
+template <bool PROD, bool HALF, int DIM = 128>
 __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
-    constexpr int CPR = StagedCfg<PROD, D64>::CHUNKS_PER_ROW;
+    constexpr int CPR = StagedCfg<PROD, DIM>::CHUNKS_PER_ROW;
     const int r = cc / CPR, ci = cc - r * CPR;
-    if constexpr (D64) {
+    if constexpr (DIM == 256) {
+        // head_dim 256, H real heads: [K idx H*128 | K norms H*4 | V idx H*128 | V norms H*4] = 264 H bytes a token;
+        // group hgrp of 4 real heads
+        int off;
+        if (ci < 32) off = 512 * hgrp + 16 * ci;
+        else if (ci == 32) off = H * 128 + 16 * hgrp;
+        else if (ci < 65) off = H * 132 + 512 * hgrp + 16 * (ci - 33);
+        else off = H * 260 + 16 * hgrp;
+        return uint32_t(r * (H * 264) + off);
+    }
+    if constexpr (DIM == 64) {
         // head_dim 64, H real heads: [K idx H*32 | K norms H*4 | V idx H*32 | V norms H*4] = 72 H bytes a token
         if constexpr (HALF) {      // 8 real heads: a row is two tokens of 576 bytes
             int tok, off;
@@ -676,16 +695,22 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     return uint32_t(r * (H * 136) + off);
 }
 
-template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false, bool STORE = false, bool D64 = false>
+template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false, bool STORE = false, int DIM = 128>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
+    constexpr bool D64 = DIM == 64, D256 = DIM == 256;
     static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
-    static_assert(!D64 || (!PROD && !STORE && CW > 0), "head_dim 64 is served by the TQ4 form with copy wavefronts");
+    static_assert(DIM == 128 || (!PROD && !STORE && CW > 0), "head_dim 64 / 256 are served by the TQ4 form with copy wavefronts");
+    static_assert(!(D256 && HALF), "head_dim 256 comes in groups of 4 KV heads");
+    // D256: the kernel's "heads" are the halves of real heads of 256 coordinates (wavefront h: real head h / 2 of the
+    // group of 4, coordinates 128 (h % 2) ...): the two wavefronts of a head exchange their halves of the scores
+    // through LDS every tile and add them, compute the same weights, and each accumulates its half of the output
+    // coordinates.  The query comes rotated (the 256 x 256 matrix is too much for a prologue).
     // D64: the kernel's "heads" are pairs of real heads of 64 coordinates, and p.G is twice the real group size: the
     // query heads of a pair are those of its first head followed by those of its second.  A query row is the real
     // row in the half of its head and zeros in the other; its scores and outputs then are the real ones, with the
     // norms of its own head and the output coordinates of its own half.
-    using Cfg = StagedCfg<PROD, D64>;
+    using Cfg = StagedCfg<PROD, DIM>;
     constexpr int kStageBytes = Cfg::STAGE_BYTES;
     constexpr int kTileBytes = Cfg::TILE_BYTES;
     constexpr int kChunksPerRow = Cfg::CHUNKS_PER_ROW;
@@ -706,6 +731,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // from slot s (one count per computing wavefront and tile)
     // STORE: [7] computing wavefronts whose part of the new token's row has reached the cache
     __shared__ uint32_t flags[8];
+    // D256: [h] score halves posted by wavefront h, [8 + h] partner halves read by wavefront h (counts of tiles)
+    __shared__ uint32_t xflags[16];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -727,13 +754,14 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // More than 8 KV heads: a workgroup serves the group of 8 heads blockIdx.z, i.e. the query heads
     // hq0 .. hq0 + 8 G - 1, and copies that group's slices of the token rows.
     const int hgrp = blockIdx.z;
-    const int HQG = (HALF ? 4 : 8) * p.G;      // query heads of a group
+    const int HQG = ((HALF || D256) ? 4 : 8) * p.G;      // query heads of a group
     const int hq0 = hgrp * HQG;
     const int row_bytes = D64 ? (HALF ? 1152 : p.H_KV * 72)
-                              : (HALF ? 1088 : p.H_KV * (PROD ? 140 : 136));   // a row of the cache as the kernel sees it
+                        : D256 ? p.H_KV * 264
+                               : (HALF ? 1088 : p.H_KV * (PROD ? 140 : 136));   // a row of the cache as the kernel sees it
     const int qsub = D64 && (n % GP) >= p.G / 2 ? 1 : 0;    // D64: this lane's query head belongs to the pair's second head
     // HALF: wavefront h works on real head h % 4 and on the tokens of parity h / 4 (rows are token pairs)
-    const int hr = HALF ? (h & 3) : h;
+    const int hr = D256 ? (h >> 1) : (HALF ? (h & 3) : h);     // D256: the real head; its half is h & 1
     const int tsel = HALF ? (h >> 2) & 1 : 0;
 
     // Every load that depends on nothing is asked for first, so that the memory
@@ -797,8 +825,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
         src_page[k] = pg;
         const int sub = (kSpreadTail && k == 4) ? 4 * (tid & 3) : 0;
-        src_off[k] = staged_src_offset<PROD, HALF, D64>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
-        dst_off[k] = kChunkDst<PROD, D64>.off[c] + sub;
+        src_off[k] = staged_src_offset<PROD, HALF, DIM>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+        dst_off[k] = kChunkDst<PROD, DIM>.off[c] + sub;
     }
     const bool has_round4 = kSpreadTail || tid < kChunksPerTile - 4 * 512;   // else whole wavefronts
     // ---- lane-constant LDS read offsets (inside a tile slot) -------------------------------
@@ -822,7 +850,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         else { blk = e >> 2; row = 4 * g + (e & 3); }
         sc_tok[e] = 16 * blk + row;
         n_rd[e] = D64 ? blk * kStageBytes + Cfg::KN_OFF + 64 * row + 8 * h + 4 * qsub
-                      : blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
+                : D256 ? blk * kStageBytes + Cfg::KN_OFF + 16 * row + 4 * (h >> 1)
+                       : blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
     }
 
     // dword d of the P operand holds slots 2d, 2d + 1: it is this lane's when its class owns them
@@ -846,11 +875,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     int L_known = -1;
     if (p.balance_slots > 0) balance_chunks<PVR, BS, HALF>(p, lane, NS, rowwide, chunk, seq, split, L_known);
 
-    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + (int64_t(seq) * p.H_Q + hq0) * (D64 ? 64 : 128);
+    const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + (int64_t(seq) * p.H_Q + hq0) * DIM;
     // eight elements of query row `row` of this workgroup, from element `v` (a multiple of 8) of the 128 the kernel
     // works on.  D64: the real row of 64 in the half of its head, zeros in the other half.
     auto q_chunk = [&](int row, int v) -> uint4v {
-        if constexpr (!D64) {
+        if constexpr (D256) {
+            return *reinterpret_cast<const uint4v*>(qseq + row * 256 + 128 * (h & 1) + v);     // this wavefront's half
+        } else if constexpr (!D64) {
             return *reinterpret_cast<const uint4v*>(qseq + row * 128 + v);
         } else {
             const int in_group = row - (row / p.G) * p.G;
@@ -894,6 +925,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         // wavefront has just asked for its sequence length and page ids and none has used them yet
         // (the barrier does not wait for loads from global memory).
         if (tid < 8) flags[tid] = 0u;
+        if (D256 && tid < 16) xflags[tid] = 0u;
         __syncthreads();
         load_matrix_columns();
         load_first_heads();
@@ -928,7 +960,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     const int NS_out = HALF ? 2 * NS : NS;
     const int split_out = HALF ? 2 * split + tsel : split;
     if (begin >= end) {   // uniform over the workgroup
-        if (g == 0 && n < p.G && !copier) {
+        if (g == 0 && n < p.G && !copier && (!D256 || (h & 1) == 0)) {
             const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS_out + split_out;
             p.part_m[o] = -__builtin_inff();
             p.part_l[o] = 0.0f;
@@ -1024,8 +1056,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
                 c_page[k] = pg;
                 const int sub = (k < FULL || !kHalfTail) ? 0 : 8 * (ct & 1);
-                c_src[k] = staged_src_offset<PROD, HALF, D64>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
-                c_dst[k] = kChunkDst<PROD, D64>.off[c] + sub;
+                c_src[k] = staged_src_offset<PROD, HALF, DIM>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+                c_dst[k] = kChunkDst<PROD, DIM>.off[c] + sub;
             }
             const bool has_rest = kHalfTail || ct < REST;
             auto c_issue = [&](uint4v (&r)[NR], int t0) {
@@ -1319,7 +1351,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     float M = -__builtin_inff();
     float lsum = 0.0f;
 
-    auto compute_tile = [&](int t0, int slot) {
+    auto compute_tile = [&](int t0, int slot, int it) {
         const uint8_t* tile = slots + slot * kTileBytes;
         // operands of this lane, raw
         uint4v kraw[2];
@@ -1334,7 +1366,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
         for (int e = 0; e < NSC; ++e) {
             kn[e] = *reinterpret_cast<const float*>(tile + n_rd[e]);
-            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (D64 ? Cfg::VN_OFF - Cfg::KN_OFF : kStageVnOff - kStageKnOff));
+            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (DIM != 128 ? Cfg::VN_OFF - Cfg::KN_OFF : kStageVnOff - kStageKnOff));
             kg[e] = PROD ? *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageKgOff - kStageKnOff)) : 0.0f;
         }
         // These were all the reads of the slot (the lookups below go to the table): it is handed back
@@ -1389,6 +1421,24 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             if (b == 0) v_group(0, vb[0]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        if constexpr (D256) {
+            // ---- the other half of the head's coordinates: wavefront h ^ 1 has their part of every score.  Each
+            // posts its part (times its own query scale) in its patch of LDS behind the tile slots and adds the
+            // partner's: a + b in one wavefront, b + a in the other, the same bits.  The patch is rewritten
+            // every tile, so a wavefront waits for the partner to have read the tile before (bounded waits).
+            float4v* xb = reinterpret_cast<float4v*>(slots + 2 * kTileBytes);
+            const int hp = h ^ 1;
+            if (!lds_flag_wait(&xflags[8 + hp], uint32_t(it), p.spin_limit)) { flags[2] = 1u; handoff_failed = true; }
+            const float4v m0 = acc[0] * qscale, m1 = acc[1] * qscale;
+            xb[(2 * h) * kWave + lane] = m0;
+            xb[(2 * h + 1) * kWave + lane] = m1;
+            lds_flag_signal(&xflags[h], lane);
+            if (!lds_flag_wait(&xflags[hp], uint32_t(it) + 1u, p.spin_limit)) { flags[2] = 1u; handoff_failed = true; }
+            const float4v o0 = xb[(2 * hp) * kWave + lane], o1 = xb[(2 * hp + 1) * kWave + lane];
+            acc[0] = m0 + o0;
+            acc[1] = m1 + o1;
+            lds_flag_signal(&xflags[8 + h], lane);
+        }
 
         // ---- this lane's scores ------------------------------------------------------------------
         float a_[NSC], rv[NSC];
@@ -1413,7 +1463,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             }
             const bool live = t0 + sc_tok[e] < end_mine;
             rv[e] = live ? vn[e] : 0.0f;
-            float sc = s * kn[e] * qscale;
+            float sc = D256 ? s * kn[e] : s * kn[e] * qscale;      // D256: the scale went in before the halves were added
             if (PROD) sc = __builtin_fmaf(s2 * kg[e], qscale_s, sc);
             a_[e] = live ? sc : -__builtin_inff();
         }
@@ -1509,7 +1559,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             __syncthreads();                      // tile i is in LDS; slot of tile i - 1 is free
             write_slot((i + 1) & 1);              // tile i + 1 (its loads ran during tile i - 1)
             issue_loads(clamp_t0(t0 + 64));       // tile i + 2
-            compute_tile(t0, i & 1);
+            compute_tile(t0, i & 1, i);
         }
     } else {
         int i = 0;
@@ -1519,7 +1569,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 flags[2] = 1u;
                 handoff_failed = true;
             }
-            compute_tile(t0, i & 1);
+            compute_tile(t0, i & 1, i);
             if constexpr (STORE) {
                 if (i == 0 && stores_token && last_t0 >= begin + 64) {      // (see the prologue)
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1553,7 +1603,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             if (handoff_failed && lane == 0) atomicAdd(&g_decode_faults, 1u);
         }
     }
-    if (g == 0 && n < p.G) {
+    if (g == 0 && n < p.G && (!D256 || (h & 1) == 0)) {        // D256: both halves hold the same maximum and denominator
         const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS_out + split_out;
         p.part_m[o] = M;
         p.part_l[o] = lsum;
@@ -1566,7 +1616,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             const bool mine = !D64 || (n >> 3) == (head >= p.G / 2 ? 1 : 0);
             if (head < p.G && mine) {
                 float* dst = D64 ? p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS_out + split_out) * 64 + (n & 7) * DPL
-                                 : p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS_out + split_out) * D + n * DPL;
+                           : D256 ? p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS_out + split_out) * 256 + 128 * (h & 1) + n * DPL
+                                  : p.part_acc + ((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS_out + split_out) * D + n * DPL;
 #pragma unroll
                 for (int q4 = 0; q4 < DPL / 4; ++q4) {
                     const float4v v = {O[4 * q4][i], O[4 * q4 + 1][i], O[4 * q4 + 2][i], O[4 * q4 + 3][i]};
@@ -1915,11 +1966,11 @@ inline bool staged_d64_half_applies(int D, int H_KV, int G, int block_size, cons
 }
 template <int DT>
 int launch_staged_d64(const DecodeParams& p, int S, int rows_per_page, bool wide, bool half, hipStream_t stream) {
-    const size_t lds = 2 * size_t(StagedCfg<false, true>::TILE_BYTES);
+    const size_t lds = 2 * size_t(StagedCfg<false, 64>::TILE_BYTES);
     const dim3 grid(S, p.num_splits, half ? 1 : p.H_KV / 16), block(512 + 64 * 4);
 #define FQ_D64_GP(BSL, GPV, HALFV)                                                                                \
-    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, HALFV, false, true>, p, grid, block, lds, stream) \
-                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, HALFV, false, true>, p, grid, block, lds, stream)
+    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, HALFV, false, 64>, p, grid, block, lds, stream) \
+                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, HALFV, false, 64>, p, grid, block, lds, stream)
 #define FQ_D64_BS(BSL, HALFV)                            \
     do {                                                 \
         if (p.G <= 4) { FQ_D64_GP(BSL, 4, HALFV); }      \
@@ -1938,8 +1989,45 @@ int launch_staged_d64(const DecodeParams& p, int S, int rows_per_page, bool wide
 #undef FQ_D64_GP
 }
 
+// head_dim 256 on the staged kernel: every KV head as two heads of 128, 4 real heads a group; the query comes rotated.
+inline bool staged_d256_applies(int D, int H_KV, const DecodeVariant& v) {
+    return D == 256 && H_KV % 4 == 0 && !v.direct && v.copy_waves == 4;
+}
+template <int DT>
+int launch_staged_d256(const DecodeParams& p, int S, int BS, bool wide, hipStream_t stream) {
+    // two tile slots and the patch through which the halves of a head exchange their scores
+    const size_t lds = 2 * size_t(StagedCfg<false, 256>::TILE_BYTES) + 8 * 2 * kWave * sizeof(float4v);
+    const dim3 grid(S, p.num_splits, p.H_KV / 4), block(512 + 64 * 4);
+#define FQ_D256_GP(BSL, GPV)                                                                                       \
+    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, false, false, 256>, p, grid, block, lds, stream) \
+                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, false, false, 256>, p, grid, block, lds, stream)
+#define FQ_D256_BS(BSL)                           \
+    do {                                          \
+        if (p.G <= 4) { FQ_D256_GP(BSL, 4); }     \
+        else if (p.G <= 8) { FQ_D256_GP(BSL, 8); } \
+        else { FQ_D256_GP(BSL, 16); }             \
+    } while (0)
+    if (BS == 8) FQ_D256_BS(3);
+    else if (BS == 16) FQ_D256_BS(4);
+    else FQ_D256_BS(5);
+#undef FQ_D256_BS
+#undef FQ_D256_GP
+}
+
 template <int D, int DT>
 int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bool allow_half, const DecodeVariant& var) {
+    if constexpr (D == 256) {
+        if (p.new_key == nullptr && p.rotation == nullptr && staged_d256_applies(D, p.H_KV, var)) {
+            const int64_t max_ctx = int64_t(p.max_blocks) * BS;
+            const int64_t chunk = (((max_ctx + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
+            DecodeParams ps = p;
+            const int groups = p.H_KV / 4;
+            ps.balance_slots = staged_balance_slots(S, p.num_splits * groups);
+            if (ps.balance_slots > 0) ps.balance_slots = ps.balance_slots / groups > 0 ? ps.balance_slots / groups : 1;
+            const bool wide = chunk / BS > 64 || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256);
+            return launch_staged_d256<DT>(ps, S, BS, wide, stream);
+        }
+    }
     if constexpr (D == 64) {
         const bool d64_half = allow_half && staged_d64_half_applies(D, p.H_KV, p.G, BS, var);
         if (p.new_key == nullptr && (d64_half || staged_d64_full_applies(D, p.H_KV, p.G, var))) {

@@ -369,6 +369,24 @@ def test_paged_decode_head_dim_64_on_the_staged_kernel(hq, hkv, bs, dtype, kerne
         assert (got.float() - direct.float()).abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("hq,hkv,bs,dtype", [(16, 4, 16, torch.bfloat16), (32, 8, 16, torch.bfloat16), (8, 8, 32, torch.float16),
+                                             (64, 4, 8, torch.bfloat16), (24, 12, 16, torch.float16), (20, 4, 16, torch.bfloat16)])
+def test_paged_decode_head_dim_256_on_the_staged_kernel(hq, hkv, bs, dtype, kernel_option):
+    """head_dim 256 with a multiple of 4 KV heads: the halves of a head run as two heads of 128 on the staged kernel
+    (the two wavefronts of a head add their halves of the scores through LDS).  Against the oracle, and against the
+    direct kernel on the same inputs."""
+    c, b, r = book(256)
+    for lens, splits in (([37, 0, 16, 300, 64, 65, 1, 129], 3), ([1500, 0, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0)):
+        _decode_case(lens, hq=hq, hkv=hkv, d=256, bs=bs, num_splits=splits, dtype=dtype)
+        q, cache, table, sl = build_paged_case(lens, hq, hkv, d=256, bs=bs, seed=32, dtype=dtype)
+        dev = [t.to(DEV) for t in (q, cache, table, sl, c, r)]
+        got = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], hkv, 256, bs, num_splits=splits)
+        kernel_option("decode_direct", True)
+        direct = K.split_k_paged_decode(dev[0], dev[1], dev[2], dev[3], dev[4], dev[4], dev[5], hkv, 256, bs, num_splits=splits)
+        kernel_option("decode_direct", False)
+        assert (got.float() - direct.float()).abs().max().item() <= 2e-2
+
+
 def test_paged_decode_head_dim_64_two_codebooks_and_prerotated_query():
     """The same kernel with a value codebook of its own, and through the partials entry point with a query that
     is already rotated (16 KV heads: the form that entry point reaches)."""
