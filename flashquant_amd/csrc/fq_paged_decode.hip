@@ -1648,7 +1648,9 @@ __global__ __launch_bounds__(256) void rotate_q_kernel(const uint16_t* __restric
             a[j][2 * i + 1] = load_elem<DT>(uint16_t(w[i] >> 16));
         }
     }
-    for (int cb = wave; cb < D / 16; cb += 4) {
+    // gridDim.y workgroups share the column blocks of a row group (one round of four blocks each at head_dim 256:
+    // the rows are few, 1024 in a decode step of 32 sequences x 32 heads, and the matrix is what is fetched)
+    for (int cb = wave + 4 * int(blockIdx.y); cb < D / 16; cb += 4 * int(gridDim.y)) {
         float b[D / 32][8];
         load_rotation_any<D>(R, col_major != 0, true, 16 * cb, n, g, b);
         const float4v acc = rotate_block<D>(a, b);
@@ -1666,17 +1668,23 @@ __global__ __launch_bounds__(256) void rotate_q_kernel(const uint16_t* __restric
 // rounded again (paged_decode.py:123).  rows = num_seqs * H_Q; a workgroup owns RW rows
 // (4, 8 or 16: the fewer, the more workgroups share the combine, the more often the matrix is
 // fetched): 256 / RW threads combine a row into LDS, then all rotate from there.
-template <int D, int DT, int RW>
+// CS: the output columns of a row group are shared by CS workgroups (blockIdx.y), each combining the rows for
+// itself and fetching 1 / CS of the matrix: at head_dim 256 the matrix is 256 KB, and a workgroup that fetches all
+// of it holds 256 matrix values per lane.
+template <int D, int DT, int RW, int CS = 1>
 __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restrict__ part_acc,
                                                             const float* __restrict__ part_m,
                                                             const float* __restrict__ part_l,
                                                             const float* __restrict__ R, uint16_t* __restrict__ out,
                                                             int64_t rows, int NS, int col_major) {
-    constexpr int CBW = D / 64;            // 16-column blocks per wavefront
+    static_assert((D / 64) % CS == 0, "whole rounds of column blocks per workgroup");
+    constexpr int CBW = D / 64 / CS;       // 16-column blocks per wavefront
+    const int cb0 = 4 * CBW * int(blockIdx.y);     // first column block of this workgroup
     constexpr int OSTRIDE = D + 8;         // 16-bit words per staged row (padded: conflict-free operand reads)
     constexpr int TPR = 256 / RW;          // threads that combine one row
     constexpr int CPT = D / TPR < 2 ? 2 : D / TPR;      // coordinates per thread and pass (2, 4 or 8)
     constexpr int ACTIVE = D / CPT < TPR ? D / CPT : TPR;   // threads of a row that have coordinates
+    static_assert(CPT <= 8, "a thread stages at most eight coordinates of a row (head_dim 256: at most 8 rows a workgroup)");
     __shared__ __attribute__((aligned(16))) uint16_t os[RW * OSTRIDE];   // combined rows, query dtype
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
@@ -1773,7 +1781,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
     float rbv[CBW][D / 32][8];
     if (R != nullptr) {
 #pragma unroll
-        for (int i = 0; i < CBW; ++i) load_rotation_any<D>(R, col_major != 0, false, 16 * (wave + 4 * i), n, g, rbv[i]);
+        for (int i = 0; i < CBW; ++i) load_rotation_any<D>(R, col_major != 0, false, 16 * (cb0 + wave + 4 * i), n, g, rbv[i]);
     }
     {
         const bool live = row0 + r < rows && den > 0.0f;
@@ -1795,6 +1803,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
     }
     __syncthreads();
     if (R == nullptr) {
+        if (CS > 1 && blockIdx.y != 0) return;        // no rotation: one workgroup writes the combined rows
         for (int c = threadIdx.x; c < RW * (D / 8); c += 256) {
             const int rr = c / (D / 8), q = c % (D / 8);
             const int64_t orow = row0 + rr;
@@ -1815,7 +1824,7 @@ __global__ __launch_bounds__(256) void reduce_rotate_kernel(const float* __restr
         half8 rhi[D / 32], rlo[D / 32];
         split_rotation_block<D>(rbv[i], rhi, rlo);
         const float4v acc = rotate_block_f16<D>(a, rhi, rlo);
-        const int cb = wave + 4 * i;
+        const int cb = cb0 + wave + 4 * i;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const int rr = 4 * g + k;
@@ -2108,7 +2117,12 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
 template <int DT>
 int launch_rotate(const void* q, const float* R, int col_major, void* q_rot, int S, int H_Q, int D, hipStream_t stream) {
     const int64_t rows = int64_t(S) * H_Q;
-    const dim3 grid(unsigned((rows + kRotRows - 1) / kRotRows)), block(256);
+    // as many workgroups per group of 16 rows as it takes to fill the chip, at most one per round of column blocks
+    const int64_t row_groups = (rows + kRotRows - 1) / kRotRows;
+    const int rounds = D / 64;
+    int ysplit = int((fq_host::device_cu_count() + row_groups - 1) / row_groups);
+    ysplit = ysplit < 1 ? 1 : (ysplit > rounds ? rounds : ysplit);
+    const dim3 grid(static_cast<unsigned>(row_groups), static_cast<unsigned>(ysplit)), block(256);
     const uint16_t* src = reinterpret_cast<const uint16_t*>(q);
     uint16_t* dst = reinterpret_cast<uint16_t*>(q_rot);
     switch (D) {
@@ -2130,10 +2144,14 @@ int launch_reduce(const float* acc, const float* m, const float* l, const float*
     const int rw_opt = fq_host::option(FQ_OPT_REDUCE_ROWS);
     int rw = rows <= 4 * int64_t(cus) ? 4 : (rows <= 8 * int64_t(cus) ? 8 : 16);
     if (rw_opt == 4 || rw_opt == 8 || rw_opt == 16) rw = rw_opt;
-    const dim3 grid(unsigned((rows + rw - 1) / rw)), block(256);
+    // head_dim 256: four workgroups share the columns of a row group, 16 rows a group while that fills the chip
+    constexpr int kColumnSplit256 = 4;
+    if (D == 256) rw = (rw_opt == 4) ? 4 : 8;       // (a thread stages at most eight coordinates of a row; measured: 8 rows
+                                                    // x 4 column groups 79 us per step of 32 x 4096 tokens, 4 rows 81 us)
+    const dim3 grid(unsigned((rows + rw - 1) / rw), D == 256 ? kColumnSplit256 : 1), block(256);
     uint16_t* dst = reinterpret_cast<uint16_t*>(out);
 #define FQ_REDUCE(DD, RWV) \
-    hipLaunchKernelGGL((reduce_rotate_kernel<DD, DT, RWV>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major)
+    hipLaunchKernelGGL((reduce_rotate_kernel<DD, DT, RWV, (DD == 256 ? kColumnSplit256 : 1)>), grid, block, 0, stream, acc, m, l, R, dst, rows, NS, col_major)
 #define FQ_REDUCE_D(DD)                       \
     do {                                      \
         if (rw == 4) FQ_REDUCE(DD, 4);        \
@@ -2143,7 +2161,10 @@ int launch_reduce(const float* acc, const float* m, const float* l, const float*
     switch (D) {
         case 64: FQ_REDUCE_D(64); break;
         case 128: FQ_REDUCE_D(128); break;
-        default: FQ_REDUCE_D(256); break;
+        default:
+            if (rw == 4) FQ_REDUCE(256, 4);
+            else FQ_REDUCE(256, 8);
+            break;
     }
 #undef FQ_REDUCE_D
 #undef FQ_REDUCE

@@ -387,6 +387,16 @@ def test_paged_decode_head_dim_256_on_the_staged_kernel(hq, hkv, bs, dtype, kern
         assert (got.float() - direct.float()).abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("d,hq,hkv", [(256, 32, 4), (128, 32, 8), (64, 32, 8)])
+@pytest.mark.parametrize("rows_per_wg", [0, 4, 8, 16])
+def test_combine_kernel_rows_per_workgroup_on_many_rows(d, hq, hkv, rows_per_wg, kernel_option):
+    """More rows than 8 per CU (70 sequences x 32 heads = 2240), so that the automatic choice is the largest
+    row count per combine workgroup, and every forced count: same result against the oracle."""
+    kernel_option("reduce_rows", rows_per_wg)
+    rng_lens = [(37 * i) % 150 for i in range(70)]
+    _decode_case(rng_lens, hq=hq, hkv=hkv, d=d, bs=16, num_splits=3, seed=55)
+
+
 def test_paged_decode_head_dim_64_two_codebooks_and_prerotated_query():
     """The same kernel with a value codebook of its own, and through the partials entry point with a query that
     is already rotated (16 KV heads: the form that entry point reaches)."""
