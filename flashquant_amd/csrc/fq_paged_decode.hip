@@ -695,9 +695,20 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     return uint32_t(r * (H * 136) + off);
 }
 
-template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, bool HALF = false, bool STORE = false, int DIM = 128>
+template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, int MULTI = 0, bool STORE = false, int DIM = 128>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     constexpr bool D64 = DIM == 64, D256 = DIM == 256;
+    // MULTI: the kernel's rows are 2^MULTI consecutive tokens of 8 / 2^MULTI KV heads (1088 bytes whichever way).
+    // 1 (HALF): 4 KV heads, the sections of the two tokens interleaved by the copy plan into the layout of an
+    // 8-head row.  2, 3 (LINEAR): 2 KV heads or 1; the token rows go to LDS as they lie in the cache (their
+    // sections start at multiples of 8 and 4 bytes, not of the 16 of a copy chunk) and the computing wavefronts
+    // read their operands from where they are.
+    constexpr bool HALF = MULTI == 1;
+    constexpr bool LINEAR = MULTI >= 2;
+    constexpr int TPR = 1 << MULTI;          // tokens per row
+    constexpr int HPR = 8 / TPR;             // real KV heads per row
+    static_assert(MULTI >= 0 && MULTI <= 3, "rows of 1, 2, 4 or 8 tokens");
+    static_assert(!LINEAR || (DIM == 128 && !PROD && !STORE && CW > 0), "rows of 4 and 8 tokens: TQ4, head_dim 128, copy wavefronts");
     static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
     static_assert(DIM == 128 || (!PROD && !STORE && CW > 0), "head_dim 64 / 256 are served by the TQ4 form with copy wavefronts");
@@ -711,8 +722,11 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // row in the half of its head and zeros in the other; its scores and outputs then are the real ones, with the
     // norms of its own head and the output coordinates of its own half.
     using Cfg = StagedCfg<PROD, DIM>;
-    constexpr int kStageBytes = Cfg::STAGE_BYTES;
-    constexpr int kTileBytes = Cfg::TILE_BYTES;
+    // LINEAR: a row of 1088 bytes every 1104 in LDS, so that the rows of a block start in eight different
+    // 16-byte columns of the banks (at 1088 they would start in two)
+    constexpr int kRowLds = 1104;
+    constexpr int kStageBytes = LINEAR ? 16 * kRowLds : Cfg::STAGE_BYTES;
+    constexpr int kTileBytes = 2 * kStageBytes;
     constexpr int kChunksPerRow = Cfg::CHUNKS_PER_ROW;
     constexpr int kChunksPerTile = Cfg::CHUNKS_PER_TILE;
     constexpr int D = 128;
@@ -732,6 +746,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // STORE: [7] computing wavefronts whose part of the new token's row has reached the cache
     __shared__ uint32_t flags[8];
     // D256: [h] score halves posted by wavefront h, [8 + h] partner halves read by wavefront h (counts of tiles)
+    // LINEAR: [0] computing wavefronts that have posted their partial for the merge at the end
     __shared__ uint32_t xflags[16];
 
     const int tid = threadIdx.x;
@@ -754,15 +769,15 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // More than 8 KV heads: a workgroup serves the group of 8 heads blockIdx.z, i.e. the query heads
     // hq0 .. hq0 + 8 G - 1, and copies that group's slices of the token rows.
     const int hgrp = blockIdx.z;
-    const int HQG = ((HALF || D256) ? 4 : 8) * p.G;      // query heads of a group
+    const int HQG = (D256 ? 4 : HPR) * p.G;              // query heads of a group
     const int hq0 = hgrp * HQG;
     const int row_bytes = D64 ? (HALF ? 1152 : p.H_KV * 72)
                         : D256 ? p.H_KV * 264
-                               : (HALF ? 1088 : p.H_KV * (PROD ? 140 : 136));   // a row of the cache as the kernel sees it
+                               : (MULTI > 0 ? 1088 : p.H_KV * (PROD ? 140 : 136));   // a row of the cache as the kernel sees it
     const int qsub = D64 && (n % GP) >= p.G / 2 ? 1 : 0;    // D64: this lane's query head belongs to the pair's second head
-    // HALF: wavefront h works on real head h % 4 and on the tokens of parity h / 4 (rows are token pairs)
-    const int hr = D256 ? (h >> 1) : (HALF ? (h & 3) : h);     // D256: the real head; its half is h & 1
-    const int tsel = HALF ? (h >> 2) & 1 : 0;
+    // MULTI > 0: wavefront h works on real head h % HPR and on token h / HPR of every row
+    const int hr = D256 ? (h >> 1) : (h & (HPR - 1));          // D256: the real head; its half is h & 1
+    const int tsel = (h / HPR) & (TPR - 1);
 
     // Every load that depends on nothing is asked for first, so that the memory
     // latencies of the prologue overlap instead of adding up: the centroids, the
@@ -834,14 +849,22 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     int v_rd[2][4];             // V operand: dword n of rows 4g + i of block b
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-        k_rd[b] = b * kStageBytes + 16 * staged_slot(h, n, g);
+        if constexpr (LINEAR) {
+            // the token rows as they lie in the cache: token tsel of the row, head hr of its HPR heads
+            const int token = 136 * HPR * tsel;
+            k_rd[b] = b * kStageBytes + kRowLds * n + token + 64 * hr + 16 * g;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            v_rd[b][i] = b * kStageBytes + 8192 + 16 * staged_slot(h, 4 * g + i, n >> 2) + 4 * (n & 3);
+            for (int i = 0; i < 4; ++i) v_rd[b][i] = b * kStageBytes + kRowLds * (4 * g + i) + token + 68 * HPR + 64 * hr + 4 * n;
+        } else {
+            k_rd[b] = b * kStageBytes + 16 * staged_slot(h, n, g);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                v_rd[b][i] = b * kStageBytes + 8192 + 16 * staged_slot(h, 4 * g + i, n >> 2) + 4 * (n & 3);
+        }
     }
     // the (block, row) of this lane's scores, and the slot of each score in the P operand
     int sc_tok[NSC];            // token offset inside the tile
-    int n_rd[NSC];              // K norm offset; the V norm is 512 bytes further
+    int n_rd[NSC];              // K norm offset; the V norm is 512 bytes further (LINEAR: the V indices and K norms of the token's heads)
 #pragma unroll
     for (int e = 0; e < NSC; ++e) {
         int blk, row;
@@ -851,6 +874,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         sc_tok[e] = 16 * blk + row;
         n_rd[e] = D64 ? blk * kStageBytes + Cfg::KN_OFF + 64 * row + 8 * h + 4 * qsub
                 : D256 ? blk * kStageBytes + Cfg::KN_OFF + 16 * row + 4 * (h >> 1)
+                : LINEAR ? blk * kStageBytes + kRowLds * row + 136 * HPR * tsel + 64 * HPR + 4 * hr
                        : blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
     }
 
@@ -873,7 +897,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // leave their last splits empty
     int chunk = (((p.max_blocks * BS + NS - 1) / NS) + 63) & ~63;
     int L_known = -1;
-    if (p.balance_slots > 0) balance_chunks<PVR, BS, HALF>(p, lane, NS, rowwide, chunk, seq, split, L_known);
+    if (p.balance_slots > 0) balance_chunks<PVR, BS, TPR>(p, lane, NS, rowwide, chunk, seq, split, L_known);
 
     const uint16_t* qseq = reinterpret_cast<const uint16_t*>(p.q_rot) + (int64_t(seq) * p.H_Q + hq0) * DIM;
     // eight elements of query row `row` of this workgroup, from element `v` (a multiple of 8) of the 128 the kernel
@@ -925,7 +949,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         // wavefront has just asked for its sequence length and page ids and none has used them yet
         // (the barrier does not wait for loads from global memory).
         if (tid < 8) flags[tid] = 0u;
-        if (D256 && tid < 16) xflags[tid] = 0u;
+        if ((D256 || LINEAR) && tid < 16) xflags[tid] = 0u;
         __syncthreads();
         load_matrix_columns();
         load_first_heads();
@@ -947,20 +971,20 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         }
     }
     L = L < 0 ? 0 : L;
-    L = L > p.max_blocks * BS * (HALF ? 2 : 1) ? p.max_blocks * BS * (HALF ? 2 : 1) : L;
-    // HALF: from here on L counts rows (token pairs); a wavefront's last row may hold a token of the
-    // other parity only
-    const int rows_mine = HALF ? (L + 1 - tsel) >> 1 : L;
-    L = HALF ? (L + 1) >> 1 : L;
+    L = L > p.max_blocks * BS * TPR ? p.max_blocks * BS * TPR : L;
+    // MULTI > 0: from here on L counts rows (of TPR tokens); the last row may hold no token of this wavefront
+    const int rows_mine = (L + TPR - 1 - tsel) / TPR;
+    L = (L + TPR - 1) / TPR;
     const int begin = split * chunk;
     const int end = L < begin + chunk ? L : begin + chunk;
     const int end_mine = rows_mine < end ? rows_mine : end;      // rows < end_mine hold a token of this wavefront
     const int hq_lane = hr * p.G + n;
-    // HALF: the two parities of a head are two partials, 2 split + parity of 2 NS
-    const int NS_out = HALF ? 2 * NS : NS;
-    const int split_out = HALF ? 2 * split + tsel : split;
+    // MULTI > 0: the TPR tokens of a row are as many partials of a head, TPR split + token of TPR NS
+    // (LINEAR: merged inside the workgroup into the one partial of the split)
+    const int NS_out = LINEAR ? NS : TPR * NS;
+    const int split_out = LINEAR ? split : TPR * split + tsel;
     if (begin >= end) {   // uniform over the workgroup
-        if (g == 0 && n < p.G && !copier && (!D256 || (h & 1) == 0)) {
+        if (g == 0 && n < p.G && !copier && (!D256 || (h & 1) == 0) && (!LINEAR || tsel == 0)) {
             const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS_out + split_out;
             p.part_m[o] = -__builtin_inff();
             p.part_l[o] = 0.0f;
@@ -1056,8 +1080,13 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
                 c_page[k] = pg;
                 const int sub = (k < FULL || !kHalfTail) ? 0 : 8 * (ct & 1);
-                c_src[k] = staged_src_offset<PROD, HALF, DIM>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
-                c_dst[k] = kChunkDst<PROD, DIM>.off[c] + sub;
+                if constexpr (LINEAR) {     // the rows of a page, and of a tile in LDS, one after the other
+                    c_src[k] = 16u * uint32_t(c - pg * PC) + uint32_t(sub);
+                    c_dst[k] = kRowLds * (c / kChunksPerRow) + 16 * (c % kChunksPerRow) + sub;
+                } else {
+                    c_src[k] = staged_src_offset<PROD, HALF, DIM>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+                    c_dst[k] = kChunkDst<PROD, DIM>.off[c] + sub;
+                }
             }
             const bool has_rest = kHalfTail || ct < REST;
             auto c_issue = [&](uint4v (&r)[NR], int t0) {
@@ -1065,18 +1094,35 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 if constexpr (STORE) {
                     if (stores_token && t0 == last_t0 && !lds_flag_wait(&flags[7], 8u, p.spin_limit)) flags[2] = 1u;
                 }
-                const uint8_t* base[PPT];
+                constexpr int NBASE = LINEAR ? 1 : PPT;
+                const uint8_t* base[NBASE];
                 const int p0 = (t0 >> BSL) - split_p0;
+                if constexpr (!LINEAR) {
 #pragma unroll
-                for (int i = 0; i < PPT; ++i) base[i] = cache + int64_t(page_id(p0 + i)) * page_bytes;
+                    for (int i = 0; i < PPT; ++i) base[i] = cache + int64_t(page_id(p0 + i)) * page_bytes;
+                }
                 const uint32_t in_page = BS >= 32 ? uint32_t((t0 & (BS - 1)) * row_bytes) : 0u;
+                // LINEAR: a tile has 4 to 16 pages and a lane's chunks lie in several of them.  The tile's first page
+                // index is a multiple of its page count, so all its pages sit in one of the page-id registers, and
+                // a lane fetches the id of each of its pages from the lane that holds it.
+                int pv_tile = pv[0];
+                if constexpr (LINEAR) {
+#pragma unroll
+                    for (int r = 1; r < PVR; ++r) pv_tile = (p0 >> 6) == r ? pv[r] : pv_tile;
+                }
 #pragma unroll
                 for (int k = 0; k < NR; ++k) {
-                    constexpr bool kUniformPage = (BS * kChunksPerRow) % 64 == 0;
-                    const int pg_k = kUniformPage ? __builtin_amdgcn_readfirstlane(c_page[k]) : c_page[k];
-                    const uint8_t* b = base[0];
+                    const uint8_t* b;
+                    if constexpr (LINEAR) {
+                        const int id = __builtin_amdgcn_ds_bpermute(4 * ((p0 & 63) + c_page[k]), pv_tile);
+                        b = cache + int64_t(id) * page_bytes;
+                    } else {
+                        constexpr bool kUniformPage = (BS * kChunksPerRow) % 64 == 0;
+                        const int pg_k = kUniformPage ? __builtin_amdgcn_readfirstlane(c_page[k]) : c_page[k];
+                        b = base[0];
 #pragma unroll
-                    for (int i = 1; i < PPT; ++i) b = pg_k == i ? base[i] : b;
+                        for (int i = 1; i < PPT; ++i) b = pg_k == i ? base[i] : b;
+                    }
                     if (k < FULL) {
                         r[k] = *reinterpret_cast<const uint4v*>(b + in_page + c_src[k]);
                     } else if (!kHalfTail) {
@@ -1358,7 +1404,15 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         uint32_t vraw[2][4];
         float kn[NSC], vn[NSC], kg[NSC];
 #pragma unroll
-        for (int b = 0; b < 2; ++b) kraw[b] = *reinterpret_cast<const uint4v*>(tile + k_rd[b]);
+        for (int b = 0; b < 2; ++b) {
+            if constexpr (LINEAR) {     // a token's index bytes start at a multiple of 8 bytes
+                const uint2v lo = *reinterpret_cast<const uint2v*>(tile + k_rd[b]);
+                const uint2v hi = *reinterpret_cast<const uint2v*>(tile + k_rd[b] + 8);
+                kraw[b] = uint4v{lo.x, lo.y, hi.x, hi.y};
+            } else {
+                kraw[b] = *reinterpret_cast<const uint4v*>(tile + k_rd[b]);
+            }
+        }
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
@@ -1366,7 +1420,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
         for (int e = 0; e < NSC; ++e) {
             kn[e] = *reinterpret_cast<const float*>(tile + n_rd[e]);
-            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (DIM != 128 ? Cfg::VN_OFF - Cfg::KN_OFF : kStageVnOff - kStageKnOff));
+            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (LINEAR ? 68 * HPR : DIM != 128 ? Cfg::VN_OFF - Cfg::KN_OFF : kStageVnOff - kStageKnOff));
             kg[e] = PROD ? *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageKgOff - kStageKnOff)) : 0.0f;
         }
         // These were all the reads of the slot (the lookups below go to the table): it is handed back
@@ -1480,9 +1534,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             const float w = __builtin_amdgcn_exp2f(d);
             psum += w;
             wv[e] = w * rv[e];
-            // (HALF: the first tile of a split may hold no token of this wavefront's parity; -inf - -inf
+            // (MULTI > 0: the first tile of a split may hold no token of this wavefront; -inf - -inf
             // is then NaN in every lane, and the vote must still send the tile through the safe path)
-            redo = redo || (HALF ? !(d <= kMaxLead) : d > kMaxLead) || wv[e] > kHalfSafe;
+            redo = redo || (MULTI > 0 ? !(d <= kMaxLead) : d > kMaxLead) || wv[e] > kHalfSafe;
         }
         if (__any(redo)) {
             // The reference moves to max(M, max over the tile of (score + bias)), where the bias of a
@@ -1594,6 +1648,16 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             for (int mask = 4 * GP; mask < 64; mask <<= 1) v = sum_xor(v, mask);
             O[db][i] = v;
         }
+    if constexpr (LINEAR) {
+        // the partials of the wavefronts go through the tile slots: every computing wavefront must have fetched its
+        // operands of the last tiles (tile i lies in slot i % 2)
+        const int ntiles = (end - begin + 31) >> 5;
+        if (!lds_flag_wait(&flags[5], 8u * uint32_t((ntiles + 1) >> 1), p.spin_limit) ||
+            !lds_flag_wait(&flags[6], 8u * uint32_t(ntiles >> 1), p.spin_limit)) {
+            flags[2] = 1u;
+            handoff_failed = true;
+        }
+    }
     if constexpr (CW > 0) {
         // a hand-off that timed out, in the prologue or in the tile loop: the result cannot be
         // trusted, so it is made NaN and the fault is counted
@@ -1602,6 +1666,70 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             M = __builtin_nanf("");
             if (handoff_failed && lane == 0) atomicAdd(&g_decode_faults, 1u);
         }
+    }
+    if constexpr (LINEAR) {
+        // The TPR wavefronts of a head hold the partials of its tokens t mod TPR of every row.  They are merged here
+        // into the one partial of the split: each posts its own in LDS, and each then combines its share of the
+        // coordinates (128 / TPR of every query head) from all of them.
+        float* xacc = reinterpret_cast<float*>(slots);        // [wavefront][query head 0..15][128]
+        float* xml = xacc + 8 * 16 * 128;                     // [wavefront][query head][maximum, denominator]
+        if (g == 0 && n < p.G) {
+            xml[(h * 16 + n) * 2] = M;
+            xml[(h * 16 + n) * 2 + 1] = lsum;
+        }
+        if (g < GP / 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int head = 4 * g + i;
+                if (head < p.G) {
+                    float* dst = xacc + (h * 16 + head) * 128 + n * DPL;
+#pragma unroll
+                    for (int q4 = 0; q4 < DPL / 4; ++q4)
+                        *reinterpret_cast<float4v*>(dst + 4 * q4) = float4v{O[4 * q4][i], O[4 * q4 + 1][i], O[4 * q4 + 2][i], O[4 * q4 + 3][i]};
+                }
+            }
+        }
+        lds_flag_signal(&xflags[0], lane);
+        bool merged = lds_flag_wait(&xflags[0], 8u, p.spin_limit);
+        if (!merged && lane == 0) atomicAdd(&g_decode_faults, 1u);
+        constexpr int CPW = 128 / TPR;                        // coordinates of a head that this wavefront combines
+        auto merged_max = [&](int head, float (&mt)[TPR]) -> float {
+            float ms = -__builtin_inff();
+            bool bad = !merged;
+#pragma unroll
+            for (int t = 0; t < TPR; ++t) {
+                mt[t] = xml[((t * HPR + hr) * 16 + head) * 2];
+                bad = bad || mt[t] != mt[t];
+                ms = __builtin_fmaxf(ms, mt[t]);
+            }
+            return bad ? __builtin_nanf("") : ms;
+        };
+        for (int idx = lane; idx < p.G * CPW; idx += kWave) {
+            const int head = idx / CPW, c = CPW * tsel + (idx - head * CPW);
+            float mt[TPR];
+            const float ms = merged_max(head, mt);
+            float acc = 0.0f;
+#pragma unroll
+            for (int t = 0; t < TPR; ++t) {
+                const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(mt[t] - ms);
+                acc += w * xacc[((t * HPR + hr) * 16 + head) * 128 + c];
+            }
+            p.part_acc[((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS + split) * D + c] = acc;
+        }
+        if (tsel == 0 && lane < p.G) {
+            float mt[TPR];
+            const float ms = merged_max(lane, mt);
+            float l = 0.0f;
+#pragma unroll
+            for (int t = 0; t < TPR; ++t) {
+                const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(mt[t] - ms);
+                l += w * xml[((t * HPR + hr) * 16 + lane) * 2 + 1];
+            }
+            const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hr * p.G + lane) * NS + split;
+            p.part_m[o] = ms;
+            p.part_l[o] = l;
+        }
+        return;
     }
     if (g == 0 && n < p.G && (!D256 || (h & 1) == 0)) {        // D256: both halves hold the same maximum and denominator
         const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS_out + split_out;
@@ -1965,6 +2093,43 @@ int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wid
 #undef FQ_HALF_GP
 }
 
+// 1 or 2 KV heads of dimension 128 on pages of 16 or 32 tokens: the staged kernel on rows of 8 or 4 tokens kept in
+// LDS as they lie in the cache (`rows_per_page` = block_size * H_KV / 8); the wavefronts that share a head (one per
+// token of a row) merge their partials before they leave the workgroup.
+inline bool staged_linear_applies(int D, int H_KV, int block_size, const DecodeVariant& v) {
+    return D == 128 && (H_KV == 1 || H_KV == 2) && block_size >= 16 && !v.direct && v.copy_waves == 4;
+}
+template <int DT>
+int launch_staged_linear(const DecodeParams& p, int S, int rows_per_page, hipStream_t stream) {
+    const size_t lds = 2 * 32 * 1104;         // two tiles of 32 rows, a row every 1104 bytes
+    const dim3 grid(S, p.num_splits, 1), block(512 + 64 * 4);
+#define FQ_LINEAR_GP(BSL, GPV, MULTIV) \
+    return launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, MULTIV>, p, grid, block, lds, stream)
+#define FQ_LINEAR_BS(BSL, MULTIV)                            \
+    do {                                                     \
+        if (p.G <= 4) { FQ_LINEAR_GP(BSL, 4, MULTIV); }      \
+        else if (p.G <= 8) { FQ_LINEAR_GP(BSL, 8, MULTIV); } \
+        else { FQ_LINEAR_GP(BSL, 16, MULTIV); }              \
+    } while (0)
+    if (p.H_KV == 1) {
+        if (rows_per_page == 2) FQ_LINEAR_BS(1, 3);
+        else FQ_LINEAR_BS(2, 3);
+    } else {
+        if (rows_per_page == 4) FQ_LINEAR_BS(2, 2);
+        else FQ_LINEAR_BS(3, 2);
+    }
+#undef FQ_LINEAR_BS
+#undef FQ_LINEAR_GP
+}
+
+// Partials per split that the staged kernel writes for this shape when the switches let it run (the tokens of its
+// rows): what workspaces are sized for, whatever the switches say.
+inline int partials_per_split_room(int D, int H_KV, int block_size) {
+    if (block_size < 16) return 1;
+    if ((D == 128 && H_KV == 4) || (D == 64 && H_KV == 8)) return 2;
+    return 1;
+}
+
 // head_dim 64 on the staged kernel: pairs of neighbouring KV heads as heads of 128 (16 real heads a group), or, with
 // 8 KV heads on pages of 16 or 32 tokens, rows of two tokens of four such pairs.  Up to 8 query heads per KV head.
 inline bool staged_d64_full_applies(int D, int H_KV, int G, const DecodeVariant& v) {
@@ -2051,6 +2216,12 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
             const bool wide_rows = chunk_rows / rows_per_page > 64 || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256);
             return launch_staged_d64<DT>(ps, S, rows_per_page, wide_rows, d64_half, stream);
         }
+    }
+    if (allow_half && p.new_key == nullptr && staged_linear_applies(D, p.H_KV, BS, var)) {
+        const int rows_per_page = BS * p.H_KV / 8;
+        DecodeParams ps = p;
+        ps.balance_slots = staged_balance_slots(S, p.num_splits);
+        return launch_staged_linear<DT>(ps, S, rows_per_page, stream);
     }
     if (allow_half && staged_half_applies(D, p.H_KV, BS, var)) {
         // the kernel counts rows of two tokens: half the page size, chunks of rows
@@ -2171,7 +2342,7 @@ int launch_reduce(const float* acc, const float* m, const float* l, const float*
     return fq_host::check_launch();
 }
 
-int effective_splits(int num_splits, int num_seqs, int H_KV, int block_size, int max_blocks_per_seq);
+int effective_splits(int num_splits, int num_seqs, int H_KV, int D, int block_size, int max_blocks_per_seq);
 
 inline int check_decode_shape(int num_seqs, int H_Q, int H_KV, int D, int block_size, int max_blocks_per_seq,
                               int64_t num_blocks, int dtype, int num_splits) {
@@ -2217,25 +2388,32 @@ extern "C" int fq_paged_decode_min_splits(int block_size, int max_blocks_per_seq
     return int(ns < 1 ? 1 : ns);
 }
 
-extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_size, int max_blocks_per_seq) {
+namespace fq {
+int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_per_seq) {
     if (num_seqs <= 0 || H_KV <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 1;
     const int64_t max_ctx = int64_t(block_size) * max_blocks_per_seq;
     const int64_t tiles = (max_ctx + 63) / 64;
     // one round of workgroups over the chip (8 wavefronts per CU, one wavefront per sequence,
     // KV head and split) ...
     const int64_t target_waves = int64_t(fq_host::device_cu_count()) * 8;
-    // (4 KV heads run as 8: the staged kernel reads their tokens in pairs)
-    const int64_t heads = H_KV == 4 ? 8 : H_KV;
+    // (4 KV heads run as 8: the staged kernel reads their tokens in pairs; 1 and 2 of dimension 128 likewise, in
+    // rows of 8 and 4 tokens)
+    const bool rows_of_tokens = D == 128 && H_KV <= 2 && block_size >= 16;
+    const int64_t heads = (H_KV == 4 || rows_of_tokens) ? 8 : H_KV;
     const int64_t one_round = (target_waves + int64_t(num_seqs) * heads - 1) / (int64_t(num_seqs) * heads);
     // ... and twice that when the contexts are long enough for splits of 1024 tokens: the lengths
     // of the sequences are not known here, a ragged batch leaves many splits empty, and the
     // kernel can merge splits (it sizes its chunks from the actual lengths) but not divide them
-    int64_t ns = 2 * one_round < max_ctx / 1024 ? 2 * one_round : max_ctx / 1024;
+    // (rows of tokens: chunks of 1024 rows, not tokens)
+    const int64_t long_chunks = rows_of_tokens ? max_ctx * H_KV / 8192 : max_ctx / 1024;
+    int64_t ns = 2 * one_round < long_chunks ? 2 * one_round : long_chunks;
     if (ns < one_round) ns = one_round;
     // Fewer than 8 KV heads run the direct kernel, whose workgroups are as small as the head count: a
     // round over the chip would cut a short context into chunks that cost more to launch and combine
     // than to read (measured on 32 x 4096 tokens: 1 KV head 85 us at 64 splits, 37 us at 16).
     if (H_KV < 8 && ns > max_ctx / 256) ns = max_ctx / 256;
+    // (a chunk is at least 64 rows)
+    if (rows_of_tokens && ns > max_ctx * H_KV / 512) ns = max_ctx * H_KV / 512;
     if (ns > tiles) ns = tiles;
     // Beyond 128 splits the combine step (one pass over the maxima per 64 splits, one partial row
     // per split) costs more than the shorter chunks save (measured on 1 x 32768 tokens, 8 KV
@@ -2246,9 +2424,15 @@ extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_siz
     if (ns < 1) ns = 1;
     return int(ns);
 }
+}  // namespace fq
 
-int fq::effective_splits(int num_splits, int num_seqs, int H_KV, int block_size, int max_blocks_per_seq) {
-    if (num_splits <= 0) return fq_paged_decode_auto_splits(num_seqs, H_KV, block_size, max_blocks_per_seq);
+// (for head_dim 128; the other head dimensions differ for 1 and 2 KV heads)
+extern "C" int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_size, int max_blocks_per_seq) {
+    return fq::auto_splits(num_seqs, H_KV, 128, block_size, max_blocks_per_seq);
+}
+
+int fq::effective_splits(int num_splits, int num_seqs, int H_KV, int D, int block_size, int max_blocks_per_seq) {
+    if (num_splits <= 0) return auto_splits(num_seqs, H_KV, D, block_size, max_blocks_per_seq);
     const int floor_ns = fq_paged_decode_min_splits(block_size, max_blocks_per_seq);
     return num_splits < floor_ns ? floor_ns : num_splits;
 }
@@ -2256,9 +2440,9 @@ int fq::effective_splits(int num_splits, int num_seqs, int H_KV, int block_size,
 extern "C" size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_KV, int D, int block_size,
                                                   int max_blocks_per_seq, int num_splits) {
     if (num_seqs <= 0 || H_Q <= 0 || H_KV <= 0 || D <= 0) return 0;
-    num_splits = fq::effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
-    // room for the two partials per split of the 4-KV-head staged decode, whatever the switches say
-    if ((D == 128 && H_KV == 4 && block_size >= 16) || (D == 64 && H_KV == 8 && block_size >= 16)) num_splits *= 2;
+    num_splits = fq::effective_splits(num_splits, num_seqs, H_KV, D, block_size, max_blocks_per_seq);
+    // room for the partials per split of the staged decode on rows of several tokens
+    num_splits *= fq::partials_per_split_room(D, H_KV, block_size);
     return fq::workspace_layout(num_seqs, H_Q, D, num_splits).total;
 }
 
@@ -2387,11 +2571,12 @@ int split_k_paged_decode_impl(const void* q, const uint8_t* kv_cache, const int3
     if (num_seqs == 0) return FQ_OK;
     if (!q || !out) return FQ_ERR_NULL_POINTER;
     if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16)) return FQ_ERR_MISALIGNED;
-    num_splits = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
-    // 4 KV heads: the staged kernel reads rows of two tokens and writes one partial per token parity
+    num_splits = effective_splits(num_splits, num_seqs, H_KV, D, block_size, max_blocks_per_seq);
+    // fewer than 8 KV heads: the staged kernel reads rows of several tokens and writes one partial per token of a row
     const int G = H_Q / H_KV;
-    const bool half = staged_half_applies(D, H_KV, block_size, var) || staged_d64_half_applies(D, H_KV, G, block_size, var);
-    const int num_partials = half ? 2 * num_splits : num_splits;
+    const bool linear = token == nullptr && staged_linear_applies(D, H_KV, block_size, var);
+    const bool half = linear || staged_half_applies(D, H_KV, block_size, var) || staged_d64_half_applies(D, H_KV, G, block_size, var);
+    const int num_partials = (half && !linear) ? 2 * num_splits : num_splits;
     const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_partials);
     if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
     if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;
@@ -2523,11 +2708,11 @@ extern "C" int fq_split_k_paged_decode_static(const void* q, const uint8_t* kv_c
                                        num_splits);
     if (bad != FQ_OK) return bad;
     if (num_seqs == 0) return FQ_OK;
-    const int ns = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
+    const int ns = effective_splits(num_splits, num_seqs, H_KV, D, block_size, max_blocks_per_seq);
     // the partials of this launch must fit the array: a larger problem is refused, not truncated (room
-    // for the two partials per split of the 4-KV-head staged decode whatever the switches say, as in
+    // for the partials per split of the staged decode on rows of several tokens whatever the switches say, as in
     // fq_paged_decode_workspace_bytes: the call below reads the switches once for itself)
-    const int num_partials = ((D == 128 && H_KV == 4) || (D == 64 && H_KV == 8)) && block_size >= 16 ? 2 * ns : ns;
+    const int num_partials = ns * partials_per_split_room(D, H_KV, block_size);
     if (workspace_layout(num_seqs, H_Q, D, num_partials).total > kStaticScratchBytes) return FQ_ERR_WORKSPACE;
     void* ws = nullptr;
     const int st = static_scratch_address(&ws);
@@ -2562,7 +2747,7 @@ extern "C" int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, cons
     if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16) || !fq_host::aligned(kv_cache, 16) ||
         !fq_host::aligned(rotation, 16) || !fq_host::aligned(sketch, 16))
         return FQ_ERR_MISALIGNED;
-    num_splits = effective_splits(num_splits, num_seqs, H_KV, block_size, max_blocks_per_seq);
+    num_splits = effective_splits(num_splits, num_seqs, H_KV, D, block_size, max_blocks_per_seq);
     const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_splits);
     if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
     if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;

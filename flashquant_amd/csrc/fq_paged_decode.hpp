@@ -50,7 +50,8 @@ struct DecodeParams {
 // cheapest: same inputs, same arithmetic, same answer in every workgroup.  Larger chunks
 // only: the split count bounds the chunk from below.  On return `chunk` is the chosen size,
 // (`seq`, `split`) the pair this workgroup takes and `L_known` its sequence's length.
-template <int PVR, int BS, bool HALF>
+// TPR: tokens per row of the kernel (rows of 2, 4 or 8 consecutive tokens when the model has 4, 2 or 1 KV heads)
+template <int PVR, int BS, int TPR>
 __device__ __forceinline__ void balance_chunks(const DecodeParams& p, int lane, int NS, bool rowwide, int& chunk, int& seq,
                                                int& split, int& L_known) {
     const int cap = rowwide ? chunk * NS : 64 * PVR * BS;       // page ids of a split: 64 * PVR lanes
@@ -61,8 +62,8 @@ __device__ __forceinline__ void balance_chunks(const DecodeParams& p, int lane, 
     const float rc = __builtin_amdgcn_rcpf(float(cand));
     const int nseq = int(gridDim.x);
     int l_real = lane < nseq ? p.seq_lens[lane] : 0;
-    l_real = l_real < 0 ? 0 : (l_real > p.max_blocks * BS * (HALF ? 2 : 1) ? p.max_blocks * BS * (HALF ? 2 : 1) : l_real);
-    const int l_mine = HALF ? (l_real + 1) >> 1 : l_real;      // in rows
+    l_real = l_real < 0 ? 0 : (l_real > p.max_blocks * BS * TPR ? p.max_blocks * BS * TPR : l_real);
+    const int l_mine = (l_real + TPR - 1) / TPR;               // in rows
     float groups = 0.0f;
     for (int sq = 0; sq < nseq; ++sq)
         groups += __builtin_ceilf(float(__builtin_amdgcn_readlane(l_mine, sq)) * rc - 0.0009765625f);

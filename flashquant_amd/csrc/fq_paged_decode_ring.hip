@@ -117,7 +117,6 @@ __global__ __launch_bounds__(1024) void paged_decode_ring_kernel(const DecodePar
     constexpr int NSC = GP / 4;           // scores a lane keeps per 16-token block
     constexpr int STAGE = kRingStageBytes;
     constexpr int RPP = BS >= 16 ? 16 : 8;   // rows of a stage that lie in one page
-    constexpr bool HALF = false;
 
     __shared__ __attribute__((aligned(256))) uint32_t lut[kShared ? kLutWords / 2 : kLutWords];
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];   // kRingStages stages
@@ -185,7 +184,7 @@ __global__ __launch_bounds__(1024) void paged_decode_ring_kernel(const DecodePar
     int chunk = (((p.max_blocks * BS + NS - 1) / NS) + 63) & ~63;
     int L_known = -1;
     if (p.balance_slots > 0) {
-        balance_chunks<PVR, BS, HALF>(p, lane, NS, rowwide, chunk, seq, split, L_known);
+        balance_chunks<PVR, BS, 1>(p, lane, NS, rowwide, chunk, seq, split, L_known);
         // the same in every lane: kept in scalar registers from here on
         chunk = __builtin_amdgcn_readfirstlane(chunk);
         seq = __builtin_amdgcn_readfirstlane(seq);

@@ -486,7 +486,9 @@ int fq_prod_paged_decode(const void* q, const uint8_t* kv_cache, const int32_t* 
  */
 int fq_paged_decode_fault_count(unsigned int* count);
 
-/* Number of splits fq_split_k_paged_decode uses when num_splits == 0
+/* Number of splits fq_split_k_paged_decode uses when num_splits == 0, at
+ * head_dim 128 (with 1 or 2 KV heads the other head dimensions run another
+ * kernel and take another count)
  * (counterpart of paged_tq4_decode_num_splits, csrc/cuda/paged_decode.cu:424-426,
  * which is a constant 4 there). */
 int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_size,

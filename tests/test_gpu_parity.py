@@ -512,12 +512,42 @@ def test_paged_decode_four_kv_heads_ragged_long_contexts():
 
 @pytest.mark.parametrize("hkv,d,splits", [(1, 128, 0), (1, 128, 5), (2, 128, 3), (2, 64, 8), (1, 256, 6), (2, 256, 4),
                                           (1, 128, 40)])
-def test_paged_decode_one_or_two_kv_heads_share_a_workgroup_over_splits(hkv, d, splits):
-    """With 1 or 2 KV heads the wavefronts of a workgroup beyond the heads take the following splits (odd
-    split counts leave some of them without work, ragged lengths leave others with an empty split)."""
+def test_paged_decode_one_or_two_kv_heads_share_a_workgroup_over_splits(hkv, d, splits, kernel_option):
+    """With 1 or 2 KV heads the wavefronts of a workgroup of the direct kernel beyond the heads take the
+    following splits (odd split counts leave some of them without work, ragged lengths leave others
+    with an empty split)."""
+    kernel_option("decode_direct", True)
     lens = [70, 0, 700, 16, 129, 1, 333, 64]
     _decode_case(lens, hq=4 * hkv, hkv=hkv, d=d, bs=16, num_splits=splits, seed=47)
     _decode_case(lens, hq=hkv, hkv=hkv, d=d, bs=32, num_splits=splits, seed=48, dtype=torch.float16)
+
+
+@pytest.mark.parametrize("hq,hkv,bs,splits,dtype", [(8, 1, 16, 0, torch.bfloat16), (4, 1, 16, 3, torch.bfloat16),
+                                                    (16, 1, 32, 2, torch.float16), (1, 1, 16, 1, torch.bfloat16),
+                                                    (5, 1, 32, 5, torch.float16), (8, 1, 16, 40, torch.bfloat16),
+                                                    (8, 2, 16, 0, torch.bfloat16), (16, 2, 16, 3, torch.float16),
+                                                    (32, 2, 32, 2, torch.bfloat16), (2, 2, 32, 1, torch.float16),
+                                                    (14, 2, 16, 5, torch.bfloat16), (8, 2, 32, 40, torch.bfloat16)])
+def test_paged_decode_one_or_two_kv_heads_on_rows_of_tokens(hq, hkv, bs, splits, dtype, kernel_option):
+    """1 or 2 KV heads of dimension 128 on pages of 16 or 32 tokens run the staged kernel on rows of 8 or 4
+    tokens (the token rows lie in LDS as in the cache; token t of a head goes to the wavefront t mod 8 or
+    t mod 4 of it, and each wavefront's part is a partial of its own).  Lengths that fill a row, leave
+    every number of tokens in the last one, end one past a chunk of 64 rows, empty sequences; against
+    the oracle, and the direct kernel (also the one that serves pages of 8 tokens) agrees."""
+    lens = [70, 0, 333, 16, 129, 1, 2, 3, 5, 7, 8, 9, 513, 1025, 127, 128, 700]
+    _decode_case(lens, hq=hq, hkv=hkv, bs=bs, num_splits=splits, seed=53, dtype=dtype)
+    kernel_option("decode_direct", True)
+    _decode_case(lens, hq=hq, hkv=hkv, bs=bs, num_splits=splits, seed=53, dtype=dtype)
+
+
+def test_paged_decode_one_or_two_kv_heads_ragged_long_contexts():
+    """More (sequence, split) workgroups than CUs with 1 and 2 KV heads: chunks sized from the actual
+    lengths, counted in rows of 8 and 4 tokens."""
+    lens = [1500, 0, 37, 6001, 64, 2049, 1, 3333]
+    _decode_case(lens, hq=8, hkv=1, num_splits=40)
+    _decode_case(lens, hq=16, hkv=2, num_splits=64, bs=32, dtype=torch.float16)
+    _decode_case(lens, hq=8, hkv=2, num_splits=0, bs=8)           # pages of 8 tokens: the direct kernel
+    _decode_case([20000, 17, 9000], hq=8, hkv=1, num_splits=0)    # more than 256 pages a sequence
 
 
 def test_paged_decode_rotated_space_and_out_argument():
