@@ -589,6 +589,9 @@ def main():
         for name, (n_seq, ctx, hq, hkv, d) in ({} if args.skip_other_shapes else {
             "decode_32x16384_32q_8kv_d128": (32, 16384, 32, 8, 128),
             "decode_32x4096_32q_4kv_d128": (32, 4096, 32, 4, 128),
+            "decode_128x8192_8q_1kv_d128": (128, 8192, 8, 1, 128),      # a tensor-parallel shard of a model with 8 KV heads
+            "decode_32x4096_8q_1kv_d128": (32, 4096, 8, 1, 128),
+            "decode_128x8192_16q_2kv_d128": (128, 8192, 16, 2, 128),
             "decode_32x4096_32q_8kv_d64": (32, 4096, 32, 8, 64),
             "decode_32x4096_32q_8kv_d256": (32, 4096, 32, 8, 256),
         }).items():
