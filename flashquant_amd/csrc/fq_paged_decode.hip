@@ -708,7 +708,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     constexpr int TPR = 1 << MULTI;          // tokens per row
     constexpr int HPR = 8 / TPR;             // real KV heads per row
     static_assert(MULTI >= 0 && MULTI <= 3, "rows of 1, 2, 4 or 8 tokens");
-    static_assert(!LINEAR || (DIM == 128 && !PROD && !STORE && CW > 0), "rows of 4 and 8 tokens: TQ4, head_dim 128, copy wavefronts");
+    static_assert(!LINEAR || (DIM == 128 && !PROD && CW > 0), "rows of 4 and 8 tokens: TQ4, head_dim 128, copy wavefronts");
     static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
     static_assert(DIM == 128 || (!PROD && !STORE && CW > 0), "head_dim 64 / 256 are served by the TQ4 form with copy wavefronts");
@@ -956,12 +956,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     }
     // STORE: the new token's rows and slot are asked for with the other prologue loads, by every workgroup
     // (which one needs them depends on the sequence length, which is on its way)
-    constexpr int kNewHeads = HALF ? 4 : 8;                 // KV heads of this workgroup
+    constexpr int kNewHeads = HPR;                          // KV heads of this workgroup
     uint4v new_raw[4];
     int64_t new_slot = -1;
     if constexpr (STORE) {
         if (!copier) {
-            const int kv_heads = HALF ? 4 : p.H_KV;
+            const int kv_heads = MULTI > 0 ? HPR : p.H_KV;
             const int nr = n < 2 * kNewHeads ? n : 2 * kNewHeads - 1;     // block row: key head nr, or value head nr - KH
             const uint16_t* xrow = reinterpret_cast<const uint16_t*>(nr < kNewHeads ? p.new_key : p.new_value) +
                                    (int64_t(seq) * kv_heads + kNewHeads * hgrp + (nr & (kNewHeads - 1))) * 128;
@@ -1106,9 +1106,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 // index is a multiple of its page count, so all its pages sit in one of the page-id registers, and
                 // a lane fetches the id of each of its pages from the lane that holds it.
                 int pv_tile = pv[0];
-                if constexpr (LINEAR) {
+                if constexpr (LINEAR) {     // (masks, not selects: the compiler turns a chain of selects on pv[] into
+                                            // an indexed array in scratch memory)
+                    const int sel = __builtin_amdgcn_readfirstlane(p0 >> 6);
+                    pv_tile = 0;
 #pragma unroll
-                    for (int r = 1; r < PVR; ++r) pv_tile = (p0 >> 6) == r ? pv[r] : pv_tile;
+                    for (int r = 0; r < PVR; ++r) pv_tile |= pv[r] & (sel == r ? -1 : 0);
                 }
 #pragma unroll
                 for (int k = 0; k < NR; ++k) {
@@ -1250,8 +1253,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                     // (cpu_reference.py:22-61, vllm/impl.py:220-263).  Wavefront h holds columns 16h..16h+15.
                     // Block row r: key head r for r < KH, value head r - KH for r < 2 KH.
                     constexpr int KH = kNewHeads;
-                    const int token_row_bytes = HALF ? 544 : row_bytes;
-                    const int kv_heads = HALF ? 4 : p.H_KV;
+                    const int token_row_bytes = MULTI > 0 ? 136 * HPR : row_bytes;
+                    const int kv_heads = MULTI > 0 ? HPR : p.H_KV;
                     const int64_t slot = new_slot;
                     uint4v raw[KS];
 #pragma unroll
@@ -1693,36 +1696,37 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         bool merged = lds_flag_wait(&xflags[0], 8u, p.spin_limit);
         if (!merged && lane == 0) atomicAdd(&g_decode_faults, 1u);
         constexpr int CPW = 128 / TPR;                        // coordinates of a head that this wavefront combines
-        auto merged_max = [&](int head, float (&mt)[TPR]) -> float {
+        // maximum over the wavefronts of this head (NaN when a hand-off failed), no array: the values are read again
+        auto merged_max = [&](int head) __attribute__((always_inline)) -> float {
             float ms = -__builtin_inff();
             bool bad = !merged;
 #pragma unroll
             for (int t = 0; t < TPR; ++t) {
-                mt[t] = xml[((t * HPR + hr) * 16 + head) * 2];
-                bad = bad || mt[t] != mt[t];
-                ms = __builtin_fmaxf(ms, mt[t]);
+                const float m = xml[((t * HPR + hr) * 16 + head) * 2];
+                bad = bad || m != m;
+                ms = __builtin_fmaxf(ms, m);
             }
             return bad ? __builtin_nanf("") : ms;
         };
         for (int idx = lane; idx < p.G * CPW; idx += kWave) {
             const int head = idx / CPW, c = CPW * tsel + (idx - head * CPW);
-            float mt[TPR];
-            const float ms = merged_max(head, mt);
+            const float ms = merged_max(head);
             float acc = 0.0f;
 #pragma unroll
             for (int t = 0; t < TPR; ++t) {
-                const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(mt[t] - ms);
+                const float m = xml[((t * HPR + hr) * 16 + head) * 2];
+                const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(m - ms);
                 acc += w * xacc[((t * HPR + hr) * 16 + head) * 128 + c];
             }
             p.part_acc[((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS + split) * D + c] = acc;
         }
         if (tsel == 0 && lane < p.G) {
-            float mt[TPR];
-            const float ms = merged_max(lane, mt);
+            const float ms = merged_max(lane);
             float l = 0.0f;
 #pragma unroll
             for (int t = 0; t < TPR; ++t) {
-                const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(mt[t] - ms);
+                const float m = xml[((t * HPR + hr) * 16 + lane) * 2];
+                const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(m - ms);
                 l += w * xml[((t * HPR + hr) * 16 + lane) * 2 + 1];
             }
             const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hr * p.G + lane) * NS + split;
@@ -2103,7 +2107,10 @@ template <int DT>
 int launch_staged_linear(const DecodeParams& p, int S, int rows_per_page, hipStream_t stream) {
     const size_t lds = 2 * 32 * 1104;         // two tiles of 32 rows, a row every 1104 bytes
     const dim3 grid(S, p.num_splits, 1), block(512 + 64 * 4);
-#define FQ_LINEAR_GP(BSL, GPV, MULTIV) \
+    const bool store = p.new_key != nullptr;
+#define FQ_LINEAR_GP(BSL, GPV, MULTIV)                                                                                \
+    if (store)                                                                                                        \
+        return launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, MULTIV, true>, p, grid, block, lds, stream); \
     return launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, MULTIV>, p, grid, block, lds, stream)
 #define FQ_LINEAR_BS(BSL, MULTIV)                            \
     do {                                                     \
@@ -2217,7 +2224,7 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
             return launch_staged_d64<DT>(ps, S, rows_per_page, wide_rows, d64_half, stream);
         }
     }
-    if (allow_half && p.new_key == nullptr && staged_linear_applies(D, p.H_KV, BS, var)) {
+    if (allow_half && staged_linear_applies(D, p.H_KV, BS, var)) {
         const int rows_per_page = BS * p.H_KV / 8;
         DecodeParams ps = p;
         ps.balance_slots = staged_balance_slots(S, p.num_splits);
@@ -2574,7 +2581,7 @@ int split_k_paged_decode_impl(const void* q, const uint8_t* kv_cache, const int3
     num_splits = effective_splits(num_splits, num_seqs, H_KV, D, block_size, max_blocks_per_seq);
     // fewer than 8 KV heads: the staged kernel reads rows of several tokens and writes one partial per token of a row
     const int G = H_Q / H_KV;
-    const bool linear = token == nullptr && staged_linear_applies(D, H_KV, block_size, var);
+    const bool linear = staged_linear_applies(D, H_KV, block_size, var);
     const bool half = linear || staged_half_applies(D, H_KV, block_size, var) || staged_d64_half_applies(D, H_KV, G, block_size, var);
     const int num_partials = (half && !linear) ? 2 * num_splits : num_splits;
     const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_partials);
@@ -2641,7 +2648,8 @@ extern "C" int fq_tq4_store_and_decode(const void* key, const void* value, const
         return FQ_ERR_MISALIGNED;
     const DecodeVariant var = read_decode_variant();
     const bool in_launch = centroids_k && var.copy_waves == 4 &&
-                           ((staged_applies(D, H_KV, var) && !var.ring) || staged_half_applies(D, H_KV, block_size, var));
+                           ((staged_applies(D, H_KV, var) && !var.ring) || staged_half_applies(D, H_KV, block_size, var) ||
+                            staged_linear_applies(D, H_KV, block_size, var));
     const NewToken token{key, value, slot_mapping, boundaries, kv_cache};
     if (!in_launch) {
         const int st = fq_tq4_compress_store(key, value, dtype, rot_T_even, rot_T_odd, boundaries, kv_cache, slot_mapping,

@@ -41,14 +41,14 @@ def test_random_paged_decode(case):
                    num_splits=rng.choice([0, 1, 2, 3, 5, 8, 17]), seed=100 + case)
 
 
-@pytest.mark.parametrize("case", range(30))
+@pytest.mark.parametrize("case", range(40))
 def test_random_store_and_decode(case, kernel_option):
     """The serving step (new token stored, then decoded over) on random shapes: the in-launch store where the
     staged kernel runs, the two launches elsewhere."""
     kernel_option("compress_three_terms", True)
     rng = random.Random(9500 + case)
     d = rng.choice([128, 128, 128, 128, 64, 256])
-    hkv = rng.choice([8, 8, 8, 16, 24, 4, 2]) if d == 128 else rng.choice([8, 4, 2])
+    hkv = rng.choice([8, 8, 8, 16, 24, 4, 2, 1]) if d == 128 else rng.choice([8, 4, 2])
     g = rng.choice([1, 2, 4, 4, 5, 8, 16]) if d != 256 else rng.choice([1, 2, 4])
     n_seq = rng.choice([1, 2, 3, 5, 9, 17, 33])
     longest = rng.choice([40, 130, 300, 700, 1500, 3000])
