@@ -35,7 +35,7 @@ H_Q, H_KV, D, BS = 32, 8, 128, 16
 BATCH, CTX = 32, 4096
 EXTRA_ITERS = 20              # timed calls of every leg other than the headline
 ROW_BYTES = H_KV * (D + 8)
-DOMINANT_KERNEL = "paged_decode_staged_kernel<4,4,bf16,4,false,4,false,false,128>"
+DOMINANT_KERNEL = "paged_decode_staged_kernel<4,4,bf16,4,false,4,0,false,128>"
 
 
 def log(*a):
