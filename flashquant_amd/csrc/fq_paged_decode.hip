@@ -703,11 +703,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // 8-head row.  2, 3 (LINEAR): 2 KV heads or 1; the token rows go to LDS as they lie in the cache (their
     // sections start at multiples of 8 and 4 bytes, not of the 16 of a copy chunk) and the computing wavefronts
     // read their operands from where they are.
+    // 4: rows of 2 tokens of 4 KV heads in the LINEAR form.
     constexpr bool HALF = MULTI == 1;
     constexpr bool LINEAR = MULTI >= 2;
-    constexpr int TPR = 1 << MULTI;          // tokens per row
+    constexpr int TPR = MULTI == 4 ? 2 : 1 << MULTI;     // tokens per row
     constexpr int HPR = 8 / TPR;             // real KV heads per row
-    static_assert(MULTI >= 0 && MULTI <= 3, "rows of 1, 2, 4 or 8 tokens");
+    static_assert(MULTI >= 0 && MULTI <= 4, "rows of 1, 2, 4 or 8 tokens");
     static_assert(!LINEAR || (DIM == 128 && !PROD && CW > 0), "rows of 4 and 8 tokens: TQ4, head_dim 128, copy wavefronts");
     static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
@@ -2069,39 +2070,11 @@ int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream
     return FQ_ERR_UNSUPPORTED_BLOCK;
 }
 
-// 4 KV heads of dimension 128 on pages of 16 or 32 tokens: the staged kernel on rows of two tokens
-// (`rows_per_page` = block_size / 2), with its copy wavefronts.
-inline bool staged_half_applies(int D, int H_KV, int block_size, const DecodeVariant& v) {
-    return D == 128 && H_KV == 4 && block_size >= 16 && !v.direct && v.copy_waves == 4;
-}
-template <int DT>
-int launch_staged_half(const DecodeParams& p, int S, int rows_per_page, bool wide, hipStream_t stream) {
-    const size_t lds = 2 * size_t(StagedCfg<false>::TILE_BYTES);
-    const dim3 grid(S, p.num_splits, 1), block(512 + 64 * 4);
-    const bool store = p.new_key != nullptr;
-#define FQ_HALF_GP(BSL, GPV)                                                                                      \
-    if (store)                                                                                                    \
-        return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, true, true>, p, grid, block, lds, stream) \
-                    : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, true, true>, p, grid, block, lds, stream); \
-    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, true>, p, grid, block, lds, stream) \
-                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, true>, p, grid, block, lds, stream)
-#define FQ_HALF_BS(BSL)                          \
-    do {                                         \
-        if (p.G <= 4) { FQ_HALF_GP(BSL, 4); }    \
-        else if (p.G <= 8) { FQ_HALF_GP(BSL, 8); } \
-        else { FQ_HALF_GP(BSL, 16); }            \
-    } while (0)
-    if (rows_per_page == 8) FQ_HALF_BS(3);
-    else FQ_HALF_BS(4);
-#undef FQ_HALF_BS
-#undef FQ_HALF_GP
-}
-
-// 1 or 2 KV heads of dimension 128 on pages of 16 or 32 tokens: the staged kernel on rows of 8 or 4 tokens kept in
-// LDS as they lie in the cache (`rows_per_page` = block_size * H_KV / 8); the wavefronts that share a head (one per
+// 1, 2 or 4 KV heads of dimension 128 on pages of 16 or 32 tokens: the staged kernel on rows of 8, 4 or 2 tokens kept
+// in LDS as they lie in the cache (`rows_per_page` = block_size * H_KV / 8); the wavefronts that share a head (one per
 // token of a row) merge their partials before they leave the workgroup.
 inline bool staged_linear_applies(int D, int H_KV, int block_size, const DecodeVariant& v) {
-    return D == 128 && (H_KV == 1 || H_KV == 2) && block_size >= 16 && !v.direct && v.copy_waves == 4;
+    return D == 128 && (H_KV == 1 || H_KV == 2 || H_KV == 4) && block_size >= 16 && !v.direct && v.copy_waves == 4;
 }
 template <int DT>
 int launch_staged_linear(const DecodeParams& p, int S, int rows_per_page, hipStream_t stream) {
@@ -2121,9 +2094,12 @@ int launch_staged_linear(const DecodeParams& p, int S, int rows_per_page, hipStr
     if (p.H_KV == 1) {
         if (rows_per_page == 2) FQ_LINEAR_BS(1, 3);
         else FQ_LINEAR_BS(2, 3);
-    } else {
+    } else if (p.H_KV == 2) {
         if (rows_per_page == 4) FQ_LINEAR_BS(2, 2);
         else FQ_LINEAR_BS(3, 2);
+    } else {
+        if (rows_per_page == 8) FQ_LINEAR_BS(3, 4);
+        else FQ_LINEAR_BS(4, 4);
     }
 #undef FQ_LINEAR_BS
 #undef FQ_LINEAR_GP
@@ -2133,7 +2109,7 @@ int launch_staged_linear(const DecodeParams& p, int S, int rows_per_page, hipStr
 // rows): what workspaces are sized for, whatever the switches say.
 inline int partials_per_split_room(int D, int H_KV, int block_size) {
     if (block_size < 16) return 1;
-    if ((D == 128 && H_KV == 4) || (D == 64 && H_KV == 8)) return 2;
+    if (D == 64 && H_KV == 8) return 2;
     return 1;
 }
 
@@ -2229,16 +2205,6 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
         DecodeParams ps = p;
         ps.balance_slots = staged_balance_slots(S, p.num_splits);
         return launch_staged_linear<DT>(ps, S, rows_per_page, stream);
-    }
-    if (allow_half && staged_half_applies(D, p.H_KV, BS, var)) {
-        // the kernel counts rows of two tokens: half the page size, chunks of rows
-        const int rows_per_page = BS / 2;
-        const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
-        const int64_t chunk_rows = (((max_rows + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
-        DecodeParams ps = p;
-        ps.balance_slots = staged_balance_slots(S, p.num_splits);
-        const bool wide_rows = chunk_rows / rows_per_page > 64 || ps.balance_slots > 0 || (p.max_blocks > 64 && p.max_blocks <= 256);
-        return launch_staged_half<DT>(ps, S, rows_per_page, wide_rows, stream);
     }
     // pages a split can span: its tokens are ceil(max_ctx / splits) rounded up to a tile
     const int64_t max_ctx = int64_t(p.max_blocks) * BS;
@@ -2404,8 +2370,8 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     // KV head and split) ...
     const int64_t target_waves = int64_t(fq_host::device_cu_count()) * 8;
     // (4 KV heads run as 8: the staged kernel reads their tokens in pairs; 1 and 2 of dimension 128 likewise, in
-    // rows of 8 and 4 tokens)
-    const bool rows_of_tokens = D == 128 && H_KV <= 2 && block_size >= 16;
+    // rows of 8 and 4 tokens; `rows_of_tokens`: the forms that count their chunks in such rows)
+    const bool rows_of_tokens = D == 128 && (H_KV == 1 || H_KV == 2 || H_KV == 4) && block_size >= 16;
     const int64_t heads = (H_KV == 4 || rows_of_tokens) ? 8 : H_KV;
     const int64_t one_round = (target_waves + int64_t(num_seqs) * heads - 1) / (int64_t(num_seqs) * heads);
     // ... and twice that when the contexts are long enough for splits of 1024 tokens: the lengths
@@ -2582,7 +2548,7 @@ int split_k_paged_decode_impl(const void* q, const uint8_t* kv_cache, const int3
     // fewer than 8 KV heads: the staged kernel reads rows of several tokens and writes one partial per token of a row
     const int G = H_Q / H_KV;
     const bool linear = staged_linear_applies(D, H_KV, block_size, var);
-    const bool half = linear || staged_half_applies(D, H_KV, block_size, var) || staged_d64_half_applies(D, H_KV, G, block_size, var);
+    const bool half = linear || staged_d64_half_applies(D, H_KV, G, block_size, var);
     const int num_partials = (half && !linear) ? 2 * num_splits : num_splits;
     const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_partials);
     if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
@@ -2648,8 +2614,7 @@ extern "C" int fq_tq4_store_and_decode(const void* key, const void* value, const
         return FQ_ERR_MISALIGNED;
     const DecodeVariant var = read_decode_variant();
     const bool in_launch = centroids_k && var.copy_waves == 4 &&
-                           ((staged_applies(D, H_KV, var) && !var.ring) || staged_half_applies(D, H_KV, block_size, var) ||
-                            staged_linear_applies(D, H_KV, block_size, var));
+                           ((staged_applies(D, H_KV, var) && !var.ring) || staged_linear_applies(D, H_KV, block_size, var));
     const NewToken token{key, value, slot_mapping, boundaries, kv_cache};
     if (!in_launch) {
         const int st = fq_tq4_compress_store(key, value, dtype, rot_T_even, rot_T_odd, boundaries, kv_cache, slot_mapping,
