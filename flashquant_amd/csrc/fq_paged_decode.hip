@@ -960,6 +960,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     constexpr int kNewHeads = HPR;                          // KV heads of this workgroup
     uint4v new_raw[4];
     int64_t new_slot = -1;
+    float bnd_mine = 0.0f;      // boundary `lane` of the 15 (asked for here: at its use it would be a round trip of its own)
     if constexpr (STORE) {
         if (!copier) {
             const int kv_heads = MULTI > 0 ? HPR : p.H_KV;
@@ -969,6 +970,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
             for (int j = 0; j < 4; ++j) new_raw[j] = *reinterpret_cast<const uint4v*>(xrow + 32 * j + 8 * g);
             new_slot = p.new_slots[seq];
+            bnd_mine = p.boundaries[lane < 15 ? lane : 14];
         }
     }
     L = L < 0 ? 0 : L;
@@ -1260,7 +1262,6 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                     uint4v raw[KS];
 #pragma unroll
                     for (int j = 0; j < KS; ++j) raw[j] = new_raw[j];
-                    const float bnd_mine = p.boundaries[lane < 15 ? lane : 14];
                     float ss = 0.0f;         // sum of squares of row n: this lane's 32 elements, then over g
 #pragma unroll
                     for (int j = 0; j < KS; ++j) {
