@@ -699,10 +699,10 @@ template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, int MULTI = 0, bo
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     constexpr bool D64 = DIM == 64, D256 = DIM == 256;
     // MULTI: the kernel's rows are 2^MULTI consecutive tokens of 8 / 2^MULTI KV heads (1088 bytes whichever way).
-    // 1 (HALF): 4 KV heads, the sections of the two tokens interleaved by the copy plan into the layout of an
-    // 8-head row.  2, 3 (LINEAR): 2 KV heads or 1; the token rows go to LDS as they lie in the cache (their
-    // sections start at multiples of 8 and 4 bytes, not of the 16 of a copy chunk) and the computing wavefronts
-    // read their operands from where they are.
+    // 1 (HALF; in use at head_dim 64 with 8 KV heads): the sections of the two tokens interleaved by the copy plan
+    // into the layout of an 8-head row, one partial per token parity.  2, 3 (LINEAR): 2 KV heads or 1; the token rows
+    // go to LDS as they lie in the cache (their sections start at multiples of 8 and 4 bytes, not of the 16 of a copy
+    // chunk), the computing wavefronts read their operands from where they are and merge their partials at the end.
     // 4: rows of 2 tokens of 4 KV heads in the LINEAR form.
     constexpr bool HALF = MULTI == 1;
     constexpr bool LINEAR = MULTI >= 2;
@@ -2201,7 +2201,7 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
             return launch_staged_d64<DT>(ps, S, rows_per_page, wide_rows, d64_half, stream);
         }
     }
-    if (allow_half && staged_linear_applies(D, p.H_KV, BS, var)) {
+    if (staged_linear_applies(D, p.H_KV, BS, var)) {     // (one partial per split: also for callers that bring their own partial buffers)
         const int rows_per_page = BS * p.H_KV / 8;
         DecodeParams ps = p;
         ps.balance_slots = staged_balance_slots(S, p.num_splits);

@@ -540,6 +540,24 @@ def test_paged_decode_one_or_two_kv_heads_on_rows_of_tokens(hq, hkv, bs, splits,
     _decode_case(lens, hq=hq, hkv=hkv, bs=bs, num_splits=splits, seed=53, dtype=dtype)
 
 
+@pytest.mark.parametrize("hq,hkv,bs", [(8, 1, 16), (16, 2, 32), (16, 4, 16)])
+def test_paged_decode_few_kv_heads_through_the_partials_entry_point(hq, hkv, bs):
+    """The two-kernel form (partials into the caller's buffers, then the combine) on 1, 2 and 4 KV heads, query
+    rotated by the caller: the staged kernel on rows of tokens writes one partial per split there too."""
+    C = load_native()
+    c, b, r = book(128)
+    lens = [300, 17, 1000, 0, 9]
+    q, cache, table, sl = build_paged_case(lens, hq, hkv, bs=bs, seed=79)
+    want = O.split_k_paged_decode(q, cache, table, sl, c, c, r, hkv, 128, bs)
+    dev = [t.to(DEV) for t in (q, cache, table, sl, c, c, r)]
+    q_rot = (q.float() @ r.T).to(q.dtype).to(DEV)
+    for splits in (1, 4):
+        acc, m, l = C.paged_tq4_decode_partials(q_rot, dev[1], dev[2], dev[3], dev[4], dev[5], hkv, 128, bs, 1.0 / math.sqrt(128), splits)
+        assert acc.shape[-2] == splits
+        out = C.split_k_reduce(acc, m, l, dev[6], q.dtype)
+        assert (out.cpu().float() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item())
+
+
 def test_paged_decode_one_or_two_kv_heads_ragged_long_contexts():
     """More (sequence, split) workgroups than CUs with 1 and 2 KV heads: chunks sized from the actual
     lengths, counted in rows of 8 and 4 tokens."""
