@@ -73,11 +73,13 @@ def test_paged_decode_at_the_benchmark_size():
     assert rel <= 2e-2, f"max error {rel} of the row magnitude"
 
 
-def test_paged_decode_of_four_kv_heads_on_long_ragged_contexts():
-    """4 KV heads (rows of two tokens in the staged kernel) at contexts of thousands of tokens, odd and
-    even lengths, the library's own split count: against the oracle, and the direct kernel agrees."""
+@pytest.mark.parametrize("hq,hkv,bs", [(16, 4, 16), (16, 2, 32), (8, 1, 16)])
+def test_paged_decode_of_few_kv_heads_on_long_ragged_contexts(hq, hkv, bs):
+    """4, 2 and 1 KV heads (rows of 2, 4 and 8 tokens in the staged kernel) at contexts of thousands of tokens,
+    lengths that leave every kind of last row, the library's own split count: against the oracle, and the direct
+    kernel agrees."""
     c, b, r = book(128)
-    lens, hq, hkv, bs = [4096, 4095, 2049, 1, 3001, 0, 4033, 640], 16, 4, 16
+    lens = [4096, 4095, 2049, 1, 3001, 0, 4033, 640, 8193, 5003]
 
     def rows(s, n):
         return outlier_rows(n, hkv, 128, 6000 + 2 * s), outlier_rows(n, hkv, 128, 6001 + 2 * s)
@@ -194,12 +196,14 @@ def test_prod_paged_decode_on_long_ragged_contexts():
     assert math.isfinite(err) and err <= 2e-2, f"max abs error {err}"
 
 
-def test_serving_step_at_the_benchmark_size():
+@pytest.mark.parametrize("hq,hkv,L", [(32, 8, 4096), (8, 1, 4093), (8, 2, 4090)])
+def test_serving_step_at_the_benchmark_size(hq, hkv, L):
     """The benchmark's serving step: batch 32, 4096 tokens of context of which the last is the step's new token,
-    stored and attended over in one call (fq_tq4_store_and_decode).  The oracle stores its own compress of the
-    same rows and decodes; every sequence is compared."""
+    stored and attended over in one call (fq_tq4_store_and_decode); and the shards of that model over 8 and 4
+    GPUs (1 and 2 KV heads, the new token in the middle of a row of the kernel).  The oracle stores its own
+    compress of the same rows and decodes; every sequence is compared."""
     c, b, r = book(128)
-    B, L, hq, hkv, bs = 32, 4096, 32, 8, 16
+    B, bs = 32, 16
 
     def rows(s, n):
         return outlier_rows(n, hkv, 128, 6000 + 2 * s), outlier_rows(n, hkv, 128, 6001 + 2 * s)
