@@ -8,7 +8,10 @@
 //   out   = (softmax(...) V) @ R, rounded once (contiguous operands) or rounded before and after
 //           the rotation (paged operands, as the serving path rounds)
 //
-// A workgroup of 4 wavefronts owns 64 query rows of one query head, 16 per wavefront.  Per
+// A workgroup of 8 wavefronts owns 128 query rows that share their keys and values, 16 per wavefront:
+// 64 positions of two query heads of one KV head (an even number of query heads per KV head), else 128
+// positions of one query head.  One workgroup per CU: its byte -> centroid-pair tables are kept in 32
+// copies (one per bank, as in the decode kernels), and a tile is dequantised once for 128 rows.  Per
 // 32-token tile all threads dequantise K (row-major) and V (transposed) into LDS; a wavefront
 // then computes S = q K^T in the MFMA accumulator layout (lane = token column, registers = 4 query
 // rows), keeps the running maximum per row with row-wide DPP reductions, moves P through a
@@ -45,36 +48,44 @@ struct AnyDimCfg {
     static constexpr int VSTRIDE = 32 + 8;                // halves per V^T tile row
     static constexpr int K_BYTES = 32 * KSTRIDE * 2;
     static constexpr int V_BYTES = D * VSTRIDE * 2;
-    static constexpr int P_BYTES = 4 * 16 * VSTRIDE * 2;  // one 16 x 32 patch per wavefront
-    static constexpr int Q_BYTES = 4 * 16 * KSTRIDE * 2;  // rotated query rows, fp16
-    static constexpr int LOOP_BYTES = K_BYTES + V_BYTES + P_BYTES + Q_BYTES;
-    static constexpr int O_BYTES = 4 * 16 * (D + 4) * 4;  // float32 rows for the rotation back
-    static constexpr int LDS_BYTES = LOOP_BYTES > O_BYTES ? LOOP_BYTES : O_BYTES;
+    static constexpr int WAVES = 8;
+    static constexpr int P_BYTES = WAVES * 16 * VSTRIDE * 2;  // one 16 x 32 patch per wavefront
+    static constexpr int Q_BYTES = WAVES * 16 * KSTRIDE * 2;  // rotated query rows, fp16: before the loop, over the tiles
+    static constexpr int LOOP_BYTES = K_BYTES + V_BYTES + P_BYTES;
+    static constexpr int O_BYTES = 4 * 16 * (D + 4) * 4;  // float32 rows for the rotation back, four wavefronts at a time
+    static constexpr int LDS_BYTES = (LOOP_BYTES > O_BYTES ? LOOP_BYTES : O_BYTES) > Q_BYTES
+                                         ? (LOOP_BYTES > O_BYTES ? LOOP_BYTES : O_BYTES) : Q_BYTES;
+    static constexpr int COPIES = 32;                     // of each byte -> centroid-pair table
 };
 
 template <int D, int DT, bool PAGED>
-__global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyDimParams p) {
+__global__ __launch_bounds__(512) void tq_attention_any_dim_kernel(const AnyDimParams p) {
     using C = AnyDimCfg<D>;
     constexpr int NJ = D / 32;          // k-steps of the score product
     constexpr int NCB = D / 16;         // 16-coordinate output blocks
-    constexpr int BPT = D / 32;         // packed bytes per thread and token in the dequantisation (16 threads per token pair)
+    constexpr int BPT = D / 64;         // packed bytes per thread and token in the dequantisation (32 threads per token pair)
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     // byte -> (fp16 centroid[high nibble], fp16 centroid[low nibble]); for V the two nibbles of the byte
     // come from two consecutive tokens (see the dequantisation)
-    __shared__ uint32_t pair_k[256], pair_v[256];
+    // (entry b of copy c at word 32 b + c: a half-wave's lookups never share a bank)
+    __shared__ __attribute__((aligned(16))) uint32_t pair_k[256 * C::COPIES], pair_v[256 * C::COPIES];
     // A row whose norm lies above 2^15 is stored divided by 2^excess (its products with a centroid
     // then fit fp16); the power of two goes back in on the float32 score (K) or weight (V).
     __shared__ int k_exc[32], v_exc[32];
     _Float16* ks = reinterpret_cast<_Float16*>(smem);
     _Float16* vt = reinterpret_cast<_Float16*>(smem + C::K_BYTES);
     _Float16* ps = reinterpret_cast<_Float16*>(smem + C::K_BYTES + C::V_BYTES);
-    _Float16* qs = reinterpret_cast<_Float16*>(smem + C::K_BYTES + C::V_BYTES + C::P_BYTES);
+    _Float16* qs = reinterpret_cast<_Float16*>(smem);      // before the first tile is dequantised
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = tid >> 6;
+    const int wl = w & 3, wg = w >> 2;                // wavefront of its group of four, group
     const int n16 = lane & 15, g4 = lane >> 4;
-    const int hq = blockIdx.y, b = blockIdx.z;
+    const int copy = lane & 31;
+    // the two groups: two query heads of one KV head on the same 64 positions, or one head on 128 positions
+    const bool two_heads = (p.G & 1) == 0;
+    const int hq = two_heads ? 2 * int(blockIdx.y) + wg : int(blockIdx.y), b = blockIdx.z;
     const int hkv = hq / p.G;
 
     int NQ = p.N_Q, NKV = p.N_KV, qoff = 0;
@@ -89,15 +100,23 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
         q_row0 = int64_t(first) * p.H_Q + hq;
         q_stride = p.H_Q * D;
     }
-    const int pos_wg = 64 * blockIdx.x;
-    if (pos_wg >= NQ) return;                         // uniform: the grid is sized for the longest sequence
-    const int pos0 = pos_wg + 16 * w;                 // first row of this wavefront
+    // causal workgroups cost what their position is: the late (long) ones are handed out first, so that the short
+    // ones fill the end of the launch
+    const int pos_block = p.causal ? int(gridDim.x) - 1 - int(blockIdx.x) : int(blockIdx.x);
+    const int pos_first = (two_heads ? 64 : 128) * pos_block;            // of the workgroup
+    if (pos_first >= NQ) return;                      // uniform: the grid is sized for the longest sequence
+    const int pos_wg = two_heads ? pos_first : pos_first + 64 * wg;       // of this group (may lie beyond the sequence:
+                                                                          // its rows are then computed and not stored)
+    const int pos0 = pos_wg + 16 * wl;                // first row of this wavefront
 
-    {
-        const half2v ck = {_Float16(p.centroids_k[tid >> 4]), _Float16(p.centroids_k[tid & 15])};
-        const half2v cv = {_Float16(p.centroids_v[tid >> 4]), _Float16(p.centroids_v[tid & 15])};
-        pair_k[tid] = __builtin_bit_cast(uint32_t, ck);
-        pair_v[tid] = __builtin_bit_cast(uint32_t, cv);
+    {   // threads 0..255 fill the key table, 256..511 the value table: entry tid % 256, all its copies
+        const int e = tid & 255;
+        const float* cen = tid < 256 ? p.centroids_k : p.centroids_v;
+        const half2v c2 = {_Float16(cen[e >> 4]), _Float16(cen[e & 15])};
+        const uint32_t bits = __builtin_bit_cast(uint32_t, c2);
+        uint32_t* row = (tid < 256 ? pair_k : pair_v) + e * C::COPIES;
+#pragma unroll
+        for (int k = 0; k < C::COPIES; k += 4) *reinterpret_cast<uint4v*>(row + k) = uint4v{bits, bits, bits, bits};
     }
 
     // ---- rotate the 16 query rows of this wavefront, round to the query dtype, stage as fp16 ------
@@ -106,18 +125,24 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
         int pos = pos0 + n16;
         pos = pos < NQ ? pos : NQ - 1;
         const uint16_t* src = p.q + (q_row0 * D) + int64_t(pos) * q_stride;
-        float a[NJ][8];
+        // The 16-bit rows are exact in fp16 after one power of two for the block, the matrix block goes in as two
+        // fp16 terms: exact products on the fp16 MFMA, at 8 times the rate of the float32 one (at head_dim 256 the
+        // two rotations of a workgroup on the float32 MFMA took as long as 100 tiles of the loop).
+        uint4v raw[NJ];
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int k = 0; k < 8; ++k) a[j][k] = load_elem<DT>(src[32 * j + 8 * g4 + k]);
+        for (int j = 0; j < NJ; ++j) raw[j] = *reinterpret_cast<const uint4v*>(src + 32 * j + 8 * g4);
+        half8 ah[NJ];
+        float up_rows;
+        rows_as_f16<D, DT>(raw, ah, up_rows);
         float qr[NCB][4];
         float mx = 0.0f;
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
             float rb[NJ][8];
             load_rotation_any<D>(p.rotation, p.rot_col_major != 0, true, 16 * cb, n16, g4, rb);
-            const float4v acc = rotate_block<D>(a, rb);
+            half8 rhi[NJ], rlo[NJ];
+            split_rotation_block<D>(rb, rhi, rlo);
+            const float4v acc = rotate_block_f16<D>(ah, rhi, rlo) * up_rows;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 qr[cb][i] = load_elem<DT>(store_elem<DT>(acc[i]));
@@ -142,12 +167,14 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
     for (int j = 0; j < NJ; ++j)
         qa[j] = *reinterpret_cast<const half8*>(qs + (w * 16 + n16) * C::KSTRIDE + 32 * j + 8 * g4);
     const float qscale = p.scale_log2e * up;
+    __syncthreads();                                   // the query rows lie where the tiles go
 
     // ---- tiles --------------------------------------------------------------------------------------
     const int all_tiles = (NKV + 31) >> 5;
     int ntiles = all_tiles;
     if (p.causal) {
-        int last_pos = pos_wg + 63 < NQ - 1 ? pos_wg + 63 : NQ - 1;
+        const int span = two_heads ? 63 : 127;         // uniform over the workgroup: every wavefront meets every barrier
+        int last_pos = pos_first + span < NQ - 1 ? pos_first + span : NQ - 1;
         const int t = ((qoff + last_pos) >> 5) + 1;
         ntiles = t < all_tiles ? t : all_tiles;
     }
@@ -158,14 +185,14 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
 #pragma unroll
     for (int i = 0; i < 4; ++i) { m_run[i] = -__builtin_inff(); l_run[i] = 0.0f; }
 
-    const int tp = tid >> 4, part = tid & 15;         // dequantisation: token pair of the tile, sixteenth of its rows
+    const int tp = tid >> 5, part = tid & 31;         // dequantisation: token pair of the tile, 1 / 32 of its rows
     const int64_t k_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.k_cap;
     const int64_t v_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.v_cap;
     _Float16* pw = ps + w * 16 * C::VSTRIDE;
 
     // The packed bytes and norms of a tile are asked for one tile ahead (into registers), so that the
     // memory latency runs under the products of the tile before.
-    uint32_t kw[2][2] = {{0u, 0u}, {0u, 0u}}, vw[2][2] = {{0u, 0u}, {0u, 0u}};
+    uint32_t kw[2][1] = {{0u}, {0u}}, vw[2][1] = {{0u}, {0u}};
     float nk[2] = {0.0f, 0.0f}, nv[2] = {0.0f, 0.0f};
     auto load_tile = [&](int tile) {
         const int t0 = tile * 32;
@@ -191,16 +218,16 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
                 nv[u] = p.v_norms[v_row0 + tok];
             }
             if (!live) { nk[u] = 0.0f; nv[u] = 0.0f; }
-            // packed bytes part * BPT .. of the token (BPT = 2, 4 or 8)
-            if (BPT == 2) {
+            // packed bytes part * BPT .. of the token (BPT = 1, 2 or 4)
+            if (BPT == 1) {
+                kw[u][0] = kp[u][part];
+                vw[u][0] = vp[u][part];
+            } else if (BPT == 2) {
                 kw[u][0] = *reinterpret_cast<const uint16_t*>(kp[u] + 2 * part);
                 vw[u][0] = *reinterpret_cast<const uint16_t*>(vp[u] + 2 * part);
             } else {
-#pragma unroll
-                for (int c = 0; c < BPT / 4; ++c) {
-                    kw[u][c] = *reinterpret_cast<const uint32_t*>(kp[u] + BPT * part + 4 * c);
-                    vw[u][c] = *reinterpret_cast<const uint32_t*>(vp[u] + BPT * part + 4 * c);
-                }
+                kw[u][0] = *reinterpret_cast<const uint32_t*>(kp[u] + 4 * part);
+                vw[u][0] = *reinterpret_cast<const uint32_t*>(vp[u] + 4 * part);
             }
         }
     };
@@ -228,16 +255,17 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
 #pragma unroll
                 for (int j = 0; j < BPT; ++j) {
                     const uint32_t byte = (kw[u][j >> 2] >> (8 * (j & 3))) & 0xffu;
-                    const half2v c2 = __builtin_bit_cast(half2v, pair_k[byte]) * n2;
+                    const half2v c2 = __builtin_bit_cast(half2v, pair_k[byte * C::COPIES + copy]) * n2;
                     wd[j] = __builtin_bit_cast(uint32_t, c2);
                 }
                 // the thread's run of the row in 8- or 16-byte stores (single dwords from 64 lanes that lie 16
                 // to 32 bytes apart fall into a few banks)
-                if constexpr (BPT == 2) {
+                if constexpr (BPT == 1) {
+                    *dst = wd[0];
+                } else if constexpr (BPT == 2) {
                     *reinterpret_cast<uint2v*>(dst) = uint2v{wd[0], wd[1]};
                 } else {
-#pragma unroll
-                    for (int j = 0; j < BPT; j += 4) *reinterpret_cast<uint4v*>(dst + j) = uint4v{wd[j], wd[j + 1], wd[j + 2], wd[j + 3]};
+                    *reinterpret_cast<uint4v*>(dst) = uint4v{wd[0], wd[1 % BPT], wd[2 % BPT], wd[3 % BPT]};
                 }
             }
             // V, transposed: a 2 x 2 nibble transpose makes a byte hold one coordinate of the two tokens,
@@ -256,8 +284,8 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
 #pragma unroll
                     for (int j = 0; j < (BPT < 4 ? BPT : 4); ++j) {
                         const int d = 2 * (BPT * part + 4 * c + j);
-                        const half2v xe = __builtin_bit_cast(half2v, pair_v[(X >> (8 * j)) & 0xffu]) * n2;
-                        const half2v yo = __builtin_bit_cast(half2v, pair_v[(Y >> (8 * j)) & 0xffu]) * n2;
+                        const half2v xe = __builtin_bit_cast(half2v, pair_v[((X >> (8 * j)) & 0xffu) * C::COPIES + copy]) * n2;
+                        const half2v yo = __builtin_bit_cast(half2v, pair_v[((Y >> (8 * j)) & 0xffu) * C::COPIES + copy]) * n2;
                         *reinterpret_cast<uint32_t*>(vt + d * C::VSTRIDE + 2 * vcol) = __builtin_bit_cast(uint32_t, xe);
                         *reinterpret_cast<uint32_t*>(vt + (d + 1) * C::VSTRIDE + 2 * vcol) = __builtin_bit_cast(uint32_t, yo);
                     }
@@ -336,31 +364,45 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
     }
 
     // ---- normalise, rotate back, store ------------------------------------------------------------------
-    __syncthreads();                                   // the staging rows overlay the tiles and the query rows
-    float* os = reinterpret_cast<float*>(smem) + w * 16 * (D + 4);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float l = row16_sum(l_run[i]);
-        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-#pragma unroll
-        for (int cb = 0; cb < NCB; ++cb) {
-            float v = O[cb][i] * inv;
-            if (PAGED) v = load_elem<DT>(store_elem<DT>(v));
-            os[(4 * g4 + i) * (D + 4) + 16 * cb + n16] = v;
-        }
-    }
-    __syncthreads();
+    // The staging rows overlay the tiles, a patch per wavefront that only its own lanes write and read; the two
+    // groups of four wavefronts take the patches one after the other.
+    float* os = reinterpret_cast<float*>(smem) + wl * 16 * (D + 4);
     float a[NJ][8];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
+    for (int round = 0; round < 2; ++round) {
+        __syncthreads();                               // the tiles (round 0), the other group's patches (round 1) are free
+        if (wg == round) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) a[j][k] = os[n16 * (D + 4) + 32 * j + 8 * g4 + k];
+            for (int i = 0; i < 4; ++i) {
+                const float l = row16_sum(l_run[i]);
+                const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    float v = O[cb][i] * inv;
+                    if (PAGED) v = load_elem<DT>(store_elem<DT>(v));
+                    os[(4 * g4 + i) * (D + 4) + 16 * cb + n16] = v;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) a[j][k] = os[n16 * (D + 4) + 32 * j + 8 * g4 + k];
+        }
+    }
     uint16_t* obase = p.out + q_row0 * D;
+    // float32 rows as two fp16 terms (rows already rounded to the output type, the paged form: exact in one)
+    half8 ohi[NJ], olo[NJ];
+    float up_out;
+    rows_split_f16<D>(a, ohi, olo, up_out);
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
         float rb[NJ][8];
         load_rotation_any<D>(p.rotation, p.rot_col_major != 0, false, 16 * cb, n16, g4, rb);
-        const float4v acc = rotate_block<D>(a, rb);
+        half8 rhi[NJ], rlo[NJ];
+        split_rotation_block<D>(rb, rhi, rlo);
+        const float4v acc = (PAGED ? rotate_block_f16<D>(ohi, rhi, rlo) : rotate_block_f16x3<D>(ohi, olo, rhi, rlo)) * up_out;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int pos = pos0 + 4 * g4 + i;
@@ -371,7 +413,8 @@ __global__ __launch_bounds__(256, 2) void tq_attention_any_dim_kernel(const AnyD
 
 template <int D, bool PAGED>
 int launch_any_dim(const AnyDimParams& p, int max_q, int batch, int dtype, hipStream_t s) {
-    const dim3 grid((max_q + 63) / 64, p.H_Q, batch), block(256);
+    const bool two_heads = (p.G & 1) == 0;            // as the kernel decides
+    const dim3 grid(two_heads ? (max_q + 63) / 64 : (max_q + 127) / 128, two_heads ? p.H_Q / 2 : p.H_Q, batch), block(512);
     const size_t lds = AnyDimCfg<D>::LDS_BYTES;
     if (dtype == FQ_F16) {
         auto kern = tq_attention_any_dim_kernel<D, FQ_F16, PAGED>;
