@@ -1024,13 +1024,14 @@ def test_store_and_decode_equals_store_then_decode(hq, hkv, d, bs, dtype, kernel
         _check_serving_step(lens, hq, hkv, d, bs, dtype, splits, seed=300 + ci)
 
 
-def test_store_and_decode_in_a_captured_graph():
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 1), (16, 4)])
+def test_store_and_decode_in_a_captured_graph(hq, hkv):
     """The serving step recorded into a graph (caller workspace and output, nothing allocated) and replayed with
     new keys, values and queries in the recorded tensors, the program's own eager work in between: every replay
     must give what the eager call gives on the same inputs."""
     C = load_native()
     c, b, r = book(128)
-    hq, hkv, d, bs = 32, 8, 128, 16
+    d, bs = 128, 16
     lens = [100, 17, 1, 2500]
     q, cache, table, sl, key, value, slots = _serving_case(lens, hq, hkv, d, bs, torch.bfloat16, seed=501)
     ev, od = O.split_rotation(r)
