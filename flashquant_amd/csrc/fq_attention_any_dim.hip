@@ -185,7 +185,9 @@ __global__ __launch_bounds__(512) void tq_attention_any_dim_kernel(const AnyDimP
 #pragma unroll
     for (int i = 0; i < 4; ++i) { m_run[i] = -__builtin_inff(); l_run[i] = 0.0f; }
 
-    const int tp = tid >> 5, part = tid & 31;         // dequantisation: token pair of the tile, 1 / 32 of its rows
+    // dequantisation: token pair of the tile, 1 / 32 of its coordinates.  A wavefront takes 4 token pairs x 16 parts,
+    // so that its transposed V stores (below) reach all banks
+    const int tp = (lane >> 4) + 4 * (w >> 1), part = (lane & 15) + 16 * (w & 1);
     const int64_t k_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.k_cap;
     const int64_t v_row0 = PAGED ? 0 : (int64_t(b) * p.H_KV + hkv) * p.v_cap;
     _Float16* pw = ps + w * 16 * C::VSTRIDE;
@@ -272,17 +274,20 @@ __global__ __launch_bounds__(512) void tq_attention_any_dim_kernel(const AnyDimP
             // so one lookup yields the dword (token 2 tp, token 2 tp + 1) of a coordinate row
             {
                 const half2v n2 = {_Float16(nv[0]), _Float16(nv[1])};
-                // The rows of the 16 threads of a token pair lie 2 BPT rows apart, a multiple of 64 banks at 256
+                // The rows of the threads of a token pair lie 2 BPT rows apart, a multiple of 32 banks at 256
                 // coordinates: with the pair's own column every one of their stores would hit the same bank.
                 // The groups of four columns (8 tokens, what an operand read takes) are rotated by the thread's
-                // index, so that the 64 lanes of a store spread over 16 banks (the 16 columns of a row).
+                // part, and the parts walk through their coordinates in rotated order (a row further is 8 banks
+                // further): the 64 lanes of a store (4 token pairs x 16 parts) fall two to a bank, the minimum.
                 const int vcol = (tp + 4 * part) & 15;
+                constexpr int JN = BPT < 4 ? BPT : 4;
 #pragma unroll
                 for (int c = 0; c < (BPT + 3) / 4; ++c) {
                     const uint32_t X = (vw[0][c] & 0xF0F0F0F0u) | ((vw[1][c] >> 4) & 0x0F0F0F0Fu);   // even coordinates
                     const uint32_t Y = ((vw[0][c] << 4) & 0xF0F0F0F0u) | (vw[1][c] & 0x0F0F0F0Fu);   // odd coordinates
 #pragma unroll
-                    for (int j = 0; j < (BPT < 4 ? BPT : 4); ++j) {
+                    for (int j0 = 0; j0 < JN; ++j0) {
+                        const int j = (j0 + (part >> 2)) & (JN - 1);
                         const int d = 2 * (BPT * part + 4 * c + j);
                         const half2v xe = __builtin_bit_cast(half2v, pair_v[((X >> (8 * j)) & 0xffu) * C::COPIES + copy]) * n2;
                         const half2v yo = __builtin_bit_cast(half2v, pair_v[((Y >> (8 * j)) & 0xffu) * C::COPIES + copy]) * n2;
