@@ -2373,7 +2373,12 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     // (4 KV heads run as 8: the staged kernel reads their tokens in pairs; 1 and 2 of dimension 128 likewise, in
     // rows of 8 and 4 tokens; `rows_of_tokens`: the forms that count their chunks in such rows)
     const bool rows_of_tokens = D == 128 && (H_KV == 1 || H_KV == 2 || H_KV == 4) && block_size >= 16;
-    const int64_t heads = (H_KV == 4 || rows_of_tokens) ? 8 : H_KV;
+    int64_t heads = (H_KV == 4 || rows_of_tokens) ? 8 : H_KV;
+    // (a workgroup of the staged kernel has 8 wavefronts whatever they serve: a KV head of 256 coordinates takes two
+    // of them, a pair of KV heads of 64 coordinates one; measured on 32 x 4096 tokens: head_dim 256 with 8 KV heads
+    // 87 us at 8 splits, 82 at 4; head_dim 64 with 16 KV heads 54 us at 4 splits, 37 at 8)
+    if (D == 256 && H_KV % 4 == 0) heads = 2 * int64_t(H_KV);
+    if (D == 64 && H_KV % 16 == 0) heads = H_KV / 2;
     const int64_t one_round = (target_waves + int64_t(num_seqs) * heads - 1) / (int64_t(num_seqs) * heads);
     // ... and twice that when the contexts are long enough for splits of 1024 tokens: the lengths
     // of the sequences are not known here, a ragged batch leaves many splits empty, and the
