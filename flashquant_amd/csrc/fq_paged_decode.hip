@@ -2387,10 +2387,10 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     const int64_t long_chunks = rows_of_tokens ? max_ctx * H_KV / 8192 : max_ctx / 1024;
     int64_t ns = 2 * one_round < long_chunks ? 2 * one_round : long_chunks;
     if (ns < one_round) ns = one_round;
-    // Fewer than 8 KV heads run the direct kernel, whose workgroups are as small as the head count: a
+    // Where fewer than 8 KV heads run the direct kernel, its workgroups are as small as the head count: a
     // round over the chip would cut a short context into chunks that cost more to launch and combine
     // than to read (measured on 32 x 4096 tokens: 1 KV head 85 us at 64 splits, 37 us at 16).
-    if (H_KV < 8 && ns > max_ctx / 256) ns = max_ctx / 256;
+    if (H_KV < 8 && !rows_of_tokens && ns > max_ctx / 256) ns = max_ctx / 256;
     // (a chunk is at least 64 rows)
     if (rows_of_tokens && ns > max_ctx * H_KV / 512) ns = max_ctx * H_KV / 512;
     if (ns > tiles) ns = tiles;
