@@ -2390,7 +2390,10 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     // Where fewer than 8 KV heads run the direct kernel, its workgroups are as small as the head count: a
     // round over the chip would cut a short context into chunks that cost more to launch and combine
     // than to read (measured on 32 x 4096 tokens: 1 KV head 85 us at 64 splits, 37 us at 16).
-    if (H_KV < 8 && !rows_of_tokens && ns > max_ctx / 256) ns = max_ctx / 256;
+    const bool staged_form = rows_of_tokens || (D == 256 && H_KV % 4 == 0) || (D == 64 && H_KV == 8 && block_size >= 16);
+    if (H_KV < 8 && !staged_form && ns > max_ctx / 256) ns = max_ctx / 256;
+    // (8 KV heads of dimension 64 write two partials per split: 128 of them at most, as below)
+    if (D == 64 && H_KV == 8 && block_size >= 16 && ns > 64) ns = 64;
     // (a chunk is at least 64 rows)
     if (rows_of_tokens && ns > max_ctx * H_KV / 512) ns = max_ctx * H_KV / 512;
     if (ns > tiles) ns = tiles;
