@@ -635,11 +635,7 @@ __device__ unsigned int g_decode_faults = 0u;
 // Byte offset, inside a page of `H` KV heads, of chunk `cc` of the 8-head rows that head group `hgrp`
 // (heads 8 hgrp .. 8 hgrp + 7) sees: the group's slices of the four sections of a token row laid end
 // to end, kChunksPerRow chunks per token.  With 8 heads the slices are the row itself (16 cc).
-//
-// HALF (4 KV heads): the kernel works on rows of 8 "heads" made of two consecutive tokens, head h of
-// the even token as head h and of the odd token as head 4 + h, so row r is the real rows 2 r and
-// 2 r + 1 (544 bytes each) with their sections interleaved; a page then holds half as many rows.
-template <bool PROD, bool HALF, int DIM = 128>
+template <bool PROD, int DIM = 128>
 __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     constexpr int CPR = StagedCfg<PROD, DIM>::CHUNKS_PER_ROW;
     const int r = cc / CPR, ci = cc - r * CPR;
@@ -655,14 +651,6 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
     }
     if constexpr (DIM == 64) {
         // head_dim 64, H real heads: [K idx H*32 | K norms H*4 | V idx H*32 | V norms H*4] = 72 H bytes a token
-        if constexpr (HALF) {      // 8 real heads: a row is two tokens of 576 bytes
-            int tok, off;
-            if (ci < 32) { tok = ci >> 4; off = 16 * (ci & 15); }                            // K indices, 256 bytes per token
-            else if (ci < 36) { tok = (ci - 32) >> 1; off = 256 + 16 * ((ci - 32) & 1); }    // K norms, 32 bytes
-            else if (ci < 68) { tok = (ci - 36) >> 4; off = 288 + 16 * ((ci - 36) & 15); }   // V indices
-            else { tok = (ci - 68) >> 1; off = 544 + 16 * ((ci - 68) & 1); }                 // V norms
-            return uint32_t((2 * r + tok) * 576 + off);
-        }
         int off;                   // group hgrp of 16 real heads
         if (ci < 32) off = 512 * hgrp + 16 * ci;
         else if (ci < 36) off = H * 32 + 64 * hgrp + 16 * (ci - 32);
@@ -679,14 +667,6 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
         else off = H * 136 + 32 * hgrp + 16 * (ci - 68);
         return uint32_t(r * (H * 140) + off);
     }
-    if constexpr (HALF) {
-        int tok, off;                                      // which of the two tokens, offset in its 544-byte row
-        if (ci < 32) { tok = ci >> 4; off = 16 * (ci & 15); }                      // K indices, 256 bytes per token
-        else if (ci < 34) { tok = ci - 32; off = 256; }                            // K norms, 16 bytes
-        else if (ci < 66) { tok = (ci - 34) >> 4; off = 272 + 16 * ((ci - 34) & 15); }   // V indices
-        else { tok = ci - 66; off = 528; }                                         // V norms
-        return uint32_t((2 * r + tok) * 544 + off);
-    }
     int off;
     if (ci < 32) off = 512 * hgrp + 16 * ci;                               // K indices
     else if (ci < 34) off = H * 64 + 32 * hgrp + 16 * (ci - 32);           // K norms
@@ -698,22 +678,19 @@ __device__ __forceinline__ uint32_t staged_src_offset(int cc, int H, int hgrp) {
 template <int BSL, int GP, int DT, int PVR, bool PROD, int CW, int MULTI = 0, bool STORE = false, int DIM = 128>
 __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(const DecodeParams p) {
     constexpr bool D64 = DIM == 64, D256 = DIM == 256;
-    // MULTI: the kernel's rows are 2^MULTI consecutive tokens of 8 / 2^MULTI KV heads (1088 bytes whichever way).
-    // 1 (HALF; in use at head_dim 64 with 8 KV heads): the sections of the two tokens interleaved by the copy plan
-    // into the layout of an 8-head row, one partial per token parity.  2, 3 (LINEAR): 2 KV heads or 1; the token rows
-    // go to LDS as they lie in the cache (their sections start at multiples of 8 and 4 bytes, not of the 16 of a copy
-    // chunk), the computing wavefronts read their operands from where they are and merge their partials at the end.
-    // 4: rows of 2 tokens of 4 KV heads in the LINEAR form.
-    constexpr bool HALF = MULTI == 1;
+    // MULTI (0, 2, 3, 4): the kernel's rows are 1, 4, 8 or 2 consecutive tokens of 8, 2, 1 or 4 KV heads of dimension
+    // 128 (1088 bytes whichever way), or, at head_dim 64, of as many pairs of heads.  Rows of several tokens (LINEAR)
+    // go to LDS as they lie in the cache (with 1 and 2 heads their sections start at multiples of 4 and 8 bytes, not of
+    // the 16 of a copy chunk), the computing wavefronts read their operands from where they are and merge their
+    // partials at the end.
     constexpr bool LINEAR = MULTI >= 2;
     constexpr int TPR = MULTI == 4 ? 2 : 1 << MULTI;     // tokens per row
     constexpr int HPR = 8 / TPR;             // real KV heads per row
-    static_assert(MULTI >= 0 && MULTI <= 4, "rows of 1, 2, 4 or 8 tokens");
-    static_assert(!LINEAR || (DIM == 128 && !PROD && CW > 0), "rows of 4 and 8 tokens: TQ4, head_dim 128, copy wavefronts");
-    static_assert(!(HALF && PROD), "two-token rows are a TQ4 form");
+    static_assert(MULTI == 0 || (MULTI >= 2 && MULTI <= 4), "rows of 1, 2, 4 or 8 tokens");
+    static_assert(!LINEAR || (!PROD && CW > 0 && (DIM == 128 || (DIM == 64 && MULTI == 4))),
+                  "rows of several tokens as they lie in the cache: TQ4, copy wavefronts, head_dim 128 or (rows of 2 tokens) 64");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
     static_assert(DIM == 128 || (!PROD && !STORE && CW > 0), "head_dim 64 / 256 are served by the TQ4 form with copy wavefronts");
-    static_assert(!(D256 && HALF), "head_dim 256 comes in groups of 4 KV heads");
     // D256: the kernel's "heads" are the halves of real heads of 256 coordinates (wavefront h: real head h / 2 of the
     // group of 4, coordinates 128 (h % 2) ...): the two wavefronts of a head exchange their halves of the scores
     // through LDS every tile and add them, compute the same weights, and each accumulates its half of the output
@@ -725,7 +702,11 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     using Cfg = StagedCfg<PROD, DIM>;
     // LINEAR: a row of 1088 bytes every 1104 in LDS, so that the rows of a block start in eight different
     // 16-byte columns of the banks (at 1088 they would start in two)
-    constexpr int kRowLds = 1104;
+    constexpr int kRowLds = 16 * Cfg::CHUNKS_PER_ROW + 16;    // 1104; head_dim 64: 1168
+    // LINEAR: bytes of a token in such a row, and of its key (or value) norms; HPR counts heads of 128 coordinates,
+    // at head_dim 64 pairs of real heads
+    constexpr int kTokenBytes = (D64 ? 144 : 136) * HPR;
+    constexpr int kTokenNormBytes = (D64 ? 8 : 4) * HPR;
     constexpr int kStageBytes = LINEAR ? 16 * kRowLds : Cfg::STAGE_BYTES;
     constexpr int kTileBytes = 2 * kStageBytes;
     constexpr int kChunksPerRow = Cfg::CHUNKS_PER_ROW;
@@ -772,7 +753,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     const int hgrp = blockIdx.z;
     const int HQG = (D256 ? 4 : HPR) * p.G;              // query heads of a group
     const int hq0 = hgrp * HQG;
-    const int row_bytes = D64 ? (HALF ? 1152 : p.H_KV * 72)
+    const int row_bytes = D64 ? (MULTI > 0 ? 1152 : p.H_KV * 72)
                         : D256 ? p.H_KV * 264
                                : (MULTI > 0 ? 1088 : p.H_KV * (PROD ? 140 : 136));   // a row of the cache as the kernel sees it
     const int qsub = D64 && (n % GP) >= p.G / 2 ? 1 : 0;    // D64: this lane's query head belongs to the pair's second head
@@ -841,7 +822,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         for (int i = 1; i < PPT; ++i) pg += c >= i * PC ? 1 : 0;
         src_page[k] = pg;
         const int sub = (kSpreadTail && k == 4) ? 4 * (tid & 3) : 0;
-        src_off[k] = staged_src_offset<PROD, HALF, DIM>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+        src_off[k] = staged_src_offset<PROD, DIM>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
         dst_off[k] = kChunkDst<PROD, DIM>.off[c] + sub;
     }
     const bool has_round4 = kSpreadTail || tid < kChunksPerTile - 4 * 512;   // else whole wavefronts
@@ -852,10 +833,11 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     for (int b = 0; b < 2; ++b) {
         if constexpr (LINEAR) {
             // the token rows as they lie in the cache: token tsel of the row, head hr of its HPR heads
-            const int token = 136 * HPR * tsel;
+            const int token = kTokenBytes * tsel;
             k_rd[b] = b * kStageBytes + kRowLds * n + token + 64 * hr + 16 * g;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v_rd[b][i] = b * kStageBytes + kRowLds * (4 * g + i) + token + 68 * HPR + 64 * hr + 4 * n;
+            for (int i = 0; i < 4; ++i)
+                v_rd[b][i] = b * kStageBytes + kRowLds * (4 * g + i) + token + 64 * HPR + kTokenNormBytes + 64 * hr + 4 * n;
         } else {
             k_rd[b] = b * kStageBytes + 16 * staged_slot(h, n, g);
 #pragma unroll
@@ -873,9 +855,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         else if (GP == 8) { blk = cls; row = 4 * g + e; }
         else { blk = e >> 2; row = 4 * g + (e & 3); }
         sc_tok[e] = 16 * blk + row;
-        n_rd[e] = D64 ? blk * kStageBytes + Cfg::KN_OFF + 64 * row + 8 * h + 4 * qsub
+        n_rd[e] = LINEAR ? blk * kStageBytes + kRowLds * row + kTokenBytes * tsel + 64 * HPR + (D64 ? 8 * hr + 4 * qsub : 4 * hr)
+                : D64 ? blk * kStageBytes + Cfg::KN_OFF + 64 * row + 8 * h + 4 * qsub
                 : D256 ? blk * kStageBytes + Cfg::KN_OFF + 16 * row + 4 * (h >> 1)
-                : LINEAR ? blk * kStageBytes + kRowLds * row + 136 * HPR * tsel + 64 * HPR + 4 * hr
                        : blk * kStageBytes + kStageKnOff + 32 * row + 4 * h;
     }
 
@@ -982,10 +964,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     const int end = L < begin + chunk ? L : begin + chunk;
     const int end_mine = rows_mine < end ? rows_mine : end;      // rows < end_mine hold a token of this wavefront
     const int hq_lane = hr * p.G + n;
-    // MULTI > 0: the TPR tokens of a row are as many partials of a head, TPR split + token of TPR NS
-    // (LINEAR: merged inside the workgroup into the one partial of the split)
-    const int NS_out = LINEAR ? NS : TPR * NS;
-    const int split_out = LINEAR ? split : TPR * split + tsel;
+    // (rows of several tokens: the wavefronts of a head merge their partials into the one of the split)
+    const int NS_out = NS;
+    const int split_out = split;
     if (begin >= end) {   // uniform over the workgroup
         if (g == 0 && n < p.G && !copier && (!D256 || (h & 1) == 0) && (!LINEAR || tsel == 0)) {
             const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hq_lane) * NS_out + split_out;
@@ -1087,7 +1068,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                     c_src[k] = 16u * uint32_t(c - pg * PC) + uint32_t(sub);
                     c_dst[k] = kRowLds * (c / kChunksPerRow) + 16 * (c % kChunksPerRow) + sub;
                 } else {
-                    c_src[k] = staged_src_offset<PROD, HALF, DIM>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
+                    c_src[k] = staged_src_offset<PROD, DIM>(c - pg * PC, p.H_KV, hgrp) + uint32_t(sub);
                     c_dst[k] = kChunkDst<PROD, DIM>.off[c] + sub;
                 }
             }
@@ -1425,7 +1406,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
 #pragma unroll
         for (int e = 0; e < NSC; ++e) {
             kn[e] = *reinterpret_cast<const float*>(tile + n_rd[e]);
-            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (LINEAR ? 68 * HPR : DIM != 128 ? Cfg::VN_OFF - Cfg::KN_OFF : kStageVnOff - kStageKnOff));
+            vn[e] = *reinterpret_cast<const float*>(tile + n_rd[e] + (LINEAR ? 64 * HPR + kTokenNormBytes : DIM != 128 ? Cfg::VN_OFF - Cfg::KN_OFF : kStageVnOff - kStageKnOff));
             kg[e] = PROD ? *reinterpret_cast<const float*>(tile + n_rd[e] + (kStageKgOff - kStageKnOff)) : 0.0f;
         }
         // These were all the reads of the slot (the lookups below go to the table): it is handed back
@@ -1720,7 +1701,12 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(m - ms);
                 acc += w * xacc[((t * HPR + hr) * 16 + head) * 128 + c];
             }
-            p.part_acc[((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS + split) * D + c] = acc;
+            if constexpr (D64) {     // a query head's output: the half of the 128 coordinates that is its own head's
+                if ((c >> 6) == (head >= p.G / 2 ? 1 : 0))
+                    p.part_acc[((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS + split) * 64 + (c & 63)] = acc;
+            } else {
+                p.part_acc[((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS + split) * D + c] = acc;
+            }
         }
         if (tsel == 0 && lane < p.G) {
             const float ms = merged_max(lane);
@@ -2106,14 +2092,6 @@ int launch_staged_linear(const DecodeParams& p, int S, int rows_per_page, hipStr
 #undef FQ_LINEAR_GP
 }
 
-// Partials per split that the staged kernel writes for this shape when the switches let it run (the tokens of its
-// rows): what workspaces are sized for, whatever the switches say.
-inline int partials_per_split_room(int D, int H_KV, int block_size) {
-    if (block_size < 16) return 1;
-    if (D == 64 && H_KV == 8) return 2;
-    return 1;
-}
-
 // head_dim 64 on the staged kernel: pairs of neighbouring KV heads as heads of 128 (16 real heads a group), or, with
 // 8 KV heads on pages of 16 or 32 tokens, rows of two tokens of four such pairs.  Up to 8 query heads per KV head.
 inline bool staged_d64_full_applies(int D, int H_KV, int G, const DecodeVariant& v) {
@@ -2124,24 +2102,25 @@ inline bool staged_d64_half_applies(int D, int H_KV, int G, int block_size, cons
 }
 template <int DT>
 int launch_staged_d64(const DecodeParams& p, int S, int rows_per_page, bool wide, bool half, hipStream_t stream) {
-    const size_t lds = 2 * size_t(StagedCfg<false, 64>::TILE_BYTES);
+    // (rows of two tokens: as they lie in the cache, a row every 1168 bytes)
+    const size_t lds = half ? 2 * 32 * 1168 : 2 * size_t(StagedCfg<false, 64>::TILE_BYTES);
     const dim3 grid(S, p.num_splits, half ? 1 : p.H_KV / 16), block(512 + 64 * 4);
-#define FQ_D64_GP(BSL, GPV, HALFV)                                                                                \
-    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, HALFV, false, 64>, p, grid, block, lds, stream) \
-                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, HALFV, false, 64>, p, grid, block, lds, stream)
-#define FQ_D64_BS(BSL, HALFV)                            \
+#define FQ_D64_GP(BSL, GPV, MULTIV)                                                                                \
+    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, MULTIV, false, 64>, p, grid, block, lds, stream) \
+                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, MULTIV, false, 64>, p, grid, block, lds, stream)
+#define FQ_D64_BS(BSL, MULTIV)                            \
     do {                                                 \
-        if (p.G <= 4) { FQ_D64_GP(BSL, 4, HALFV); }      \
-        else if (p.G <= 8) { FQ_D64_GP(BSL, 8, HALFV); } \
-        else { FQ_D64_GP(BSL, 16, HALFV); }              \
+        if (p.G <= 4) { FQ_D64_GP(BSL, 4, MULTIV); }      \
+        else if (p.G <= 8) { FQ_D64_GP(BSL, 8, MULTIV); } \
+        else { FQ_D64_GP(BSL, 16, MULTIV); }              \
     } while (0)
     if (half) {
-        if (rows_per_page == 8) FQ_D64_BS(3, true);
-        else FQ_D64_BS(4, true);
+        if (rows_per_page == 8) FQ_D64_BS(3, 4);
+        else FQ_D64_BS(4, 4);
     } else {
-        if (rows_per_page == 8) FQ_D64_BS(3, false);
-        else if (rows_per_page == 16) FQ_D64_BS(4, false);
-        else FQ_D64_BS(5, false);
+        if (rows_per_page == 8) FQ_D64_BS(3, 0);
+        else if (rows_per_page == 16) FQ_D64_BS(4, 0);
+        else FQ_D64_BS(5, 0);
     }
 #undef FQ_D64_BS
 #undef FQ_D64_GP
@@ -2173,7 +2152,7 @@ int launch_staged_d256(const DecodeParams& p, int S, int BS, bool wide, hipStrea
 }
 
 template <int D, int DT>
-int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bool allow_half, const DecodeVariant& var) {
+int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, const DecodeVariant& var) {
     if constexpr (D == 256) {
         if (p.new_key == nullptr && p.rotation == nullptr && staged_d256_applies(D, p.H_KV, var)) {
             const int64_t max_ctx = int64_t(p.max_blocks) * BS;
@@ -2187,7 +2166,7 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, bo
         }
     }
     if constexpr (D == 64) {
-        const bool d64_half = allow_half && staged_d64_half_applies(D, p.H_KV, p.G, BS, var);
+        const bool d64_half = staged_d64_half_applies(D, p.H_KV, p.G, BS, var);
         if (p.new_key == nullptr && (d64_half || staged_d64_full_applies(D, p.H_KV, p.G, var))) {
             const int rows_per_page = d64_half ? BS / 2 : BS;
             const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
@@ -2392,8 +2371,6 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     // than to read (measured on 32 x 4096 tokens: 1 KV head 85 us at 64 splits, 37 us at 16).
     const bool staged_form = rows_of_tokens || (D == 256 && H_KV % 4 == 0) || (D == 64 && H_KV == 8 && block_size >= 16);
     if (H_KV < 8 && !staged_form && ns > max_ctx / 256) ns = max_ctx / 256;
-    // (8 KV heads of dimension 64 write two partials per split: 128 of them at most, as below)
-    if (D == 64 && H_KV == 8 && block_size >= 16 && ns > 64) ns = 64;
     // (a chunk is at least 64 rows)
     if (rows_of_tokens && ns > max_ctx * H_KV / 512) ns = max_ctx * H_KV / 512;
     if (ns > tiles) ns = tiles;
@@ -2423,8 +2400,6 @@ extern "C" size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_K
                                                   int max_blocks_per_seq, int num_splits) {
     if (num_seqs <= 0 || H_Q <= 0 || H_KV <= 0 || D <= 0) return 0;
     num_splits = fq::effective_splits(num_splits, num_seqs, H_KV, D, block_size, max_blocks_per_seq);
-    // room for the partials per split of the staged decode on rows of several tokens
-    num_splits *= fq::partials_per_split_room(D, H_KV, block_size);
     return fq::workspace_layout(num_seqs, H_Q, D, num_splits).total;
 }
 
@@ -2450,7 +2425,7 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
                     const int32_t* seq_lens, const float* centroids_k, const float* centroids_v, float* partial_acc,
                     float* partial_m, float* partial_l, int num_seqs, int H_Q, int H_KV, int D, int block_size,
                     int max_blocks_per_seq, int64_t num_blocks, float sm_scale, int dtype, int num_splits,
-                    void* stream, const DecodeVariant& var, bool allow_half = false, const NewToken* token = nullptr) {
+                    void* stream, const DecodeVariant& var, const NewToken* token = nullptr) {
     const int bad = check_decode_shape(num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, dtype,
                                        num_splits);
     if (bad != FQ_OK) return bad;
@@ -2482,8 +2457,8 @@ int decode_partials(const void* q, const float* rotation, int rotation_col_major
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define FQ_DECODE_D(DD)                                                                 \
     case DD:                                                                            \
-        return dtype == FQ_F16 ? launch_partials<DD, FQ_F16>(p, num_seqs, block_size, s, allow_half, var) \
-                               : launch_partials<DD, FQ_BF16>(p, num_seqs, block_size, s, allow_half, var);
+        return dtype == FQ_F16 ? launch_partials<DD, FQ_F16>(p, num_seqs, block_size, s, var) \
+                               : launch_partials<DD, FQ_BF16>(p, num_seqs, block_size, s, var);
     switch (D) {
         FQ_DECODE_D(64)
         FQ_DECODE_D(128)
@@ -2554,11 +2529,10 @@ int split_k_paged_decode_impl(const void* q, const uint8_t* kv_cache, const int3
     if (!q || !out) return FQ_ERR_NULL_POINTER;
     if (!fq_host::aligned(q, 16) || !fq_host::aligned(out, 16)) return FQ_ERR_MISALIGNED;
     num_splits = effective_splits(num_splits, num_seqs, H_KV, D, block_size, max_blocks_per_seq);
-    // fewer than 8 KV heads: the staged kernel reads rows of several tokens and writes one partial per token of a row
     const int G = H_Q / H_KV;
-    const bool linear = staged_linear_applies(D, H_KV, block_size, var);
-    const bool half = linear || staged_d64_half_applies(D, H_KV, G, block_size, var);
-    const int num_partials = (half && !linear) ? 2 * num_splits : num_splits;
+    // the forms of the staged kernel on rows of several tokens (they too write one partial per split)
+    const bool half = staged_linear_applies(D, H_KV, block_size, var) || staged_d64_half_applies(D, H_KV, G, block_size, var);
+    const int num_partials = num_splits;
     const WorkspaceLayout w = workspace_layout(num_seqs, H_Q, D, num_partials);
     if (!workspace || workspace_bytes < w.total) return FQ_ERR_WORKSPACE;
     if (!fq_host::aligned(workspace, 256)) return FQ_ERR_MISALIGNED;
@@ -2579,7 +2553,7 @@ int split_k_paged_decode_impl(const void* q, const uint8_t* kv_cache, const int3
     }
     int st = decode_partials(q_in, fused_rotation, rotation_col_major, kv_cache, block_table, seq_lens, centroids_k, centroids_v, acc, m,
                              l, num_seqs, H_Q, H_KV, D, block_size, max_blocks_per_seq, num_blocks, sm_scale, dtype,
-                             num_splits, stream, var, half, token);
+                             num_splits, stream, var, token);
     if (st != FQ_OK) return st;
     return fq_split_k_reduce(acc, m, l, rotation, rotation_col_major, out, num_seqs, H_Q, D, dtype, num_partials, stream);
 }
@@ -2691,10 +2665,8 @@ extern "C" int fq_split_k_paged_decode_static(const void* q, const uint8_t* kv_c
     if (bad != FQ_OK) return bad;
     if (num_seqs == 0) return FQ_OK;
     const int ns = effective_splits(num_splits, num_seqs, H_KV, D, block_size, max_blocks_per_seq);
-    // the partials of this launch must fit the array: a larger problem is refused, not truncated (room
-    // for the partials per split of the staged decode on rows of several tokens whatever the switches say, as in
-    // fq_paged_decode_workspace_bytes: the call below reads the switches once for itself)
-    const int num_partials = ns * partials_per_split_room(D, H_KV, block_size);
+    // the partials of this launch must fit the array: a larger problem is refused, not truncated
+    const int num_partials = ns;
     if (workspace_layout(num_seqs, H_Q, D, num_partials).total > kStaticScratchBytes) return FQ_ERR_WORKSPACE;
     void* ws = nullptr;
     const int st = static_scratch_address(&ws);

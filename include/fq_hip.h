@@ -499,9 +499,7 @@ int fq_paged_decode_auto_splits(int num_seqs, int H_KV, int block_size,
  * request to this value; fq_paged_tq4_decode rejects it (FQ_ERR_BAD_SHAPE). */
 int fq_paged_decode_min_splits(int block_size, int max_blocks_per_seq);
 
-/* Bytes of workspace for the given launch; num_splits == 0 means "auto".  (8 KV
- * heads of dimension 64 on pages of 16 or 32 tokens: room for two partials
- * per split, one per token parity.) */
+/* Bytes of workspace for the given launch; num_splits == 0 means "auto". */
 size_t fq_paged_decode_workspace_bytes(int num_seqs, int H_Q, int H_KV, int D,
                                        int block_size, int max_blocks_per_seq,
                                        int num_splits);
