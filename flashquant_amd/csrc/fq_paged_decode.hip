@@ -687,8 +687,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     constexpr int TPR = MULTI == 4 ? 2 : 1 << MULTI;     // tokens per row
     constexpr int HPR = 8 / TPR;             // real KV heads per row
     static_assert(MULTI == 0 || (MULTI >= 2 && MULTI <= 4), "rows of 1, 2, 4 or 8 tokens");
-    static_assert(!LINEAR || (!PROD && CW > 0 && (DIM == 128 || (DIM == 64 && MULTI == 4))),
-                  "rows of several tokens as they lie in the cache: TQ4, copy wavefronts, head_dim 128 or (rows of 2 tokens) 64");
+    static_assert(!LINEAR || (!PROD && CW > 0 && (DIM == 128 || DIM == 64)),
+                  "rows of several tokens as they lie in the cache: TQ4, copy wavefronts, head_dim 128 or 64");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
     static_assert(DIM == 128 || (!PROD && !STORE && CW > 0), "head_dim 64 / 256 are served by the TQ4 form with copy wavefronts");
     // D256: the kernel's "heads" are the halves of real heads of 256 coordinates (wavefront h: real head h / 2 of the
@@ -2093,12 +2093,13 @@ int launch_staged_linear(const DecodeParams& p, int S, int rows_per_page, hipStr
 }
 
 // head_dim 64 on the staged kernel: pairs of neighbouring KV heads as heads of 128 (16 real heads a group), or, with
-// 8 KV heads on pages of 16 or 32 tokens, rows of two tokens of four such pairs.  Up to 8 query heads per KV head.
+// 8, 4 or 2 KV heads on pages of 16 or 32 tokens, rows of 2, 4 or 8 tokens of 4, 2 or 1 such pairs.  Up to 8 query
+// heads per KV head.
 inline bool staged_d64_full_applies(int D, int H_KV, int G, const DecodeVariant& v) {
     return D == 64 && H_KV % 16 == 0 && G <= 8 && !v.direct && v.copy_waves == 4;
 }
 inline bool staged_d64_half_applies(int D, int H_KV, int G, int block_size, const DecodeVariant& v) {
-    return D == 64 && H_KV == 8 && G <= 8 && block_size >= 16 && !v.direct && v.copy_waves == 4;
+    return D == 64 && (H_KV == 8 || H_KV == 4 || H_KV == 2) && G <= 8 && block_size >= 16 && !v.direct && v.copy_waves == 4;
 }
 template <int DT>
 int launch_staged_d64(const DecodeParams& p, int S, int rows_per_page, bool wide, bool half, hipStream_t stream) {
@@ -2114,9 +2115,24 @@ int launch_staged_d64(const DecodeParams& p, int S, int rows_per_page, bool wide
         else if (p.G <= 8) { FQ_D64_GP(BSL, 8, MULTIV); } \
         else { FQ_D64_GP(BSL, 16, MULTIV); }              \
     } while (0)
-    if (half) {
+    if (half && p.H_KV == 8) {
         if (rows_per_page == 8) FQ_D64_BS(3, 4);
         else FQ_D64_BS(4, 4);
+    } else if (half) {      // 4 and 2 KV heads: always four page-id registers
+#define FQ_D64_FEW(BSL, MULTIV)                                                                                                          \
+    do {                                                                                                                                 \
+        if (p.G <= 4) return launch_with_lds(paged_decode_staged_kernel<BSL, 4, DT, 4, false, 4, MULTIV, false, 64>, p, grid, block, lds, stream);  \
+        if (p.G <= 8) return launch_with_lds(paged_decode_staged_kernel<BSL, 8, DT, 4, false, 4, MULTIV, false, 64>, p, grid, block, lds, stream);  \
+        return launch_with_lds(paged_decode_staged_kernel<BSL, 16, DT, 4, false, 4, MULTIV, false, 64>, p, grid, block, lds, stream);    \
+    } while (0)
+        if (p.H_KV == 4) {
+            if (rows_per_page == 4) FQ_D64_FEW(2, 2);
+            else FQ_D64_FEW(3, 2);
+        } else {
+            if (rows_per_page == 2) FQ_D64_FEW(1, 3);
+            else FQ_D64_FEW(2, 3);
+        }
+#undef FQ_D64_FEW
     } else {
         if (rows_per_page == 8) FQ_D64_BS(3, 0);
         else if (rows_per_page == 16) FQ_D64_BS(4, 0);
@@ -2168,7 +2184,7 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, co
     if constexpr (D == 64) {
         const bool d64_half = staged_d64_half_applies(D, p.H_KV, p.G, BS, var);
         if (p.new_key == nullptr && (d64_half || staged_d64_full_applies(D, p.H_KV, p.G, var))) {
-            const int rows_per_page = d64_half ? BS / 2 : BS;
+            const int rows_per_page = d64_half ? BS * p.H_KV / 16 : BS;
             const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
             const int64_t chunk_rows = (((max_rows + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
             DecodeParams ps = p;
@@ -2351,7 +2367,9 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     const int64_t target_waves = int64_t(fq_host::device_cu_count()) * 8;
     // (4 KV heads run as 8: the staged kernel reads their tokens in pairs; 1 and 2 of dimension 128 likewise, in
     // rows of 8 and 4 tokens; `rows_of_tokens`: the forms that count their chunks in such rows)
-    const bool rows_of_tokens = D == 128 && (H_KV == 1 || H_KV == 2 || H_KV == 4) && block_size >= 16;
+    const bool rows_of_tokens = block_size >= 16 && ((D == 128 && (H_KV == 1 || H_KV == 2 || H_KV == 4)) ||
+                                                     (D == 64 && (H_KV == 2 || H_KV == 4)));
+    const int64_t tokens_per_row = rows_of_tokens ? (D == 128 ? 8 : 16) / H_KV : 1;
     int64_t heads = (H_KV == 4 || rows_of_tokens) ? 8 : H_KV;
     // (a workgroup of the staged kernel has 8 wavefronts whatever they serve: a KV head of 256 coordinates takes two
     // of them, a pair of KV heads of 64 coordinates one; measured on 32 x 4096 tokens: head_dim 256 with 8 KV heads
@@ -2363,7 +2381,7 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     // of the sequences are not known here, a ragged batch leaves many splits empty, and the
     // kernel can merge splits (it sizes its chunks from the actual lengths) but not divide them
     // (rows of tokens: chunks of 1024 rows, not tokens)
-    const int64_t long_chunks = rows_of_tokens ? max_ctx * H_KV / 8192 : max_ctx / 1024;
+    const int64_t long_chunks = max_ctx / (1024 * tokens_per_row);
     int64_t ns = 2 * one_round < long_chunks ? 2 * one_round : long_chunks;
     if (ns < one_round) ns = one_round;
     // Where fewer than 8 KV heads run the direct kernel, its workgroups are as small as the head count: a
@@ -2372,7 +2390,7 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     const bool staged_form = rows_of_tokens || (D == 256 && H_KV % 4 == 0) || (D == 64 && H_KV == 8 && block_size >= 16);
     if (H_KV < 8 && !staged_form && ns > max_ctx / 256) ns = max_ctx / 256;
     // (a chunk is at least 64 rows)
-    if (rows_of_tokens && ns > max_ctx * H_KV / 512) ns = max_ctx * H_KV / 512;
+    if (rows_of_tokens && ns > max_ctx / (64 * tokens_per_row)) ns = max_ctx / (64 * tokens_per_row);
     if (ns > tiles) ns = tiles;
     // Beyond 128 splits the combine step (one pass over the maxima per 64 splits, one partial row
     // per split) costs more than the shorter chunks save (measured on 1 x 32768 tokens, 8 KV

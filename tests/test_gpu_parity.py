@@ -352,13 +352,15 @@ def test_paged_decode_on_a_caller_workspace_with_arbitrary_contents():
 
 @pytest.mark.parametrize("hq,hkv,bs,dtype", [(32, 8, 16, torch.bfloat16), (64, 8, 32, torch.float16), (8, 8, 16, torch.bfloat16),
                                              (24, 8, 16, torch.float16), (32, 16, 16, torch.bfloat16), (64, 16, 8, torch.float16),
-                                             (128, 16, 32, torch.bfloat16), (96, 32, 16, torch.bfloat16), (16, 16, 16, torch.float16)])
+                                             (128, 16, 32, torch.bfloat16), (96, 32, 16, torch.bfloat16), (16, 16, 16, torch.float16),
+                                             (16, 4, 16, torch.bfloat16), (32, 4, 32, torch.float16), (4, 4, 16, torch.bfloat16),
+                                             (14, 2, 16, torch.bfloat16), (16, 2, 32, torch.float16), (2, 2, 16, torch.float16)])
 def test_paged_decode_head_dim_64_on_the_staged_kernel(hq, hkv, bs, dtype, kernel_option):
-    """head_dim 64 with 8 KV heads (pages of 16 / 32 tokens) or a multiple of 16: pairs of neighbouring heads run as
-    heads of 128 on the staged kernel, the query rotation in its prologue.  Against the oracle, and against the
-    direct kernel on the same inputs."""
+    """head_dim 64 with 8, 4 or 2 KV heads (pages of 16 / 32 tokens: rows of 2, 4 or 8 tokens) or a multiple of 16:
+    pairs of neighbouring heads run as heads of 128 on the staged kernel, the query rotation in its prologue.
+    Against the oracle, and against the direct kernel on the same inputs."""
     c, b, r = book(64)
-    for lens, splits in (([37, 0, 16, 300, 64, 65, 1, 129], 3), ([1500, 0, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0)):
+    for lens, splits in (([37, 0, 16, 300, 64, 65, 1, 129, 2, 3, 5, 7, 9], 3), ([1500, 0, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0)):
         _decode_case(lens, hq=hq, hkv=hkv, d=64, bs=bs, num_splits=splits, dtype=dtype)
         q, cache, table, sl = build_paged_case(lens, hq, hkv, d=64, bs=bs, seed=31, dtype=dtype)
         dev = [t.to(DEV) for t in (q, cache, table, sl, c, r)]
