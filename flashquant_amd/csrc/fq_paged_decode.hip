@@ -687,8 +687,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     constexpr int TPR = MULTI == 4 ? 2 : 1 << MULTI;     // tokens per row
     constexpr int HPR = 8 / TPR;             // real KV heads per row
     static_assert(MULTI == 0 || (MULTI >= 2 && MULTI <= 4), "rows of 1, 2, 4 or 8 tokens");
-    static_assert(!LINEAR || (!PROD && CW > 0 && (DIM == 128 || DIM == 64)),
-                  "rows of several tokens as they lie in the cache: TQ4, copy wavefronts, head_dim 128 or 64");
+    static_assert(!LINEAR || (!PROD && CW > 0), "rows of several tokens as they lie in the cache: TQ4, copy wavefronts");
+    static_assert(!(D256 && LINEAR) || HPR % 2 == 0, "head_dim 256: the two halves of a head in one token");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
     static_assert(DIM == 128 || (!PROD && !STORE && CW > 0), "head_dim 64 / 256 are served by the TQ4 form with copy wavefronts");
     // D256: the kernel's "heads" are the halves of real heads of 256 coordinates (wavefront h: real head h / 2 of the
@@ -705,8 +705,9 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     constexpr int kRowLds = 16 * Cfg::CHUNKS_PER_ROW + 16;    // 1104; head_dim 64: 1168
     // LINEAR: bytes of a token in such a row, and of its key (or value) norms; HPR counts heads of 128 coordinates,
     // at head_dim 64 pairs of real heads
-    constexpr int kTokenBytes = (D64 ? 144 : 136) * HPR;
-    constexpr int kTokenNormBytes = (D64 ? 8 : 4) * HPR;
+    // or, at 256, halves of real heads
+    constexpr int kTokenBytes = (D64 ? 144 : D256 ? 132 : 136) * HPR;
+    constexpr int kTokenNormBytes = (D64 ? 8 : D256 ? 2 : 4) * HPR;
     constexpr int kStageBytes = LINEAR ? 16 * kRowLds : Cfg::STAGE_BYTES;
     constexpr int kTileBytes = 2 * kStageBytes;
     constexpr int kChunksPerRow = Cfg::CHUNKS_PER_ROW;
@@ -728,8 +729,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // STORE: [7] computing wavefronts whose part of the new token's row has reached the cache
     __shared__ uint32_t flags[8];
     // D256: [h] score halves posted by wavefront h, [8 + h] partner halves read by wavefront h (counts of tiles)
-    // LINEAR: [0] computing wavefronts that have posted their partial for the merge at the end
-    __shared__ uint32_t xflags[16];
+    // LINEAR: [16] computing wavefronts that have posted their partial for the merge at the end
+    __shared__ uint32_t xflags[17];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -751,14 +752,15 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     // More than 8 KV heads: a workgroup serves the group of 8 heads blockIdx.z, i.e. the query heads
     // hq0 .. hq0 + 8 G - 1, and copies that group's slices of the token rows.
     const int hgrp = blockIdx.z;
-    const int HQG = (D256 ? 4 : HPR) * p.G;              // query heads of a group
+    const int HQG = (D256 ? HPR / 2 : HPR) * p.G;        // query heads of a group
     const int hq0 = hgrp * HQG;
     const int row_bytes = D64 ? (MULTI > 0 ? 1152 : p.H_KV * 72)
-                        : D256 ? p.H_KV * 264
+                        : D256 ? (MULTI > 0 ? 1056 : p.H_KV * 264)
                                : (MULTI > 0 ? 1088 : p.H_KV * (PROD ? 140 : 136));   // a row of the cache as the kernel sees it
     const int qsub = D64 && (n % GP) >= p.G / 2 ? 1 : 0;    // D64: this lane's query head belongs to the pair's second head
     // MULTI > 0: wavefront h works on real head h % HPR and on token h / HPR of every row
-    const int hr = D256 ? (h >> 1) : (h & (HPR - 1));          // D256: the real head; its half is h & 1
+    const int hh = h & (HPR - 1);                              // the kernel's head of 128 coordinates inside a token
+    const int hr = D256 ? (hh >> 1) : hh;                      // D256: the real head; its half is h & 1
     const int tsel = (h / HPR) & (TPR - 1);
 
     // Every load that depends on nothing is asked for first, so that the memory
@@ -834,10 +836,10 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         if constexpr (LINEAR) {
             // the token rows as they lie in the cache: token tsel of the row, head hr of its HPR heads
             const int token = kTokenBytes * tsel;
-            k_rd[b] = b * kStageBytes + kRowLds * n + token + 64 * hr + 16 * g;
+            k_rd[b] = b * kStageBytes + kRowLds * n + token + 64 * hh + 16 * g;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                v_rd[b][i] = b * kStageBytes + kRowLds * (4 * g + i) + token + 64 * HPR + kTokenNormBytes + 64 * hr + 4 * n;
+                v_rd[b][i] = b * kStageBytes + kRowLds * (4 * g + i) + token + 64 * HPR + kTokenNormBytes + 64 * hh + 4 * n;
         } else {
             k_rd[b] = b * kStageBytes + 16 * staged_slot(h, n, g);
 #pragma unroll
@@ -932,7 +934,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
         // wavefront has just asked for its sequence length and page ids and none has used them yet
         // (the barrier does not wait for loads from global memory).
         if (tid < 8) flags[tid] = 0u;
-        if ((D256 || LINEAR) && tid < 16) xflags[tid] = 0u;
+        if ((D256 || LINEAR) && tid < 17) xflags[tid] = 0u;
         __syncthreads();
         load_matrix_columns();
         load_first_heads();
@@ -1675,8 +1677,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                 }
             }
         }
-        lds_flag_signal(&xflags[0], lane);
-        bool merged = lds_flag_wait(&xflags[0], 8u, p.spin_limit);
+        lds_flag_signal(&xflags[16], lane);
+        bool merged = lds_flag_wait(&xflags[16], 8u, p.spin_limit);
         if (!merged && lane == 0) atomicAdd(&g_decode_faults, 1u);
         constexpr int CPW = 128 / TPR;                        // coordinates of a head that this wavefront combines
         // maximum over the wavefronts of this head (NaN when a hand-off failed), no array: the values are read again
@@ -1685,7 +1687,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             bool bad = !merged;
 #pragma unroll
             for (int t = 0; t < TPR; ++t) {
-                const float m = xml[((t * HPR + hr) * 16 + head) * 2];
+                const float m = xml[((t * HPR + hh) * 16 + head) * 2];
                 bad = bad || m != m;
                 ms = __builtin_fmaxf(ms, m);
             }
@@ -1697,25 +1699,27 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
             float acc = 0.0f;
 #pragma unroll
             for (int t = 0; t < TPR; ++t) {
-                const float m = xml[((t * HPR + hr) * 16 + head) * 2];
+                const float m = xml[((t * HPR + hh) * 16 + head) * 2];
                 const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(m - ms);
-                acc += w * xacc[((t * HPR + hr) * 16 + head) * 128 + c];
+                acc += w * xacc[((t * HPR + hh) * 16 + head) * 128 + c];
             }
             if constexpr (D64) {     // a query head's output: the half of the 128 coordinates that is its own head's
                 if ((c >> 6) == (head >= p.G / 2 ? 1 : 0))
                     p.part_acc[((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS + split) * 64 + (c & 63)] = acc;
+            } else if constexpr (D256) {   // this wavefront's half of the head's 256 coordinates
+                p.part_acc[((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS + split) * 256 + 128 * (h & 1) + c] = acc;
             } else {
                 p.part_acc[((int64_t(seq) * p.H_Q + hq0 + hr * p.G + head) * NS + split) * D + c] = acc;
             }
         }
-        if (tsel == 0 && lane < p.G) {
+        if (tsel == 0 && lane < p.G && (!D256 || (h & 1) == 0)) {
             const float ms = merged_max(lane);
             float l = 0.0f;
 #pragma unroll
             for (int t = 0; t < TPR; ++t) {
-                const float m = xml[((t * HPR + hr) * 16 + lane) * 2];
+                const float m = xml[((t * HPR + hh) * 16 + lane) * 2];
                 const float w = ms == -__builtin_inff() ? 0.0f : __builtin_amdgcn_exp2f(m - ms);
-                l += w * xml[((t * HPR + hr) * 16 + lane) * 2 + 1];
+                l += w * xml[((t * HPR + hh) * 16 + lane) * 2 + 1];
             }
             const int64_t o = (int64_t(seq) * p.H_Q + hq0 + hr * p.G + lane) * NS + split;
             p.part_m[o] = ms;
@@ -2167,9 +2171,39 @@ int launch_staged_d256(const DecodeParams& p, int S, int BS, bool wide, hipStrea
 #undef FQ_D256_GP
 }
 
+// head_dim 256 with 2 KV heads or 1 on pages of 16 or 32 tokens: rows of 2 or 4 tokens (4 halves of heads or 2 a token).
+inline bool staged_d256_linear_applies(int D, int H_KV, int block_size, const DecodeVariant& v) {
+    return D == 256 && (H_KV == 1 || H_KV == 2) && block_size >= 16 && !v.direct && v.copy_waves == 4;
+}
+template <int DT>
+int launch_staged_d256_linear(const DecodeParams& p, int S, int rows_per_page, hipStream_t stream) {
+    // two tiles of 32 rows (1056 bytes every 1072) and the patch through which the halves of a head exchange their scores
+    const size_t lds = 2 * 32 * 1072 + 8 * 2 * kWave * sizeof(float4v);
+    const dim3 grid(S, p.num_splits, 1), block(512 + 64 * 4);
+#define FQ_D256_FEW(BSL, MULTIV)                                                                                                          \
+    do {                                                                                                                                  \
+        if (p.G <= 4) return launch_with_lds(paged_decode_staged_kernel<BSL, 4, DT, 4, false, 4, MULTIV, false, 256>, p, grid, block, lds, stream);  \
+        if (p.G <= 8) return launch_with_lds(paged_decode_staged_kernel<BSL, 8, DT, 4, false, 4, MULTIV, false, 256>, p, grid, block, lds, stream);  \
+        return launch_with_lds(paged_decode_staged_kernel<BSL, 16, DT, 4, false, 4, MULTIV, false, 256>, p, grid, block, lds, stream);    \
+    } while (0)
+    if (p.H_KV == 2) {
+        if (rows_per_page == 8) FQ_D256_FEW(3, 4);
+        else FQ_D256_FEW(4, 4);
+    } else {
+        if (rows_per_page == 4) FQ_D256_FEW(2, 2);
+        else FQ_D256_FEW(3, 2);
+    }
+#undef FQ_D256_FEW
+}
+
 template <int D, int DT>
 int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, const DecodeVariant& var) {
     if constexpr (D == 256) {
+        if (p.new_key == nullptr && p.rotation == nullptr && staged_d256_linear_applies(D, p.H_KV, BS, var)) {
+            DecodeParams ps = p;
+            ps.balance_slots = staged_balance_slots(S, p.num_splits);
+            return launch_staged_d256_linear<DT>(ps, S, BS * p.H_KV / 4, stream);
+        }
         if (p.new_key == nullptr && p.rotation == nullptr && staged_d256_applies(D, p.H_KV, var)) {
             const int64_t max_ctx = int64_t(p.max_blocks) * BS;
             const int64_t chunk = (((max_ctx + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
@@ -2368,8 +2402,9 @@ int auto_splits(int num_seqs, int H_KV, int D, int block_size, int max_blocks_pe
     // (4 KV heads run as 8: the staged kernel reads their tokens in pairs; 1 and 2 of dimension 128 likewise, in
     // rows of 8 and 4 tokens; `rows_of_tokens`: the forms that count their chunks in such rows)
     const bool rows_of_tokens = block_size >= 16 && ((D == 128 && (H_KV == 1 || H_KV == 2 || H_KV == 4)) ||
-                                                     (D == 64 && (H_KV == 2 || H_KV == 4)));
-    const int64_t tokens_per_row = rows_of_tokens ? (D == 128 ? 8 : 16) / H_KV : 1;
+                                                     (D == 64 && (H_KV == 2 || H_KV == 4)) ||
+                                                     (D == 256 && (H_KV == 1 || H_KV == 2)));
+    const int64_t tokens_per_row = rows_of_tokens ? (D == 128 ? 8 : D == 64 ? 16 : 4) / H_KV : 1;
     int64_t heads = (H_KV == 4 || rows_of_tokens) ? 8 : H_KV;
     // (a workgroup of the staged kernel has 8 wavefronts whatever they serve: a KV head of 256 coordinates takes two
     // of them, a pair of KV heads of 64 coordinates one; measured on 32 x 4096 tokens: head_dim 256 with 8 KV heads

@@ -372,13 +372,15 @@ def test_paged_decode_head_dim_64_on_the_staged_kernel(hq, hkv, bs, dtype, kerne
 
 
 @pytest.mark.parametrize("hq,hkv,bs,dtype", [(16, 4, 16, torch.bfloat16), (32, 8, 16, torch.bfloat16), (8, 8, 32, torch.float16),
-                                             (64, 4, 8, torch.bfloat16), (24, 12, 16, torch.float16), (20, 4, 16, torch.bfloat16)])
+                                             (64, 4, 8, torch.bfloat16), (24, 12, 16, torch.float16), (20, 4, 16, torch.bfloat16),
+                                             (8, 1, 16, torch.bfloat16), (4, 1, 32, torch.float16), (1, 1, 16, torch.bfloat16),
+                                             (16, 2, 16, torch.bfloat16), (6, 2, 32, torch.float16), (32, 2, 16, torch.float16)])
 def test_paged_decode_head_dim_256_on_the_staged_kernel(hq, hkv, bs, dtype, kernel_option):
-    """head_dim 256 with a multiple of 4 KV heads: the halves of a head run as two heads of 128 on the staged kernel
-    (the two wavefronts of a head add their halves of the scores through LDS).  Against the oracle, and against the
-    direct kernel on the same inputs."""
+    """head_dim 256 with a multiple of 4 KV heads, or 2 or 1 on pages of 16 / 32 tokens (rows of 2 or 4 tokens): the
+    halves of a head run as two heads of 128 on the staged kernel (the two wavefronts of a head add their halves of
+    the scores through LDS).  Against the oracle, and against the direct kernel on the same inputs."""
     c, b, r = book(256)
-    for lens, splits in (([37, 0, 16, 300, 64, 65, 1, 129], 3), ([1500, 0, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0)):
+    for lens, splits in (([37, 0, 16, 300, 64, 65, 1, 129, 2, 3, 5, 7], 3), ([1500, 0, 37, 6000, 64, 2049, 1, 3333], 40), ([70, 5, 200], 0)):
         _decode_case(lens, hq=hq, hkv=hkv, d=256, bs=bs, num_splits=splits, dtype=dtype)
         q, cache, table, sl = build_paged_case(lens, hq, hkv, d=256, bs=bs, seed=32, dtype=dtype)
         dev = [t.to(DEV) for t in (q, cache, table, sl, c, r)]
