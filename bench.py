@@ -594,6 +594,8 @@ def main():
             "decode_128x8192_16q_2kv_d128": (128, 8192, 16, 2, 128),
             "decode_32x4096_32q_8kv_d64": (32, 4096, 32, 8, 64),
             "decode_32x4096_32q_8kv_d256": (32, 4096, 32, 8, 256),
+            "decode_32x4096_8q_1kv_d256": (32, 4096, 8, 1, 256),        # one KV head of 256 coordinates
+            "decode_32x4096_16q_4kv_d64": (32, 4096, 16, 4, 64),
         }).items():
             ms, nbytes = decode_shape(n_seq, ctx, hq, hkv, d)
             shapes[name] = {"step_us": ms * 1e3, "gbps": nbytes / (ms * 1e-3) / 1e9,
