@@ -26,7 +26,7 @@ def _heads(rng):
     return d, hkv, hkv * g
 
 
-@pytest.mark.parametrize("case", range(40))
+@pytest.mark.parametrize("case", range(100))
 def test_random_paged_decode(case):
     rng = random.Random(9100 + case)
     d, hkv, hq = _heads(rng)
@@ -41,7 +41,7 @@ def test_random_paged_decode(case):
                    num_splits=rng.choice([0, 1, 2, 3, 5, 8, 17]), seed=100 + case)
 
 
-@pytest.mark.parametrize("case", range(40))
+@pytest.mark.parametrize("case", range(80))
 def test_random_store_and_decode(case, kernel_option):
     """The serving step (new token stored, then decoded over) on random shapes: the in-launch store where the
     staged kernel runs, the two launches elsewhere."""
