@@ -690,7 +690,8 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     static_assert(!LINEAR || (!PROD && CW > 0), "rows of several tokens as they lie in the cache: TQ4, copy wavefronts");
     static_assert(!(D256 && LINEAR) || HPR % 2 == 0, "head_dim 256: the two halves of a head in one token");
     static_assert(!STORE || (CW > 0 && !PROD), "the new token is stored by the TQ4 forms with copy wavefronts");
-    static_assert(DIM == 128 || (!PROD && !STORE && CW > 0), "head_dim 64 / 256 are served by the TQ4 form with copy wavefronts");
+    static_assert(DIM == 128 || (!PROD && CW > 0), "head_dim 64 / 256 are served by the TQ4 form with copy wavefronts");
+    static_assert(!STORE || DIM == 128 || (DIM == 64 && LINEAR), "the new token is stored at head_dim 128, and at 64 on rows of tokens");
     // D256: the kernel's "heads" are the halves of real heads of 256 coordinates (wavefront h: real head h / 2 of the
     // group of 4, coordinates 128 (h % 2) ...): the two wavefronts of a head exchange their halves of the scores
     // through LDS every tile and add them, compute the same weights, and each accumulates its half of the output
@@ -947,7 +948,7 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
     float bnd_mine = 0.0f;      // boundary `lane` of the 15 (asked for here: at its use it would be a round trip of its own)
     if constexpr (STORE) {
         if (!copier) {
-            const int kv_heads = MULTI > 0 ? HPR : p.H_KV;
+            const int kv_heads = MULTI > 0 ? HPR : p.H_KV;       // (head_dim 64: pairs of heads, 128 elements together)
             const int nr = n < 2 * kNewHeads ? n : 2 * kNewHeads - 1;     // block row: key head nr, or value head nr - KH
             const uint16_t* xrow = reinterpret_cast<const uint16_t*>(nr < kNewHeads ? p.new_key : p.new_value) +
                                    (int64_t(seq) * kv_heads + kNewHeads * hgrp + (nr & (kNewHeads - 1))) * 128;
@@ -1239,21 +1240,24 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                     // (cpu_reference.py:22-61, vllm/impl.py:220-263).  Wavefront h holds columns 16h..16h+15.
                     // Block row r: key head r for r < KH, value head r - KH for r < 2 KH.
                     constexpr int KH = kNewHeads;
-                    const int token_row_bytes = MULTI > 0 ? 136 * HPR : row_bytes;
+                    const int token_row_bytes = MULTI > 0 ? kTokenBytes : row_bytes;
                     const int kv_heads = MULTI > 0 ? HPR : p.H_KV;
                     const int64_t slot = new_slot;
                     uint4v raw[KS];
 #pragma unroll
                     for (int j = 0; j < KS; ++j) raw[j] = new_raw[j];
-                    float ss = 0.0f;         // sum of squares of row n: this lane's 32 elements, then over g
+                    // sum of squares of row n: this lane's 32 elements, then over g.  head_dim 64: a row is a pair of heads,
+                    // elements 0..63 the first and 64..127 the second; wavefront h holds columns of head h / 4 of the pair
+                    float ss = 0.0f;
 #pragma unroll
                     for (int j = 0; j < KS; ++j) {
                         const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+                        const bool mine = !D64 || (j >> 1) == (h >> 2);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             const float a = load_elem<DT>(uint16_t(w[i] & 0xffffu)), b = load_elem<DT>(uint16_t(w[i] >> 16));
-                            ss = __builtin_fmaf(a, a, ss);
-                            ss = __builtin_fmaf(b, b, ss);
+                            ss = mine ? __builtin_fmaf(a, a, ss) : ss;
+                            ss = mine ? __builtin_fmaf(b, b, ss) : ss;
                         }
                     }
                     ss += xor_shuffle(ss, 16);
@@ -1295,12 +1299,17 @@ __global__ __launch_bounds__(512 + 64 * CW) void paged_decode_staged_kernel(cons
                             hi |= uint32_t(__shfl_xor(int(hi), mask, kWave));
                         }
                         const int head = KH * hgrp + (r & (KH - 1));
-                        const int sect = r < KH ? 0 : kv_heads * (D / 2 + 4);            // key sections, then value sections
+                        const int sect = r < KH ? 0 : kv_heads * (D / 2 + (D64 ? 8 : 4));   // key sections, then value sections
                         const bool row_live = stored && r < 2 * KH;
                         if (row_live && n == 0)
                             *reinterpret_cast<uint2v*>(crow + sect + head * (D / 2) + 8 * h) = uint2v{lo, hi};
-                        if (row_live && n == 1 && h == 0)
-                            *reinterpret_cast<float*>(crow + sect + kv_heads * (D / 2) + 4 * head) = nrm;
+                        if constexpr (D64) {     // two norms a pair: wavefronts 0 and 4 hold those of its first and second head
+                            if (row_live && n == 1 && (h & 3) == 0)
+                                *reinterpret_cast<float*>(crow + sect + kv_heads * (D / 2) + 8 * head + 4 * (h >> 2)) = nrm;
+                        } else {
+                            if (row_live && n == 1 && h == 0)
+                                *reinterpret_cast<float*>(crow + sect + kv_heads * (D / 2) + 4 * head) = nrm;
+                        }
                     }
                     // The row must be in the cache before the copy wavefronts ask for the split's last tile.  They
                     // ask for the first two tiles at once; when the last tile is one of those the stores are waited
@@ -2119,9 +2128,28 @@ int launch_staged_d64(const DecodeParams& p, int S, int rows_per_page, bool wide
         else if (p.G <= 8) { FQ_D64_GP(BSL, 8, MULTIV); } \
         else { FQ_D64_GP(BSL, 16, MULTIV); }              \
     } while (0)
-    if (half && p.H_KV == 8) {
+    const bool store = p.new_key != nullptr;     // (rows of tokens only)
+    if (half && p.H_KV == 8 && !store) {
         if (rows_per_page == 8) FQ_D64_BS(3, 4);
         else FQ_D64_BS(4, 4);
+    } else if (half && store) {
+#define FQ_D64_STORE(BSL, MULTIV)                                                                                                        \
+    do {                                                                                                                                 \
+        if (p.G <= 4) return launch_with_lds(paged_decode_staged_kernel<BSL, 4, DT, 4, false, 4, MULTIV, true, 64>, p, grid, block, lds, stream);   \
+        if (p.G <= 8) return launch_with_lds(paged_decode_staged_kernel<BSL, 8, DT, 4, false, 4, MULTIV, true, 64>, p, grid, block, lds, stream);   \
+        return launch_with_lds(paged_decode_staged_kernel<BSL, 16, DT, 4, false, 4, MULTIV, true, 64>, p, grid, block, lds, stream);     \
+    } while (0)
+        if (p.H_KV == 8) {
+            if (rows_per_page == 8) FQ_D64_STORE(3, 4);
+            else FQ_D64_STORE(4, 4);
+        } else if (p.H_KV == 4) {
+            if (rows_per_page == 4) FQ_D64_STORE(2, 2);
+            else FQ_D64_STORE(3, 2);
+        } else {
+            if (rows_per_page == 2) FQ_D64_STORE(1, 3);
+            else FQ_D64_STORE(2, 3);
+        }
+#undef FQ_D64_STORE
     } else if (half) {      // 4 and 2 KV heads: always four page-id registers
 #define FQ_D64_FEW(BSL, MULTIV)                                                                                                          \
     do {                                                                                                                                 \
@@ -2217,7 +2245,7 @@ int launch_partials(const DecodeParams& p, int S, int BS, hipStream_t stream, co
     }
     if constexpr (D == 64) {
         const bool d64_half = staged_d64_half_applies(D, p.H_KV, p.G, BS, var);
-        if (p.new_key == nullptr && (d64_half || staged_d64_full_applies(D, p.H_KV, p.G, var))) {
+        if (d64_half || (p.new_key == nullptr && staged_d64_full_applies(D, p.H_KV, p.G, var))) {
             const int rows_per_page = d64_half ? BS * p.H_KV / 16 : BS;
             const int64_t max_rows = int64_t(p.max_blocks) * rows_per_page;
             const int64_t chunk_rows = (((max_rows + p.num_splits - 1) / p.num_splits) + 63) & ~int64_t(63);
@@ -2650,7 +2678,8 @@ extern "C" int fq_tq4_store_and_decode(const void* key, const void* value, const
         return FQ_ERR_MISALIGNED;
     const DecodeVariant var = read_decode_variant();
     const bool in_launch = centroids_k && var.copy_waves == 4 &&
-                           ((staged_applies(D, H_KV, var) && !var.ring) || staged_linear_applies(D, H_KV, block_size, var));
+                           ((staged_applies(D, H_KV, var) && !var.ring) || staged_linear_applies(D, H_KV, block_size, var) ||
+                            staged_d64_half_applies(D, H_KV, H_Q / H_KV, block_size, var));
     const NewToken token{key, value, slot_mapping, boundaries, kv_cache};
     if (!in_launch) {
         const int st = fq_tq4_compress_store(key, value, dtype, rot_T_even, rot_T_odd, boundaries, kv_cache, slot_mapping,

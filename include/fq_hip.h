@@ -361,7 +361,8 @@ int fq_split_k_paged_decode(const void* q, const uint8_t* kv_cache,
  *   everything else as for fq_split_k_paged_decode; rotation must not be NULL;
  *   seq_lens counts the new token.
  * Where the staged decode kernel runs (D == 128 and H_KV a multiple of 8, or
- * H_KV == 1, 2 or 4 on pages of 16 or 32 tokens; default switches) this is one launch
+ * H_KV == 1, 2 or 4 on pages of 16 or 32 tokens; D == 64 and H_KV == 2, 4 or 8 on
+ * such pages, up to 8 query heads per KV head; default switches) this is one launch
  * fewer: the workgroup whose split ends with a
  * sequence's last token compresses and stores that token in its prologue and
  * reads the row back with its last tile.  For that form slot_mapping[s] must be

@@ -1014,9 +1014,12 @@ def _check_serving_step(lens, hq, hkv, d, bs, dtype, splits, seed):
                                                (128, 8, 128, 32, torch.bfloat16), (32, 16, 128, 16, torch.bfloat16),
                                                (32, 4, 128, 16, torch.bfloat16), (8, 1, 128, 16, torch.bfloat16),
                                                (4, 1, 128, 32, torch.float16), (16, 2, 128, 16, torch.float16),
-                                               (10, 2, 128, 32, torch.bfloat16), (8, 2, 64, 16, torch.float16)])
+                                               (10, 2, 128, 32, torch.bfloat16), (8, 2, 64, 16, torch.float16),
+                                               (32, 8, 64, 16, torch.bfloat16), (16, 4, 64, 32, torch.float16),
+                                               (64, 8, 64, 32, torch.bfloat16), (32, 16, 64, 16, torch.bfloat16),
+                                               (8, 4, 256, 16, torch.bfloat16)])
 def test_store_and_decode_equals_store_then_decode(hq, hkv, d, bs, dtype, kernel_option):
-    """The serving step as one call.  Where the staged kernel runs (all shapes but the last) the workgroup
+    """The serving step as one call.  Where the staged kernel stores (head_dim 128, and 64 on rows of tokens) the workgroup
     that owns a sequence's last token compresses and stores it itself, with the exact float32 rotation:
     the cache must then hold what compress-and-store writes in its three-term mode (indices equal up to
     coordinates within float32 rounding of a boundary, norms to 2e-6), nothing else in the cache may

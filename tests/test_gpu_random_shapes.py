@@ -48,7 +48,7 @@ def test_random_store_and_decode(case, kernel_option):
     kernel_option("compress_three_terms", True)
     rng = random.Random(9500 + case)
     d = rng.choice([128, 128, 128, 128, 64, 256])
-    hkv = rng.choice([8, 8, 8, 16, 24, 4, 2, 1]) if d == 128 else rng.choice([8, 4, 2])
+    hkv = rng.choice([8, 8, 8, 16, 24, 4, 2, 1]) if d == 128 else rng.choice([8, 4, 2, 16])
     g = rng.choice([1, 2, 4, 4, 5, 8, 16]) if d != 256 else rng.choice([1, 2, 4])
     n_seq = rng.choice([1, 2, 3, 5, 9, 17, 33])
     longest = rng.choice([40, 130, 300, 700, 1500, 3000])
