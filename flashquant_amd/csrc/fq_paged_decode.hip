@@ -2044,15 +2044,13 @@ int launch_staged_any(const DecodeParams& p, int S, int BS, bool wide, hipStream
         if constexpr (!PROD) {                                                                                  \
             if (store) {                                                                                        \
                 if (copy_waves != 4) return FQ_ERR_LAUNCH;                                                      \
-                return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4, false, true>, p, S, stream, 4) \
-                            : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 4, false, true>, p, S, stream, 4); \
+                return launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4, false, true>, p, S, stream, 4); \
             }                                                                                                   \
         }                                                                                                       \
         if (copy_waves == 4)                                                                                    \
-            return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4>, p, S, stream, 4) \
-                        : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 4>, p, S, stream, 4); \
-        return wide ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 0>, p, S, stream) \
-                    : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 1, PROD, 0>, p, S, stream); \
+            return (wide || PROD) ? launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 4>, p, S, stream, 4) \
+                                  : launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, PROD ? 4 : 1, PROD, 4>, p, S, stream, 4); \
+        return launch_staged<PROD>(paged_decode_staged_kernel<BSL, GPV, DT, 4, PROD, 0>, p, S, stream); \
     }
 #define FQ_STAGED_BS(BSL)                         \
     do {                                          \
@@ -2120,8 +2118,7 @@ int launch_staged_d64(const DecodeParams& p, int S, int rows_per_page, bool wide
     const size_t lds = half ? 2 * 32 * 1168 : 2 * size_t(StagedCfg<false, 64>::TILE_BYTES);
     const dim3 grid(S, p.num_splits, half ? 1 : p.H_KV / 16), block(512 + 64 * 4);
 #define FQ_D64_GP(BSL, GPV, MULTIV)                                                                                \
-    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, MULTIV, false, 64>, p, grid, block, lds, stream) \
-                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, MULTIV, false, 64>, p, grid, block, lds, stream)
+    return launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, MULTIV, false, 64>, p, grid, block, lds, stream)
 #define FQ_D64_BS(BSL, MULTIV)                            \
     do {                                                 \
         if (p.G <= 4) { FQ_D64_GP(BSL, 4, MULTIV); }      \
@@ -2184,8 +2181,7 @@ int launch_staged_d256(const DecodeParams& p, int S, int BS, bool wide, hipStrea
     const size_t lds = 2 * size_t(StagedCfg<false, 256>::TILE_BYTES) + 8 * 2 * kWave * sizeof(float4v);
     const dim3 grid(S, p.num_splits, p.H_KV / 4), block(512 + 64 * 4);
 #define FQ_D256_GP(BSL, GPV)                                                                                       \
-    return wide ? launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, false, false, 256>, p, grid, block, lds, stream) \
-                : launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 1, false, 4, false, false, 256>, p, grid, block, lds, stream)
+    return launch_with_lds(paged_decode_staged_kernel<BSL, GPV, DT, 4, false, 4, false, false, 256>, p, grid, block, lds, stream)
 #define FQ_D256_BS(BSL)                           \
     do {                                          \
         if (p.G <= 4) { FQ_D256_GP(BSL, 4); }     \
