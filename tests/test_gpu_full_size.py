@@ -228,17 +228,21 @@ def test_serving_step_at_the_benchmark_size(hq, hkv, L):
     row_scale = want.float().abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
     rel = ((got.cpu().float() - want.float()).abs() / row_scale).max().item()
     assert rel <= 2e-2, f"max error {rel} of the row magnitude"
-    # the stored rows against the oracle's: at most 1e-4 of the indices differ, by one bucket; the rest of the cache untouched
+    # the stored rows against the oracle's: an index differs by one bucket at most, and only where the coordinate
+    # (rotated in float64) lies within float32 rounding of a bucket boundary; the rest of the cache untouched
     flat_got, flat_ref = cache_d.cpu().reshape(-1, hkv * 136), ref_cache.reshape(-1, hkv * 136)
     keep = torch.ones(flat_got.shape[0], dtype=torch.bool)
     keep[slots] = False
     assert torch.equal(flat_got[keep], flat_ref[keep])
     half = hkv * 68
-    for base in (0, half):
+    for base, rows_in in ((0, key), (half, value)):
         i1 = O.nibble_unpack(flat_got[slots][:, base:base + hkv * 64].contiguous())
         i2 = O.nibble_unpack(flat_ref[slots][:, base:base + hkv * 64].contiguous())
-        assert (i1 != i2).float().mean().item() <= 1e-4
         assert (i1.int() - i2.int()).abs().max().item() <= 1
+        for row, col in (i1 != i2).nonzero().tolist():
+            x = rows_in[row].reshape(hkv, 128)[col // 128].double()
+            y = (r.double() @ (x / (x.norm() + 1e-10)))[col % 128]
+            assert (b.double() - y).abs().min().item() <= 1e-6, (row, col)
 
 
 def test_prod_paged_decode_at_the_benchmark_batch():

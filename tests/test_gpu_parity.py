@@ -988,11 +988,17 @@ def _check_serving_step(lens, hq, hkv, d, bs, dtype, splits, seed):
     assert torch.equal(one[keep], cache.reshape(-1, hkv * (d + 8))[keep])          # no other row touched
     rows1, rows2 = one[slots[slots >= 0]], two[slots[slots >= 0]]
     half = hkv * (d // 2 + 4)
-    for base in (0, half):
+    stored = (slots >= 0).nonzero().flatten()
+    for base, rows_in in ((0, key), (half, value)):
         i1 = O.nibble_unpack(rows1[:, base:base + hkv * (d // 2)].contiguous())
         i2 = O.nibble_unpack(rows2[:, base:base + hkv * (d // 2)].contiguous())
-        assert (i1 != i2).float().mean().item() <= 1e-4
         assert (i1.int() - i2.int()).abs().max().item() <= 1
+        # the two float32 rotations sum in different orders: an index may differ only where the coordinate, rotated
+        # in float64, lies within float32 rounding of a bucket boundary (a rate would depend on the sample size)
+        for row, col in (i1 != i2).nonzero().tolist():
+            x = rows_in[stored][row].reshape(hkv, d)[col // d].double()
+            y = (r.double() @ (x / (x.norm() + 1e-10)))[col % d]
+            assert (b.double() - y).abs().min().item() <= 1e-6, (lens, row, col)
         n1 = rows1[:, base + hkv * (d // 2):base + half].contiguous().view(torch.float32)
         n2 = rows2[:, base + hkv * (d // 2):base + half].contiguous().view(torch.float32)
         assert ((n1 - n2).abs() / n2).max().item() <= 2e-6
