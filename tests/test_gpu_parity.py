@@ -454,6 +454,53 @@ def test_paged_decode_fp16_and_large_norms():
     _decode_case([100, 33], hq=8, hkv=2, kv_scale=1e-3)
 
 
+def _poison_unused_table_entries(table, lens, bs, nb):
+    """Block-table entries past a sequence's last page: values no valid page has."""
+    bad = torch.tensor([-1, 2 ** 30, -2 ** 31, nb, 2 ** 31 - 1, -7], dtype=torch.int64)
+    out = table.clone()
+    for s, L in enumerate(lens):
+        used = (L + bs - 1) // bs
+        n = out.shape[1] - used
+        if n > 0:
+            out[s, used:] = bad[(torch.arange(n) + s) % len(bad)].to(torch.int32)
+    return out
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs", [(32, 8, 128, 16), (16, 16, 128, 8), (8, 1, 128, 16), (8, 2, 128, 32), (16, 4, 128, 16),
+                                         (12, 3, 128, 16), (32, 16, 64, 16), (16, 4, 64, 16), (8, 2, 256, 16),
+                                         (16, 4, 256, 32)])
+@pytest.mark.parametrize("num_splits", [0, 3])
+def test_paged_decode_ignores_table_entries_past_a_sequence(hq, hkv, d, bs, num_splits):
+    """A serving engine leaves stale or filler ids in the block-table columns a sequence does not use
+    (the reference indexes the table only below `seq_len`, cpu_reference.py:293-296): whatever they hold,
+    negative or beyond the cache, the result is bit for bit what a clean table gives, on every kernel form."""
+    lens = [37, 0, 16, 700, 64, 65, 1, 129, 2100]
+    c, b, r = book(d)
+    q, cache, table, sl = build_paged_case(lens, hq, hkv, d=d, bs=bs, seed=77, dtype=torch.bfloat16)
+    dirty = _poison_unused_table_entries(table, lens, bs, cache.shape[0])
+    assert not torch.equal(dirty, table)
+    cd, rd, qd, cached, sld = c.to(DEV), r.to(DEV), q.to(DEV), cache.to(DEV), sl.to(DEV)
+    want = K.split_k_paged_decode(qd, cached, table.to(DEV), sld, cd, cd, rd, hkv, d, bs, num_splits=num_splits)
+    got = K.split_k_paged_decode(qd, cached, dirty.to(DEV), sld, cd, cd, rd, hkv, d, bs, num_splits=num_splits)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (4, 2, 64), (4, 1, 256)])
+def test_paged_prefill_ignores_table_entries_past_a_sequence(hq, hkv, d):
+    kv, ql, bs = [45, 64, 300, 131, 500, 0], [7, 64, 1, 130, 32, 0], 16
+    c, b, r = book(d)
+    _, cache, table, sl = build_paged_case(kv, hq, hkv, d=d, bs=bs, seed=78, dtype=torch.bfloat16)
+    dirty = _poison_unused_table_entries(table, kv, bs, cache.shape[0])
+    q = torch.randn(sum(ql), hq, d, generator=torch.Generator().manual_seed(79)).to(torch.bfloat16).to(DEV)
+    cu = torch.tensor([0] + list(torch.tensor(ql).cumsum(0)), dtype=torch.int32).to(DEV)
+    cd, rd, cached, sld = c.to(DEV), r.to(DEV), cache.to(DEV), sl.to(DEV)
+    want = K.paged_tq4_prefill(q, cu, max(ql), cached, table.to(DEV), sld, cd, cd, rd, hkv, d, bs)
+    got = K.paged_tq4_prefill(q, cu, max(ql), cached, dirty.to(DEV), sld, cd, cd, rd, hkv, d, bs)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
 def test_paged_decode_failed_handoff_is_loud(kernel_option):
     """The wavefronts of the staged kernel meet through bounded waits.  With the bound forced down
     to two polls from the host the waits give up: every wavefront still runs to the end (nothing
