@@ -35,10 +35,15 @@ Pinned by (see tests/test_oracle_*.py):
       queries), paged_decode_gather for one query per sequence, SDPA with an
       explicit bottom-right mask for a chunked prefill.
   prod_quantize / prod_inner_product
-      unbiasedness of the estimator over many draws, sign/zero rule.
+      sign/zero rule; with the identity as sketch the correction term equals
+      gamma * sqrt(pi/2)/d * <q, sign(residual)> exactly; its mean over 400
+      sketches is <q, residual> / sqrt(d) (the reference's normalisation,
+      core/quantizer.py:264-268, 355-370, reproduced as is); the gain over
+      many keys; explicit sums.  A dropped, halved or doubled term fails these.
   prod_paged_decode
-      parity unpinned as a layout (the reference has no paged TurboQuantProd
-      path); its score formula is pinned through prod_inner_product.
+      against explicit prod_inner_product scores + softmax + mse_dequantize
+      values through the packed page; the page layout itself is parity
+      unpinned (the reference has no paged TurboQuantProd path).
 """
 
 from __future__ import annotations
